@@ -1,0 +1,64 @@
+"""Compile the HIP sources of the vtkv library for gfx950 into ``glake_amd/lib/libvtkv.so``.
+
+Usage: ``python -m glake_amd.build`` (hipcc cross-compiles, no GPU needed).
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_HERE, "csrc")
+LIB_DIR = os.path.join(_HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libvtkv.so")
+SOURCES = ["vtkv_vmm.cpp", "vtkv_cache.hip", "vtkv_attention.hip"]
+
+# Packed-FP32 instruction selection is switched off for all device code of this library.
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the vtkv library cannot be built")
+    return exe
+
+
+def build_library(verbose: bool = False) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(_HERE, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    hipcc = _hipcc()
+
+    def compile_one(src: str) -> str:
+        obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+        cmd = [hipcc, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        # the host pass does not know the device-only feature flag and says so: not an error
+        err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
+        objs = list(ex.map(compile_one, SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    res = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs, "-lpthread"],
+                         capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("linking libvtkv.so failed:\n" + res.stderr)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

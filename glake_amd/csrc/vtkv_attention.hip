@@ -1,0 +1,372 @@
+// Decode attention over per-sequence contiguous KV ranges ("vTensor" layout) for gfx950.
+//
+// One query token per sequence attends to the first seq_len rows of that sequence's K and V
+// ranges, both token-major [T, Hkv, D].  The work is bound by HBM reads of K and V
+// (2*Hkv*D*e bytes per token, 2*G/e flop per byte with G = Hq/Hkv), so the design goal is to read
+// every K/V byte exactly once and keep many 16-byte loads in flight:
+//
+//  * split-K: grid (Hkv, partitions, sequences); a workgroup of four wave64 handles one kv head
+//    over one partition of `part_tokens` rows and ALL G query heads of that kv head's group
+//    share the pass (the reference launches one block per query head and re-reads KV G times,
+//    csrc/attention/attention_kernels.cu:625 grid(num_heads, num_seqs, 1)).
+//  * inside a wave a tile is 16 rows.  S^T = K_tile . Q^T runs on v_mfma_f32_16x16x32_bf16 with the
+//    G query heads padded to the 16 columns: K rows are the A operand, and a lane's 16-byte
+//    global load of one row piece already IS its A operand, so K never touches LDS.
+//  * softmax statistics stay in registers: in the MFMA C layout a lane owns one head column and four
+//    rows, so a head's max/sum over the tile is an in-lane reduction plus two cross-row-group
+//    exchanges; an online (running-max) rescale keeps one pass.
+//  * O^T += V_tile^T . P^T runs on v_mfma_f32_16x16x16_bf16.  P^T is the C layout of S^T as is.  V is
+//    row-major but the A operand needs four rows per lane, so V tiles go through a wave-private,
+//    XOR-swizzled LDS tile and come back with ds_read_b64_tr_b16 (the transposing LDS read).
+//  * each wave keeps (m, l, O) for its rows; the four waves merge through LDS and the workgroup
+//    writes one normalised partial (max, sum, O/sum) per head; a second small kernel merges the
+//    partitions of each sequence with the log-sum-exp rule of the reference's split kernel
+//    (csrc/attention/attention_kernels.cu:486-583; CPU twin csrc/cpu/attention.cpp:583-644).
+//
+// Numerics: bf16 q.k products accumulated in fp32 and softmax in fp32 as in the reference
+// (csrc/attention/attention_kernels.cu:226-283).  The reference CUDA kernel rounds P to bf16
+// before P.V (:326-327) while its CPU twin keeps P in fp32 (csrc/cpu/attention.cpp:197-211); here P
+// enters the MFMA as a bf16 head plus a bf16 tail (two MFMAs), which is as good as fp32 P for the
+// tolerance in force.  fp32 accumulation, output rounded to bf16 once.  No epsilon is added to the softmax denominator (the
+// CPU twin has none, csrc/cpu/attention.cpp:43-67).
+#include <algorithm>
+
+#include "vtkv_common.h"
+#include "vtkv_fp8.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kD = 128;            // head size
+constexpr int kTile = 16;          // rows per MFMA tile
+constexpr int kWaves = 4;          // waves per workgroup
+constexpr int kRowBytes = kD * 2;  // bf16 row of one head
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct AttnParams {
+  const uint16_t *q;
+  const int64_t *k_ptrs, *v_ptrs, *slot_ids;
+  const int32_t *seq_lens;
+  const float *alibi_slopes;
+  float *part_max, *part_sum, *part_out;  // [B,Hq,P], [B,Hq,P], [B,Hq,P,D]
+  void *out;                              // [B,Hq,D] bf16, or fp32 when out_f32
+  int out_f32;
+  int64_t q_stride;
+  int num_heads, num_kv_heads, group;  // Hq, Hkv, G
+  int part_tokens, max_parts;
+  float scale_log2;  // scale * log2(e) [* k_scale for fp8 K]
+  float v_scale;
+};
+
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+  // round to nearest even, as the reference's from_float(bf16) does
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  bf16x2 v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(unsigned, v);
+}
+
+// LDS tile of 16 V rows x 256 bytes.  The 16-byte piece p of row r lives at piece slot
+// p ^ (2*(r & 7)): a transposing read then touches all 64 banks evenly (rows of one read differ
+// in r, pieces in one read are the pair {2*dblk, 2*dblk+1}).
+__device__ __forceinline__ int v_lds_offset(int row, int piece16) {
+  return row * kRowBytes + ((piece16 ^ ((row & 7) << 1)) << 4);
+}
+
+template <bool FP8>
+__global__ void __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnParams p) {
+  // wave-private V tiles (4 KiB each); reused after the main loop for the cross-wave merge
+  __shared__ __attribute__((aligned(16))) char smem[kWaves * kTile * kRowBytes + 1024];
+
+  const int kvh = blockIdx.x, part = blockIdx.y, b = blockIdx.z;
+  const int seq_len = p.seq_lens[b];
+  const int part_start = part * p.part_tokens;
+  if (part_start >= seq_len) return;
+  const int part_end = min(seq_len, part_start + p.part_tokens);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int g = lane >> 4;   // row group of the MFMA layouts
+  const int n = lane & 15;   // column: query head inside the group (S^T, O^T), or row of the tile (A operand)
+  const int G = p.group;
+  const int Hkv = p.num_kv_heads;
+
+  const int64_t slot = p.slot_ids[b];
+  const char *k_base = reinterpret_cast<const char *>(p.k_ptrs[slot]);
+  const char *v_base = reinterpret_cast<const char *>(p.v_ptrs[slot]);
+  constexpr int EB = FP8 ? 1 : 2;
+  const int64_t row_stride = (int64_t)Hkv * kD * EB;  // bytes between consecutive tokens
+  k_base += (int64_t)kvh * kD * EB;
+  v_base += (int64_t)kvh * kD * EB;
+
+  // B operand of S^T = K.Q^T: lane (n, g) holds q[head n][32*ks + 8*g .. +8], zero for padded heads
+  bf16x8 qop[4];
+  {
+    const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * kD;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + ks * 32 + g * 8);
+      if (n >= G) raw = (u32x4){0, 0, 0, 0};
+      qop[ks] = __builtin_bit_cast(bf16x8, raw);
+    }
+  }
+  const float slope_log2 =
+      (p.alibi_slopes != nullptr && n < G) ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
+
+  f32x4 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY;  // running max of scaled logits (log2 units) of head n
+  float l_run = 0.f;        // this lane's share of the running sum
+
+  char *v_tile = smem + wave * (kTile * kRowBytes);
+  const int last_row = seq_len - 1;
+
+  // global -> register loads of one 16-row tile.
+  //   K: lane (n, g) takes row t0+n, bytes [64*ks + 16*g, +16): exactly its MFMA A operand.
+  //   V: lane l takes row t0 + 4*j + (l>>4), piece16 (l & 15): four full rows per load instruction.
+  // Rows past the end of the sequence are redirected to the last valid row (their logits are
+  // masked below) so no lane ever reads beyond the mapped part of the range.
+  u32x4 kreg[4], vreg[4];
+  auto load_tile = [&](int t0, u32x4 *kr, u32x4 *vr) {
+    const int krow = min(t0 + n, last_row);
+    const char *kp = k_base + (int64_t)krow * row_stride + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) kr[ks] = *reinterpret_cast<const u32x4 *>(kp + ks * 64);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int vrow = min(t0 + 4 * j + g, last_row);
+      vr[j] = *reinterpret_cast<const u32x4 *>(v_base + (int64_t)vrow * row_stride + n * 16);
+    }
+  };
+
+  int t0 = part_start + wave * kTile;
+  if (t0 < part_end) load_tile(t0, kreg, vreg);
+
+  for (; t0 < part_end; t0 += kWaves * kTile) {
+    // prefetch the wave's next tile while this one is consumed
+    u32x4 knext[4], vnext[4];
+    const int t_next = t0 + kWaves * kTile;
+    if (t_next < part_end) load_tile(t_next, knext, vnext);
+
+    // S^T[row, head] = sum_d K[row, d] q[head, d]
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kreg[ks]), qop[ks], s, 0, 0, 0);
+
+    // stage V for the transposing read
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(4 * j + g, n)) = vreg[j];
+
+    // logits in log2 units; lane owns rows t0 + 4*g + i of head n
+    float x[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = t0 + 4 * g + i;
+      x[i] = s[i] * p.scale_log2 + slope_log2 * (float)(t - seq_len + 1);
+      if (t >= seq_len) x[i] = -INFINITY;
+    }
+    float tmax = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+    const float m_new = fmaxf(m_run, tmax);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
+    m_run = m_new;
+    float pr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pr[i] = __builtin_amdgcn_exp2f(x[i] - m_new);
+    l_run = l_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+    }
+    // P^T as B operand (row 4g+i, head n), split into a bf16 head and a bf16 tail so that P.V keeps
+    // ~16 mantissa bits of P: the result then tracks an fp32-P reference, not just a bf16-P one.
+    float plo[4];
+    u32x2 pb_hi = {pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3])};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned hi_bits = (i & 1) ? (pb_hi[i >> 1] & 0xffff0000u) : (pb_hi[i >> 1] << 16);
+      plo[i] = pr[i] - __builtin_bit_cast(float, hi_bits);
+    }
+    u32x2 pb_lo = {pack_bf16x2(plo[0], plo[1]), pack_bf16x2(plo[2], plo[3])};
+    const s16x4 pop_hi = __builtin_bit_cast(s16x4, pb_hi);
+    const s16x4 pop_lo = __builtin_bit_cast(s16x4, pb_lo);
+
+    // O^T[d, head] += sum_row V[row, d] P[row, head], 16 d per MFMA.  LDS operations of one wave
+    // execute in order, so the fences only pin the compiler's ordering of tile writes and reads.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+    for (int db = 0; db < 8; ++db) {
+      const int row = 4 * g + (n >> 2);
+      const int off = row * kRowBytes + (((2 * db + ((n >> 1) & 1)) ^ ((row & 7) << 1)) << 4) + ((n & 1) << 3);
+      const s16x4 vop = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4 *)(v_tile + off));
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop, pop_hi, acc[db], 0, 0, 0);
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop, pop_lo, acc[db], 0, 0, 0);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    if (t_next < part_end) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        kreg[j] = knext[j];
+        vreg[j] = vnext[j];
+      }
+    }
+  }
+
+  // ---- merge the four waves.  l_run is still split over the four row groups of a lane column.
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
+  __syncthreads();  // every wave is done with its V tile: smem is free for the merge
+  float *sm_m = reinterpret_cast<float *>(smem + kWaves * kTile * kRowBytes);  // [4][16]
+  float *sm_l = sm_m + kWaves * 16;                                               // [4][16]
+  float *sm_o = reinterpret_cast<float *>(smem);                                  // [4][G][128] (<= 16 KiB at G<=8)
+  if (g == 0) {
+    sm_m[wave * 16 + n] = m_run;
+    sm_l[wave * 16 + n] = l_run;
+  }
+  __syncthreads();
+  float m_wg = fmaxf(fmaxf(sm_m[n], sm_m[16 + n]), fmaxf(sm_m[32 + n], sm_m[48 + n]));
+  const float f = __builtin_amdgcn_exp2f(m_run - m_wg);  // 0 for a wave that saw no row
+  // G <= 8 fits the 16 KiB; for larger groups the merge runs in two halves of 8 heads
+  for (int h0 = 0; h0 < G; h0 += 8) {
+    if (h0 > 0) __syncthreads();
+    if (n >= h0 && n < min(G, h0 + 8)) {
+#pragma unroll
+      for (int db = 0; db < 8; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          sm_o[(wave * 8 + (n - h0)) * kD + db * 16 + 4 * g + i] = acc[db][i] * f;
+    }
+    __syncthreads();
+    const int nh = min(G, h0 + 8) - h0;
+    for (int idx = threadIdx.x; idx < nh * kD; idx += kWaves * 64) {
+      const int hh = idx / kD, d = idx % kD;
+      const int head = h0 + hh;
+      const float mw = fmaxf(fmaxf(sm_m[head], sm_m[16 + head]), fmaxf(sm_m[32 + head], sm_m[48 + head]));
+      float lsum = 0.f, o = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        lsum += sm_l[w * 16 + head] * __builtin_amdgcn_exp2f(sm_m[w * 16 + head] - mw);
+        o += sm_o[(w * 8 + hh) * kD + d];
+      }
+      const int64_t pidx = ((int64_t)b * p.num_heads + kvh * G + head) * p.max_parts + part;
+      p.part_out[pidx * kD + d] = o / lsum;
+      if (d == 0) {
+        p.part_max[pidx] = mw;   // log2 units
+        p.part_sum[pidx] = lsum;
+      }
+    }
+  }
+}
+
+// Merge the partitions of one (sequence, head): out = sum_j o_j w_j / sum_j w_j with
+// w_j = l_j * 2^(m_j - max m)  (csrc/attention/attention_kernels.cu:515-582).
+__global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
+  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int seq_len = p.seq_lens[b];
+  if (seq_len <= 0) return;
+  const int nparts = (seq_len + p.part_tokens - 1) / p.part_tokens;
+  const int64_t base = ((int64_t)b * p.num_heads + head) * p.max_parts;
+  float m = -INFINITY;
+  for (int j = 0; j < nparts; ++j) m = fmaxf(m, p.part_max[base + j]);
+  float wsum = 0.f, o = 0.f;
+  for (int j = 0; j < nparts; ++j) {
+    const float w = p.part_sum[base + j] * __builtin_amdgcn_exp2f(p.part_max[base + j] - m);
+    wsum += w;
+    o += p.part_out[(base + j) * kD + d] * w;
+  }
+  const float r = o / wsum * p.v_scale;
+  const int64_t oi = ((int64_t)b * p.num_heads + head) * kD + d;
+  if (p.out_f32)
+    reinterpret_cast<float *>(p.out)[oi] = r;
+  else
+    reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
+}
+
+int default_part_tokens(int max_seq_len) {
+  (void)max_seq_len;
+  return 256;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_seq_len,
+                                              int partition_tokens) {
+  if (num_seqs <= 0 || num_heads <= 0 || head_size <= 0 || max_seq_len <= 0) return 0;
+  const int pt = partition_tokens > 0 ? partition_tokens : default_part_tokens(max_seq_len);
+  const int64_t parts = (max_seq_len + pt - 1) / pt;
+  return (int64_t)num_seqs * num_heads * parts * (head_size + 2) * (int64_t)sizeof(float);
+}
+
+int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                          const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
+                          int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                          const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                          float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream) {
+  VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids && seq_lens, "null argument");
+  VTKV_REQUIRE(num_seqs >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
+               "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
+  VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
+  VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
+  VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
+  VTKV_REQUIRE(kv_dtype == VTKV_BF16, "kv_dtype must be BF16");
+  const int group = num_heads / num_kv_heads;
+  VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
+  VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0,
+               "q rows must be 16-byte aligned and at least num_heads*head_size apart");
+  VTKV_REQUIRE(max_seq_len > 0, "max_seq_len must be > 0");
+  if (num_seqs == 0) return VTKV_OK;
+  const int pt = partition_tokens > 0 ? partition_tokens : default_part_tokens(max_seq_len);
+  VTKV_REQUIRE(pt % (kWaves * kTile) == 0, "partition_tokens must be a multiple of %d", kWaves * kTile);
+  const int64_t parts = (max_seq_len + pt - 1) / pt;
+  VTKV_REQUIRE(parts <= 65535 && num_seqs <= 65535, "grid too large: %lld partitions, %d sequences",
+               (long long)parts, num_seqs);
+  const int64_t need = vtkv_decode_attention_workspace_bytes(num_seqs, num_heads, head_size, max_seq_len, pt);
+  if (!workspace || workspace_bytes < need)
+    return vtkv::fail(VTKV_ENOMEM, "workspace of %lld bytes is smaller than the %lld needed",
+                      (long long)workspace_bytes, (long long)need);
+  VTKV_REQUIRE((uintptr_t)workspace % 16 == 0, "workspace must be 16-byte aligned");
+  (void)k_scale;
+
+  AttnParams p;
+  p.q = (const uint16_t *)q;
+  p.k_ptrs = k_ptrs;
+  p.v_ptrs = v_ptrs;
+  p.slot_ids = slot_ids;
+  p.seq_lens = seq_lens;
+  p.alibi_slopes = alibi_slopes;
+  const int64_t n_stat = (int64_t)num_seqs * num_heads * parts;
+  p.part_out = (float *)workspace;
+  p.part_max = p.part_out + n_stat * kD;
+  p.part_sum = p.part_max + n_stat;
+  p.out = out;
+  p.out_f32 = out_dtype == VTKV_F32;
+  p.q_stride = q_stride;
+  p.num_heads = num_heads;
+  p.num_kv_heads = num_kv_heads;
+  p.group = group;
+  p.part_tokens = pt;
+  p.max_parts = (int)parts;
+  p.scale_log2 = scale * kLog2e;
+  p.v_scale = 1.f;
+  (void)v_scale;
+
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(decode_attn_partial_kernel<false>, dim3(num_kv_heads, (unsigned)parts, num_seqs),
+                     dim3(kWaves * 64), 0, st, p);
+  hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
+  VTKV_HIP(hipGetLastError());
+  return VTKV_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,455 @@
+// Physical chunk pool and per-sequence virtual ranges on the HIP virtual-memory API.
+//
+// Each sequence slot owns, per layer, one K and one V address range reserved with
+// hipMemAddressReserve; 2 MiB physical chunks created once with hipMemCreate are mapped at the
+// end of the ranges as the sequence grows and go back to the pool when it is released, so KV of
+// one sequence is always one contiguous [T, Hkv, D] array and kernels need no block table.
+//
+// Replaces the reference's vmm_allocator module (vmm_allocator/vmm_allocator.{h,cpp}).  What is
+// deliberately different: one mutex guards the pool and every segment (the reference pops its
+// request queue and touches the pool from two threads without a lock, vmm_allocator.cpp:43-48,
+// 222-228); growth in the decode step is done in the calling thread instead of a detached busy-
+// spinning thread signalling through POSIX shared memory (vmm_allocator.cpp:40-72,113-151);
+// failed growth leaves the segment unchanged instead of half-mapped; ranges are freed on destroy.
+#include <mutex>
+#include <unordered_set>
+#include <vector>
+
+#include "vtkv_common.h"
+
+namespace vtkv {
+
+thread_local char g_err[512] = "";
+char *error_buffer() { return g_err; }
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+namespace {
+
+constexpr int64_t kChunk = 2ll << 20;  // vmm_allocator.h:45 granularitySize
+
+struct Pool {
+  std::mutex mu;
+  int device = -1;
+  std::vector<hipMemGenericAllocationHandle_t> free_chunks;
+  int64_t total = 0;
+  std::unordered_set<vtkv_segment *> segments;
+};
+Pool g_pool;
+
+}  // namespace
+}  // namespace vtkv
+
+struct vtkv_segment {
+  int layer_num = 0;
+  int64_t context_max = 0;  // reserved bytes per range
+  int64_t expand_bytes = 0; // what release keeps mapped
+  int64_t mapped = 0;       // actual_size: bytes mapped per range
+  int64_t used = 0;         // used_size: bytes written per range
+  std::vector<char *> k_base, v_base;
+  // chunks mapped into layer l's K (resp. V) range, in address order
+  std::vector<std::vector<hipMemGenericAllocationHandle_t>> k_chunks, v_chunks;
+};
+
+using vtkv::g_pool;
+using vtkv::kChunk;
+
+namespace {
+
+// Map `n` chunks at offset `at` of every range.  Caller holds the pool mutex and has checked the
+// pool holds 2*layers*n chunks.  On a HIP failure everything mapped by this call is rolled back.
+int map_chunks_locked(vtkv_segment *s, int n) {
+  hipMemAccessDesc ad = {};
+  ad.location.type = hipMemLocationTypeDevice;
+  ad.location.id = g_pool.device;
+  ad.flags = hipMemAccessFlagsProtReadWrite;
+  struct Done { char *va; hipMemGenericAllocationHandle_t h; std::vector<hipMemGenericAllocationHandle_t> *list; };
+  std::vector<Done> done;
+  hipError_t err = hipSuccess;
+  for (int l = 0; l < s->layer_num && err == hipSuccess; ++l) {
+    for (int j = 0; j < n && err == hipSuccess; ++j) {
+      for (int which = 0; which < 2 && err == hipSuccess; ++which) {
+        char *va = (which ? s->v_base[l] : s->k_base[l]) + s->mapped + (int64_t)j * kChunk;
+        hipMemGenericAllocationHandle_t h = g_pool.free_chunks.back();
+        err = hipMemMap(va, kChunk, 0, h, 0);
+        if (err != hipSuccess) break;
+        g_pool.free_chunks.pop_back();
+        auto *list = which ? &s->v_chunks[l] : &s->k_chunks[l];
+        list->push_back(h);
+        done.push_back({va, h, list});
+        err = hipMemSetAccess(va, kChunk, &ad, 1);
+      }
+    }
+  }
+  if (err != hipSuccess) {
+    for (auto it = done.rbegin(); it != done.rend(); ++it) {
+      (void)hipMemUnmap(it->va, kChunk);
+      it->list->pop_back();
+      g_pool.free_chunks.push_back(it->h);
+    }
+    return vtkv::fail(VTKV_EHIP, "mapping a chunk failed: %s", hipGetErrorString(err));
+  }
+  s->mapped += (int64_t)n * kChunk;
+  return VTKV_OK;
+}
+
+int expand_locked(vtkv_segment *s, int n) {
+  if (n <= 0) return VTKV_OK;
+  if (s->mapped + (int64_t)n * kChunk > s->context_max)
+    return vtkv::fail(VTKV_EINVAL, "segment would grow to %lld bytes, beyond its reserved %lld",
+                      (long long)(s->mapped + (int64_t)n * kChunk), (long long)s->context_max);
+  const int64_t need = 2ll * s->layer_num * n;
+  if ((int64_t)g_pool.free_chunks.size() < need)
+    return vtkv::fail(VTKV_ENOMEM, "chunk pool exhausted: need %lld, free %lld", (long long)need,
+                      (long long)g_pool.free_chunks.size());
+  return map_chunks_locked(s, n);
+}
+
+// Unmap every chunk at offset >= keep_bytes of every range and return them to the pool.
+int shrink_locked(vtkv_segment *s, int64_t keep_bytes) {
+  if (keep_bytes >= s->mapped) return VTKV_OK;
+  const int64_t keep_n = keep_bytes / kChunk;
+  for (int l = 0; l < s->layer_num; ++l) {
+    for (int which = 0; which < 2; ++which) {
+      auto &list = which ? s->v_chunks[l] : s->k_chunks[l];
+      char *base = which ? s->v_base[l] : s->k_base[l];
+      // one call per mapping: each chunk was mapped on its own
+      while ((int64_t)list.size() > keep_n) {
+        VTKV_HIP(hipMemUnmap(base + ((int64_t)list.size() - 1) * kChunk, kChunk));
+        g_pool.free_chunks.push_back(list.back());
+        list.pop_back();
+      }
+    }
+  }
+  s->mapped = keep_n * kChunk;
+  return VTKV_OK;
+}
+
+int ensure_locked(vtkv_segment *s, int64_t token_bytes) {
+  if (s->used + token_bytes <= s->mapped) return 0;
+  const int64_t gap = s->used + token_bytes - s->mapped;
+  const int n = (int)((gap + kChunk - 1) / kChunk);
+  int rc = expand_locked(s, n);
+  return rc < 0 ? rc : 1;
+}
+
+int reserve_locked(vtkv_segment *s, int64_t token_bytes, int64_t kv_size) {
+  // vmm_allocator.cpp:322-337: room for the new rows plus a 100-row slack, rounded up to chunks
+  const int64_t want = s->used + token_bytes + 100 * kv_size;
+  if (want > s->mapped) {
+    int64_t n = (want - s->mapped + kChunk - 1) / kChunk;
+    // the slack must not push a sequence past its reserved range
+    const int64_t room = (s->context_max - s->mapped) / kChunk;
+    if (n > room) n = room;
+    if (s->used + token_bytes > s->mapped + n * kChunk)
+      return vtkv::fail(VTKV_EINVAL, "sequence of %lld bytes does not fit its reserved %lld",
+                        (long long)(s->used + token_bytes), (long long)s->context_max);
+    int rc = expand_locked(s, (int)n);
+    if (rc < 0) return rc;
+  }
+  s->used += token_bytes;
+  return VTKV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *vtkv_last_error(void) { return vtkv::error_buffer(); }
+int vtkv_version(void) { return 100; }
+int64_t vtkv_chunk_bytes(void) { return kChunk; }
+
+int vtkv_pool_init(int device, int64_t num_chunks) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  VTKV_REQUIRE(num_chunks >= 0, "num_chunks must be >= 0");
+  if (g_pool.device >= 0 && g_pool.device != device)
+    return vtkv::fail(VTKV_ESTATE, "pool already lives on device %d", g_pool.device);
+  VTKV_HIP(hipSetDevice(device));
+  int vmm = 0;
+  VTKV_HIP(hipDeviceGetAttribute(&vmm, hipDeviceAttributeVirtualMemoryManagementSupported, device));
+  if (!vmm) return vtkv::fail(VTKV_EHIP, "device %d has no virtual memory management support", device);
+  hipMemAllocationProp prop = {};
+  prop.type = hipMemAllocationTypePinned;
+  prop.location.type = hipMemLocationTypeDevice;
+  prop.location.id = device;
+  size_t gran = 0;
+  VTKV_HIP(hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityMinimum));
+  if (gran == 0 || kChunk % (int64_t)gran != 0)
+    return vtkv::fail(VTKV_EHIP, "allocation granularity %zu does not divide the 2 MiB chunk", gran);
+  g_pool.device = device;
+  g_pool.free_chunks.reserve(g_pool.free_chunks.size() + num_chunks);
+  for (int64_t i = 0; i < num_chunks; ++i) {
+    hipMemGenericAllocationHandle_t h;
+    hipError_t e = hipMemCreate(&h, kChunk, &prop, 0);
+    if (e != hipSuccess)
+      return vtkv::fail(VTKV_ENOMEM, "hipMemCreate failed after %lld of %lld chunks: %s", (long long)i,
+                        (long long)num_chunks, hipGetErrorString(e));
+    g_pool.free_chunks.push_back(h);
+    ++g_pool.total;
+  }
+  return VTKV_OK;
+}
+
+int64_t vtkv_pool_free_chunks(void) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  return (int64_t)g_pool.free_chunks.size();
+}
+
+int64_t vtkv_pool_total_chunks(void) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  return g_pool.total;
+}
+
+int vtkv_pool_destroy(void) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  if (!g_pool.segments.empty())
+    return vtkv::fail(VTKV_ESTATE, "%zu segments still alive", g_pool.segments.size());
+  for (auto h : g_pool.free_chunks) VTKV_HIP(hipMemRelease(h));
+  g_pool.free_chunks.clear();
+  g_pool.total = 0;
+  g_pool.device = -1;
+  return VTKV_OK;
+}
+
+vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t expand_bytes, int expand) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  if (g_pool.device < 0) {
+    vtkv::fail(VTKV_ESTATE, "vtkv_pool_init has not been called");
+    return nullptr;
+  }
+  if (layer_num <= 0 || context_max_bytes <= 0 || context_max_bytes % kChunk != 0 || expand_bytes < 0 ||
+      expand_bytes % kChunk != 0 || expand_bytes > context_max_bytes) {
+    vtkv::fail(VTKV_EINVAL, "layer_num must be > 0 and sizes multiples of the 2 MiB chunk (max %lld, expand %lld)",
+               (long long)context_max_bytes, (long long)expand_bytes);
+    return nullptr;
+  }
+  auto *s = new vtkv_segment;
+  s->layer_num = layer_num;
+  s->context_max = context_max_bytes;
+  s->expand_bytes = expand_bytes;
+  s->k_chunks.resize(layer_num);
+  s->v_chunks.resize(layer_num);
+  auto unwind = [&](hipError_t e) {
+    for (char *p : s->k_base) (void)hipMemAddressFree(p, context_max_bytes);
+    for (char *p : s->v_base) (void)hipMemAddressFree(p, context_max_bytes);
+    delete s;
+    vtkv::fail(VTKV_EHIP, "hipMemAddressReserve failed: %s", hipGetErrorString(e));
+    return (vtkv_segment *)nullptr;
+  };
+  for (int l = 0; l < layer_num; ++l) {
+    void *k = nullptr, *v = nullptr;
+    hipError_t e = hipMemAddressReserve(&k, context_max_bytes, kChunk, nullptr, 0);
+    if (e != hipSuccess) return unwind(e);
+    s->k_base.push_back((char *)k);
+    e = hipMemAddressReserve(&v, context_max_bytes, kChunk, nullptr, 0);
+    if (e != hipSuccess) return unwind(e);
+    s->v_base.push_back((char *)v);
+  }
+  if (expand && expand_bytes > 0) {
+    if (expand_locked(s, (int)(expand_bytes / kChunk)) < 0) {
+      for (char *p : s->k_base) (void)hipMemAddressFree(p, context_max_bytes);
+      for (char *p : s->v_base) (void)hipMemAddressFree(p, context_max_bytes);
+      delete s;
+      return nullptr;
+    }
+  }
+  g_pool.segments.insert(s);
+  return s;
+}
+
+#define SEG_CHECK(s)                                                                                  \
+  if (!(s) || !g_pool.segments.count(const_cast<vtkv_segment *>(s)))                                  \
+  return vtkv::fail(VTKV_ESTATE, "not a live segment")
+
+int vtkv_seg_destroy(vtkv_segment *s) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  int rc = shrink_locked(s, 0);
+  if (rc < 0) return rc;
+  for (char *p : s->k_base) VTKV_HIP(hipMemAddressFree(p, s->context_max));
+  for (char *p : s->v_base) VTKV_HIP(hipMemAddressFree(p, s->context_max));
+  g_pool.segments.erase(s);
+  delete s;
+  return VTKV_OK;
+}
+
+uint64_t vtkv_seg_key_ptr(const vtkv_segment *s, int layer) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  if (!s || !g_pool.segments.count(const_cast<vtkv_segment *>(s)) || layer < 0 || layer >= s->layer_num) {
+    vtkv::fail(VTKV_EINVAL, "bad segment or layer %d", layer);
+    return 0;
+  }
+  return (uint64_t)(uintptr_t)s->k_base[layer];
+}
+
+uint64_t vtkv_seg_value_ptr(const vtkv_segment *s, int layer) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  if (!s || !g_pool.segments.count(const_cast<vtkv_segment *>(s)) || layer < 0 || layer >= s->layer_num) {
+    vtkv::fail(VTKV_EINVAL, "bad segment or layer %d", layer);
+    return 0;
+  }
+  return (uint64_t)(uintptr_t)s->v_base[layer];
+}
+
+int64_t vtkv_seg_get_used(const vtkv_segment *s) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  return s->used;
+}
+
+int vtkv_seg_set_used(vtkv_segment *s, int64_t used) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  VTKV_REQUIRE(used >= 0 && used <= s->context_max, "used_bytes %lld outside [0, %lld]", (long long)used,
+               (long long)s->context_max);
+  s->used = used;
+  return VTKV_OK;
+}
+
+int64_t vtkv_seg_mapped_bytes(const vtkv_segment *s) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  return s->mapped;
+}
+
+int vtkv_seg_expand(vtkv_segment *s, int n) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  VTKV_REQUIRE(n >= 0, "num_chunks must be >= 0");
+  return expand_locked(s, n);
+}
+
+int vtkv_seg_reserve(vtkv_segment *s, int64_t token_bytes, int64_t kv_size) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  VTKV_REQUIRE(token_bytes >= 0 && kv_size >= 0, "sizes must be >= 0");
+  return reserve_locked(s, token_bytes, kv_size);
+}
+
+int vtkv_seg_ensure(vtkv_segment *s, int64_t token_bytes) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  VTKV_REQUIRE(token_bytes >= 0, "token_bytes must be >= 0");
+  return ensure_locked(s, token_bytes);
+}
+
+int vtkv_seg_preempt(vtkv_segment *s) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  int rc = shrink_locked(s, 0);
+  if (rc < 0) return rc;
+  s->used = 0;
+  return VTKV_OK;
+}
+
+int vtkv_seg_release(vtkv_segment *s) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  // vmm_allocator.cpp:393-420: keep the first expand_size bytes mapped when at least that much is
+  // mapped, otherwise (fewer bytes mapped than expand_size) unmap everything.
+  const int64_t keep = s->mapped >= s->expand_bytes ? s->expand_bytes : 0;
+  int rc = shrink_locked(s, keep);
+  if (rc < 0) return rc;
+  s->used = 0;
+  return VTKV_OK;
+}
+
+int vtkv_extend_kv_cache_batch(vtkv_segment *const *segs, int n, const int64_t *token_bytes,
+                               const int64_t *set_used_tokens, int64_t kv_size, int gen, int64_t *slot_m_out) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  VTKV_REQUIRE(n >= 0 && (n == 0 || (segs && token_bytes && slot_m_out)), "null argument");
+  for (int i = 0; i < n; ++i) SEG_CHECK(segs[i]);
+  for (int i = 0; i < n; ++i) {
+    vtkv_segment *s = segs[i];
+    if (set_used_tokens && set_used_tokens[i] > 0) s->used = set_used_tokens[i] * kv_size;
+    slot_m_out[i] = s->used;
+    if (gen) {
+      int rc = ensure_locked(s, token_bytes[i]);
+      if (rc < 0) return rc;
+      s->used += token_bytes[i];
+    } else {
+      int rc = reserve_locked(s, token_bytes[i], kv_size);
+      if (rc < 0) return rc;
+    }
+  }
+  return VTKV_OK;
+}
+
+uint64_t vtkv_ptr_table_create(int num_seqs) {
+  if (num_seqs <= 0) {
+    vtkv::fail(VTKV_EINVAL, "num_seqs must be > 0");
+    return 0;
+  }
+  void *p = nullptr;
+  hipError_t e = hipMalloc(&p, (size_t)num_seqs * sizeof(uint64_t));
+  if (e != hipSuccess) {
+    vtkv::fail(VTKV_EHIP, "hipMalloc failed: %s", hipGetErrorString(e));
+    return 0;
+  }
+  (void)hipMemset(p, 0, (size_t)num_seqs * sizeof(uint64_t));
+  return (uint64_t)(uintptr_t)p;
+}
+
+int vtkv_ptr_table_destroy(uint64_t table) {
+  VTKV_HIP(hipFree((void *)(uintptr_t)table));
+  return VTKV_OK;
+}
+
+int vtkv_ptr_table_set(uint64_t table, int slot, uint64_t ptr) {
+  VTKV_REQUIRE(table != 0 && slot >= 0, "bad table or slot");
+  VTKV_HIP(hipMemcpy((char *)(uintptr_t)table + (size_t)slot * 8, &ptr, 8, hipMemcpyHostToDevice));
+  return VTKV_OK;
+}
+
+int vtkv_ptr_table_fill(uint64_t table, vtkv_segment *const *segs, int n, int layer, int which) {
+  std::vector<uint64_t> host(n > 0 ? n : 0);
+  {
+    std::lock_guard<std::mutex> lk(g_pool.mu);
+    VTKV_REQUIRE(table != 0 && n >= 0 && (n == 0 || segs), "bad table or segment list");
+    for (int i = 0; i < n; ++i) {
+      SEG_CHECK(segs[i]);
+      VTKV_REQUIRE(layer >= 0 && layer < segs[i]->layer_num, "layer %d out of range", layer);
+      host[i] = (uint64_t)(uintptr_t)(which ? segs[i]->v_base[layer] : segs[i]->k_base[layer]);
+    }
+  }
+  if (n > 0) VTKV_HIP(hipMemcpy((void *)(uintptr_t)table, host.data(), (size_t)n * 8, hipMemcpyHostToDevice));
+  return VTKV_OK;
+}
+
+int vtkv_memcpy_h2d(uint64_t dst, const void *src, int64_t bytes) {
+  VTKV_REQUIRE(bytes >= 0 && (bytes == 0 || (dst && src)), "null argument");
+  if (bytes) VTKV_HIP(hipMemcpy((void *)(uintptr_t)dst, src, (size_t)bytes, hipMemcpyHostToDevice));
+  return VTKV_OK;
+}
+
+int vtkv_memcpy_d2h(void *dst, uint64_t src, int64_t bytes) {
+  VTKV_REQUIRE(bytes >= 0 && (bytes == 0 || (dst && src)), "null argument");
+  if (bytes) VTKV_HIP(hipMemcpy(dst, (const void *)(uintptr_t)src, (size_t)bytes, hipMemcpyDeviceToHost));
+  return VTKV_OK;
+}
+
+void *vtkv_host_alloc(int64_t bytes) {
+  void *p = nullptr;
+  if (bytes <= 0) {
+    vtkv::fail(VTKV_EINVAL, "bytes must be > 0");
+    return nullptr;
+  }
+  hipError_t e = hipHostMalloc(&p, (size_t)bytes, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    vtkv::fail(VTKV_EHIP, "hipHostMalloc(%lld) failed: %s", (long long)bytes, hipGetErrorString(e));
+    return nullptr;
+  }
+  return p;
+}
+
+int vtkv_host_free(void *p) {
+  if (p) VTKV_HIP(hipHostFree(p));
+  return VTKV_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,213 @@
+"""Facade with the names of the reference's ``vmmAllocator`` pybind module
+(vmm_allocator/vmm_allocator.h:190-219) and of its ``KV_cache`` wrapper
+(vmm_allocator/vmm_allocator.py:5-19), over the HIP virtual-memory pool of ``libvtkv.so``.
+
+Differences a caller can observe, all deliberate:
+  * growth during decode is done by the calling thread inside ``extend_kv_cache_batch`` /
+    ``eagerExtend`` instead of a detached thread, so ``query_shm`` / ``query_cycle`` always report
+    "ready" and there is nothing to spin on (llama.py:322-326 becomes a no-op);
+  * pool exhaustion raises ``VtkvOutOfChunks`` instead of printing and carrying on
+    (vmm_allocator.cpp:232-235,330-333);
+  * segments can be destroyed (the reference never frees address ranges).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Sequence
+
+import numpy as np
+
+from . import _C
+
+granularitySize = 2 * 1024 * 1024  # vmm_allocator.h:45
+
+
+def init_physical_handle(num_blocks: int, device_id: int) -> bool:
+    """Create ``num_blocks`` 2 MiB physical chunks on ``device_id`` (vmm_allocator.cpp:113-151)."""
+    _C.check(_C.lib().vtkv_pool_init(int(device_id), int(num_blocks)))
+    return True
+
+
+def showFreeBlocks() -> int:
+    return int(_C.check(_C.lib().vtkv_pool_free_chunks()))
+
+
+def totalBlocks() -> int:
+    return int(_C.check(_C.lib().vtkv_pool_total_chunks()))
+
+
+def destroy_pool() -> None:
+    _C.check(_C.lib().vtkv_pool_destroy())
+
+
+class KVcacheSegment:
+    """One sequence slot: per layer a K and a V virtual range (vmm_allocator.cpp:177-456)."""
+
+    def __init__(self, layer_num: int, context_max_size: int, expand_size: int, expand: bool):
+        self._h = _C.check_ptr(
+            _C.lib().vtkv_seg_create(int(layer_num), int(context_max_size), int(expand_size), int(bool(expand))),
+            "KVcacheSegment")
+        self.layer_num = int(layer_num)
+        self.context_max_size = int(context_max_size)
+        self.expand_size = int(expand_size)
+
+    # --- pointers
+    def getKeyDevicePtr(self, layer_index: int) -> int:
+        return int(_C.check_ptr(_C.lib().vtkv_seg_key_ptr(self._h, int(layer_index)), "getKeyDevicePtr"))
+
+    def getValueDevicePtr(self, layer_index: int) -> int:
+        return int(_C.check_ptr(_C.lib().vtkv_seg_value_ptr(self._h, int(layer_index)), "getValueDevicePtr"))
+
+    # --- accounting
+    def get_used_slot(self) -> int:
+        return int(_C.check(_C.lib().vtkv_seg_get_used(self._h)))
+
+    def set_used_size(self, used_size: int) -> None:
+        _C.check(_C.lib().vtkv_seg_set_used(self._h, int(used_size)))
+
+    @property
+    def used_size(self) -> int:
+        return self.get_used_slot()
+
+    @property
+    def actual_size(self) -> int:
+        return int(_C.check(_C.lib().vtkv_seg_mapped_bytes(self._h)))
+
+    # --- growth / shrink
+    def expandMultiSegment(self, expand_num: int) -> bool:
+        _C.check(_C.lib().vtkv_seg_expand(self._h, int(expand_num)))
+        return True
+
+    def copy_kv_cache(self, token_size: int, kv_size: int) -> None:
+        _C.check(_C.lib().vtkv_seg_reserve(self._h, int(token_size), int(kv_size)))
+
+    def eagerExtend(self, token_size: int, seq_id: int) -> None:
+        """Map ahead so the next ``token_size`` bytes fit (vmm_allocator.cpp:307-320); done
+        in the calling thread."""
+        _C.check(_C.lib().vtkv_seg_ensure(self._h, int(token_size)))
+
+    def preempt_seq(self, seq_id: int = -1) -> None:
+        _C.check(_C.lib().vtkv_seg_preempt(self._h))
+
+    def release_seq(self, seq_id: int = -1) -> None:
+        _C.check(_C.lib().vtkv_seg_release(self._h))
+
+    def show_info(self, seq_id: int) -> List[int]:
+        # [seq_id, actual_size, used_size, ready flag, cycle] (vmm_allocator.cpp:448-456)
+        return [int(seq_id), self.actual_size, self.used_size, 1, 0]
+
+    # --- debugging helpers (vmm_allocator.cpp:423-446), layer 0 K range
+    def write_string(self, s: str) -> None:
+        data = s.encode()
+        used = self.get_used_slot()
+        _C.check(_C.lib().vtkv_seg_ensure(self._h, len(data)))
+        _C.check(_C.lib().vtkv_memcpy_h2d(self.getKeyDevicePtr(0) + used, data, len(data)))
+        self.set_used_size(used + len(data))
+
+    def read_string(self) -> str:
+        used = self.get_used_slot()
+        buf = C.create_string_buffer(max(used, 1))
+        if used:
+            _C.check(_C.lib().vtkv_memcpy_d2h(buf, self.getKeyDevicePtr(0), used))
+        return buf.raw[:used].decode()
+
+    def destroy(self) -> None:
+        if self._h:
+            _C.check(_C.lib().vtkv_seg_destroy(self._h))
+            self._h = None
+
+    def __del__(self):  # best effort: the pool may already be gone at interpreter exit
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class KVCache:
+    """Device array of per-slot base pointers (vmm_allocator.cpp:458-470)."""
+
+    def __init__(self, num_seqs: int):
+        self.num_seqs = int(num_seqs)
+        self._table = int(_C.check_ptr(_C.lib().vtkv_ptr_table_create(self.num_seqs), "KVCache"))
+
+    def getKVCachePtr(self) -> int:
+        return self._table
+
+    def AddKVCache(self, slot: int, kv_cache: int) -> None:
+        if not 0 <= slot < self.num_seqs:
+            raise _C.VtkvError(_C.EINVAL, f"slot {slot} outside [0, {self.num_seqs})")
+        _C.check(_C.lib().vtkv_ptr_table_set(self._table, int(slot), int(kv_cache)))
+
+    def to_numpy(self) -> np.ndarray:
+        out = np.zeros(self.num_seqs, np.int64)
+        _C.check(_C.lib().vtkv_memcpy_d2h(out.ctypes.data_as(C.c_void_p), self._table, out.nbytes))
+        return out
+
+    def destroy(self) -> None:
+        if self._table:
+            _C.check(_C.lib().vtkv_ptr_table_destroy(self._table))
+            self._table = 0
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class KV_cache:
+    """Per-layer handle the model code passes around (vmm_allocator/vmm_allocator.py:5-19)."""
+
+    def __init__(self, max_seqs: int, layer_index: int) -> None:
+        self.max_seqs = max_seqs
+        self.layer_index = layer_index
+        self.kv_cache = KVCache(self.max_seqs)
+        self.vmm_ptr = self.kv_cache.getKVCachePtr()
+
+
+def _seg_array(segments: Sequence[KVcacheSegment]):
+    return (C.c_void_p * len(segments))(*[s._h for s in segments])
+
+
+def extend_kv_cache_batch(k_cache_batch, v_cache_batch, slot_mapping: Sequence[int], token_size: Sequence[int],
+                          segment: Sequence[KVcacheSegment], set_used_size: Sequence[int], kv_size: int,
+                          gen: bool) -> List[int]:
+    """Per-step bookkeeping (vmm_allocator.h:138-168): returns each sequence's byte offset
+    before this step's rows, then advances it.  ``k_cache_batch`` / ``v_cache_batch`` are
+    accepted and ignored, as in the reference (its table refresh is commented out)."""
+    n = len(slot_mapping)
+    if not (len(token_size) == len(segment) == len(set_used_size) == n):
+        raise _C.VtkvError(_C.EINVAL, "extend_kv_cache_batch: argument lists differ in length")
+    tok = (C.c_int64 * n)(*[int(t) for t in token_size])
+    used = (C.c_int64 * n)(*[int(u) for u in set_used_size])
+    out = (C.c_int64 * n)()
+    _C.check(_C.lib().vtkv_extend_kv_cache_batch(_seg_array(segment), n, tok, used, int(kv_size), int(bool(gen)),
+                                                 out))
+    return list(out)
+
+
+def copy_kv_cache(k_cache_batch: Sequence[KVCache], v_cache_batch: Sequence[KVCache],
+                  segment: Sequence[KVcacheSegment]) -> None:
+    """Fill every layer's K and V pointer table from the segments (vmm_allocator.h:170-182)."""
+    segs = _seg_array(segment)
+    for layer, (k, v) in enumerate(zip(k_cache_batch, v_cache_batch)):
+        _C.check(_C.lib().vtkv_ptr_table_fill(k.getKVCachePtr(), segs, len(segment), layer, 0))
+        _C.check(_C.lib().vtkv_ptr_table_fill(v.getKVCachePtr(), segs, len(segment), layer, 1))
+
+
+# Readiness queries of the reference's background mapper (vmm_allocator.cpp:74-111).  Mapping is
+# synchronous here, so every slot is always ready and nothing is pending.
+def query_shm(seq_ids: Sequence[int]) -> bool:
+    return True
+
+
+def query_cycle(seq_ids: Sequence[int]) -> bool:
+    return False
+
+
+def query_unmap(seq_ids: Sequence[int]) -> List[bool]:
+    return [True for _ in seq_ids]
+
+
+def print_shm_state(seq_ids: Sequence[int]) -> List[int]:
+    return [1 for _ in seq_ids]

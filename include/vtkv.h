@@ -1,0 +1,214 @@
+/*
+ * vtkv - C ABI of the MI355X (gfx950) vTensor KV-cache hot path.
+ *
+ * Every entry point takes plain pointers and sizes (no framework types), returns
+ * 0 on success or a negative VTKV_E* code, and leaves a human-readable message in
+ * vtkv_last_error().  Device pointers are HIP device addresses of the current
+ * device; `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ * All kernels are asynchronous on `stream`; nothing here synchronises unless the
+ * comment says so.
+ *
+ * Each declaration cites the interface of the reference (paths relative to its
+ * GLakeServe/ directory) that it replaces.
+ */
+#ifndef VTKV_H
+#define VTKV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VTKV_OK 0
+#define VTKV_EINVAL (-1)   /* bad argument (shape, dtype, alignment, null pointer)      */
+#define VTKV_EHIP (-2)     /* a HIP runtime call failed                                 */
+#define VTKV_ENOMEM (-3)   /* physical chunk pool exhausted / workspace too small       */
+#define VTKV_ESTATE (-4)   /* call order violated (pool not initialised, double free …) */
+
+/* element types */
+#define VTKV_F32 0
+#define VTKV_BF16 1
+#define VTKV_F16 2
+#define VTKV_FP8_E4M3 3 /* OCP e4m3fn, one byte per element, per-tensor scale */
+
+/* copy directions for vtkv_swap_* */
+#define VTKV_D2H 0
+#define VTKV_H2D 1
+#define VTKV_D2D 2
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *vtkv_last_error(void);
+/* ABI version: major*10000 + minor*100 + patch. */
+int vtkv_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Physical chunk pool and per-sequence virtual ranges.
+ * Replaces the pybind module `vmmAllocator` (vmm_allocator/vmm_allocator.h:190-219).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Size of one physical chunk in bytes (2 MiB; vmm_allocator/vmm_allocator.h:45 granularitySize). */
+int64_t vtkv_chunk_bytes(void);
+
+/* Create `num_chunks` physical chunks on `device` and keep them in the free pool.
+ * Replaces init_physical_handle(num_blocks, device_id) (vmm_allocator.cpp:113-151).
+ * May be called again to add chunks. */
+int vtkv_pool_init(int device, int64_t num_chunks);
+/* Free chunks in the pool; replaces showFreeBlocks() (vmm_allocator.cpp:472-474). <0 on error. */
+int64_t vtkv_pool_free_chunks(void);
+/* Chunks ever created and still owned (free + mapped). */
+int64_t vtkv_pool_total_chunks(void);
+/* Release every chunk and every segment's address range.  All segments must have been destroyed. */
+int vtkv_pool_destroy(void);
+
+typedef struct vtkv_segment vtkv_segment;
+
+/* One sequence slot: for each of `layer_num` layers a K range and a V range of
+ * `context_max_bytes` reserved virtual addresses; nothing mapped unless `expand` is non-zero, in
+ * which case expand_bytes/chunk chunks are mapped at once.  `expand_bytes` is also what release
+ * keeps mapped.  Replaces KVcacheSegment(layer_num, context_max_size, expand_size, expand)
+ * (vmm_allocator.cpp:177-211).  Returns NULL on failure. */
+vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t expand_bytes, int expand);
+/* Unmap everything, return the chunks to the pool and free the address ranges (the reference never frees them). */
+int vtkv_seg_destroy(vtkv_segment *seg);
+/* Base device address of the K / V range of `layer`; replaces getKeyDevicePtr / getValueDevicePtr
+ * (vmm_allocator.cpp:299-305).  0 on error. */
+uint64_t vtkv_seg_key_ptr(const vtkv_segment *seg, int layer);
+uint64_t vtkv_seg_value_ptr(const vtkv_segment *seg, int layer);
+/* used_size (bytes written per range) get/set; replaces get_used_slot / set_used_size (vmm_allocator.cpp:339-345). */
+int64_t vtkv_seg_get_used(const vtkv_segment *seg);
+int vtkv_seg_set_used(vtkv_segment *seg, int64_t used_bytes);
+/* actual_size: bytes currently mapped per range (vmm_allocator.h:98). */
+int64_t vtkv_seg_mapped_bytes(const vtkv_segment *seg);
+/* Map `num_chunks` more chunks at the end of every K and V range of every layer (2*layers*num_chunks
+ * chunks in total); replaces expandMultiSegment (vmm_allocator.cpp:214-297).  VTKV_ENOMEM leaves the
+ * segment unchanged. */
+int vtkv_seg_expand(vtkv_segment *seg, int num_chunks);
+/* Prefill-side growth: make room for `token_bytes` more bytes plus a slack of 100*kv_size bytes, map the
+ * chunks needed, then used += token_bytes.  Replaces KVcacheSegment::copy_kv_cache (vmm_allocator.cpp:322-337). */
+int vtkv_seg_reserve(vtkv_segment *seg, int64_t token_bytes, int64_t kv_size);
+/* Decode-side growth that the reference spreads over eagerExtend + its background thread
+ * (vmm_allocator.cpp:40-72,307-320): map one more chunk when used + token_bytes would pass the mapped
+ * size.  Returns 1 if a chunk was mapped, 0 if not, <0 on error. */
+int vtkv_seg_ensure(vtkv_segment *seg, int64_t token_bytes);
+/* Unmap all chunks, used = 0; replaces preempt_seq (vmm_allocator.cpp:348-381). */
+int vtkv_seg_preempt(vtkv_segment *seg);
+/* Unmap all but the first expand_bytes, used = 0; replaces release_seq (vmm_allocator.cpp:383-421). */
+int vtkv_seg_release(vtkv_segment *seg);
+
+/* Batched bookkeeping of one model step; replaces extend_kv_cache_batch (vmm_allocator.h:138-168).
+ * For i < n: if set_used_tokens[i] > 0, used = set_used_tokens[i]*kv_size; slot_m_out[i] = used;
+ * then gen ? (ensure mapped, used += token_bytes[i]) : reserve(token_bytes[i], kv_size).
+ * Unlike the reference the decode branch maps a chunk itself when the new token crosses the mapped
+ * size (the reference leaves that to a racing background thread). */
+int vtkv_extend_kv_cache_batch(vtkv_segment *const *segs, int n, const int64_t *token_bytes,
+                               const int64_t *set_used_tokens, int64_t kv_size, int gen, int64_t *slot_m_out);
+
+/* Device array of `num_seqs` base addresses; replaces KVCache(num_seqs) / getKVCachePtr
+ * (vmm_allocator.cpp:458-470).  Returns a device address, 0 on error. */
+uint64_t vtkv_ptr_table_create(int num_seqs);
+int vtkv_ptr_table_destroy(uint64_t table);
+/* table[slot] = ptr (synchronous); replaces KVCache::AddKVCache (vmm_allocator.cpp:463-466). */
+int vtkv_ptr_table_set(uint64_t table, int slot, uint64_t ptr);
+/* table[j] = K (which=0) or V (which=1) base of segs[j] for `layer`; replaces copy_kv_cache (vmm_allocator.h:170-182). */
+int vtkv_ptr_table_fill(uint64_t table, vtkv_segment *const *segs, int n, int layer, int which);
+
+/* Synchronous byte copies between host memory and any device address (mapped VMM ranges included).
+ * For tests and debugging; replaces write_string / read_string (vmm_allocator.cpp:423-446). */
+int vtkv_memcpy_h2d(uint64_t dst, const void *src, int64_t bytes);
+int vtkv_memcpy_d2h(void *dst, uint64_t src, int64_t bytes);
+
+/* ------------------------------------------------------------------------------------------
+ * Cache ops.  Replace vllm._C.cache_ops (csrc/pybind.cpp:88-117, csrc/cache.h:8-44).
+ * ---------------------------------------------------------------------------------------- */
+
+/* vTensor scatter of new K/V rows; replaces reshape_and_cache (csrc/cache.h:18-29,
+ * csrc/cache_kernels.cu:153-200,257-297).
+ *   key,value      [num_tokens, num_heads, head_size] of src_dtype, row strides in elements
+ *   k_ptrs,v_ptrs  device int64[max_seqs] base addresses (one per slot)
+ *   slot_m         device int64[batch] byte offset of each sequence's next row (<0: skip)
+ *   slot_ids       device int64[batch] slot of each sequence (python `slot_mapping`)
+ *   seq_lens       device int32[batch] rows to write per sequence (ignored when max_seq_len == 1)
+ *   cache_seq_lens device int32[batch] first source row of each sequence (ignored when max_seq_len == 1)
+ * For sequence b, token t < max_seq_len: dst = ptrs[slot_ids[b]] + slot_m[b] + t*num_heads*head_size*e_kv,
+ * src row = (max_seq_len == 1) ? b : cache_seq_lens[b] + t.
+ * kv_dtype == src_dtype copies bits; kv_dtype == VTKV_FP8_E4M3 stores e4m3fn(x / scale) (round to
+ * nearest even, saturating at +-448), slot_m is then in bytes of the fp8 range. */
+int vtkv_reshape_and_cache(const void *key, const void *value, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                           const int64_t *slot_m, const int64_t *slot_ids, const int32_t *seq_lens,
+                           const int32_t *cache_seq_lens, int batch, int max_seq_len, int num_heads, int head_size,
+                           int64_t key_stride, int64_t value_stride, int src_dtype, int kv_dtype, float k_scale,
+                           float v_scale, void *stream);
+
+/* Upstream paged scatter, the layout the reference's kernel tests pin; replaces the 7-argument
+ * reshape_and_cache (csrc/cpu/cache.cpp:103-128, tests/kernels/test_cache.py:115-193).
+ * K cache [num_blocks, H, D/x, block_size, x], V cache [num_blocks, H, D, block_size], x = 16/elem_bytes;
+ * slot_mapping device int64[num_tokens] (<0: skip). */
+int vtkv_reshape_and_cache_paged(const void *key, const void *value, void *key_cache, void *value_cache,
+                                 const int64_t *slot_mapping, int num_tokens, int num_heads, int head_size,
+                                 int block_size, int64_t key_stride, int64_t value_stride, int elem_bytes,
+                                 void *stream);
+
+/* Copy whole blocks between two buffers; replaces swap_blocks (csrc/cache_kernels.cu:24-69).
+ * `mapping` is a HOST int64[num_pairs,2] of (src_block, dst_block); one async copy of block_bytes per
+ * maximal run of consecutive pairs, on `stream`.  Host buffers should be pinned. */
+int vtkv_swap_blocks(const void *src, void *dst, int64_t block_bytes, const int64_t *mapping, int num_pairs,
+                     int direction, void *stream);
+
+/* Move `n` byte ranges (e.g. the mapped K and V ranges of swapped sequences) between device and pinned
+ * host memory: every range is cut into pieces of at most piece_bytes (0 = default 16 MiB) that are dealt
+ * round-robin to `num_streams` internal copy streams (<=8; 0 = default 2).  The copies start after the
+ * work already queued on `stream` and `stream` waits for them to finish (event fork/join), so callers
+ * keep ordinary stream semantics.  vTensor form of CacheEngine.swap_in/swap_out
+ * (vllm/worker/cache_engine.py:131-139): the unit is a sequence's range, not a 16-token block. */
+int vtkv_swap_ranges(const uint64_t *src, const uint64_t *dst, const int64_t *bytes, int n, int direction,
+                     int64_t piece_bytes, int num_streams, void *stream);
+
+/* Pinned host arena for swapped-out KV. */
+void *vtkv_host_alloc(int64_t bytes);
+int vtkv_host_free(void *p);
+
+/* In-GPU block copies across layers; replaces copy_blocks (csrc/cache_kernels.cu:74-149).
+ * key_caches/value_caches: HOST arrays of num_layers device base addresses; `mapping`: DEVICE
+ * int64[num_pairs,2]; block_bytes must be a multiple of 16. */
+int vtkv_copy_blocks(const uint64_t *key_caches, const uint64_t *value_caches, int num_layers,
+                     const int64_t *mapping, int num_pairs, int64_t block_bytes, void *stream);
+
+/* Elementwise fp8 conversion; replaces convert_fp8 (csrc/cache_kernels.cu:346-422).
+ * to_fp8 != 0: dst u8[n] = e4m3fn(src[n] / scale); else dst[n] = float(src u8[n]) * scale.
+ * wide_dtype is the non-fp8 side (VTKV_F32, VTKV_BF16 or VTKV_F16). */
+int vtkv_convert_fp8(void *dst, const void *src, int64_t n, float scale, int to_fp8, int wide_dtype, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Decode attention.  Replaces paged_attention_v1 / v2 (csrc/ops.h:6-19, csrc/attention/
+ * attention_kernels.cu:85-448,608-737; split-K form :451-583) and the external fwd_kvcache
+ * call (vllm/attention/backends/xformers.py:407-430).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Bytes of scratch vtkv_decode_attention needs for these sizes (partition_tokens: 0 = library default). */
+int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_seq_len,
+                                              int partition_tokens);
+
+/* out[b,h,:] = softmax(scale * q[b,h,:] . K_b^T [+ alibi]) V_b over the first seq_lens[b] rows of the
+ * sequence's contiguous [T, num_kv_heads, head_size] K and V ranges, kv head = h / (num_heads/num_kv_heads).
+ *   out        [num_seqs, num_heads, head_size] out_dtype, contiguous; out_dtype is q_dtype as in the
+ *              reference, or VTKV_F32 to receive the result before its final rounding
+ *   q          [num_seqs, num_heads, head_size] q_dtype, row stride q_stride elements
+ *   k_ptrs,v_ptrs device int64[max_seqs]; slot_ids device int64[num_seqs]; seq_lens device int32[num_seqs]
+ *   max_seq_len  host upper bound of seq_lens (sizes the grid, as in the reference launcher)
+ *   alibi_slopes device float[num_heads] or NULL
+ *   kv_dtype     q_dtype, or VTKV_FP8_E4M3 with k_scale / v_scale (x = code * scale)
+ *   workspace    device scratch of at least vtkv_decode_attention_workspace_bytes(...) bytes
+ * Supported: q_dtype VTKV_BF16, head_size 128, num_heads/num_kv_heads in 1..16. */
+int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                          const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
+                          int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                          const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                          float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
+                          void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VTKV_H */

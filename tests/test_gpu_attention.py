@@ -1,0 +1,117 @@
+"""GPU parity of decode attention: the HIP split-K kernel, called through the C ABI, against the
+CPU oracle on the same seeded inputs.
+
+Tolerance for bf16 KV: |gpu - oracle| <= 2e-3 + 2e-3 * |oracle|, checked on the values BEFORE the
+final store to bf16 on both sides (fp32 `out` on the GPU; the oracle run with an fp32 query/output
+holding the same bf16-representable values): a bf16 store alone moves a value by up to 2^-8 = 3.9e-3
+relative, so two correctly computed bf16 tensors can differ by more than the tolerance.  For the
+bf16 output the checks are: it is the round-to-nearest-even of the kernel's fp32 result bit for
+bit, and it is never more than one bf16 step from the oracle's bf16 output."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from_bits
+
+pytestmark = pytest.mark.gpu
+
+ATOL = RTOL = 2e-3
+
+
+def run_case(vmm, seed, seq_lens, hq, hkv, d=128, partition_tokens=0, alibi=False, shuffle_slots=True, version="v1"):
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(seed)
+    b = len(seq_lens)
+    num_slots = b + 3
+    slots = rng.permutation(num_slots)[:b] if shuffle_slots else np.arange(b)
+    gpu = GpuSeqs(vmm, num_slots, hkv, d, 2, max(seq_lens))
+    k_host = [np.zeros((1, hkv, d), np.uint16) for _ in range(num_slots)]
+    v_host = [np.zeros((1, hkv, d), np.uint16) for _ in range(num_slots)]
+    for i, t in enumerate(seq_lens):
+        k_host[slots[i]] = bf16_randn(rng, (t, hkv, d))
+        v_host[slots[i]] = bf16_randn(rng, (t, hkv, d))
+        gpu.upload(int(slots[i]), k_host[slots[i]], v_host[slots[i]])
+    q = bf16_randn(rng, (b, hq, d))
+    scale = float(d) ** -0.5
+    slopes = rng.standard_normal(hq).astype(np.float32) if alibi else None
+
+    cache = O.VTensorCache(k_host, v_host, slots, hkv, d)
+    expect = O.paged_attention_v1(q, cache, scale, seq_lens, slopes)               # bf16, round to nearest
+    expect32 = O.paged_attention_v1(O.bf16_to_f32(q), cache, scale, seq_lens, slopes)  # before the final rounding
+
+    kt, vt = gpu.table_tensors()
+    out = torch.empty(b, hq, d, dtype=torch.bfloat16, device="cuda")
+    out32 = torch.empty(b, hq, d, dtype=torch.float32, device="cuda")
+    q_t = torch_bf16_from_bits(q)
+    sl_t = torch.tensor(seq_lens, dtype=torch.int32, device="cuda")
+    slot_t = torch.tensor(slots, dtype=torch.int64, device="cuda")
+    al_t = None if slopes is None else torch.from_numpy(slopes).cuda()
+    for o in (out, out32):
+        if version == "v1":
+            ops.paged_attention_v1(o, q_t, kt, vt, hkv, scale, sl_t, 1, max(seq_lens), al_t, "auto", 1.0, slot_t,
+                                   partition_tokens=partition_tokens)
+        else:
+            ops.paged_attention_v2(o, None, None, None, q_t, kt, vt, hkv, scale, sl_t, 1, max(seq_lens), al_t,
+                                   "auto", 1.0, slot_t)
+    torch.cuda.synchronize()
+    got_bits = bits_from_torch_bf16(out)
+    got = out32.cpu().numpy()
+    want = O.bf16_to_f32(expect)
+    gpu.close()
+    assert np.array_equal(got_bits, O.f32_to_bf16(got)), "bf16 output is not RNE(fp32 output)"
+    err = np.abs(got - expect32)
+    bound = ATOL + RTOL * np.abs(expect32)
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert np.all(err <= bound), (f"max err {err.max():.3e}, worst excess {(err - bound).max():.3e} at (seq, head, d)="
+                                  f"{worst}: got {got[worst]!r} want {expect32[worst]!r}, len {seq_lens[worst[0]]}"
+                                  + (f", slope {slopes[worst[1]]!r}" if slopes is not None else ""))
+    # bf16 results: at most one representable step apart (sign-magnitude bit patterns are ordered)
+    def key(bits):
+        b = bits.astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
+    steps = np.abs(key(got_bits) - key(expect))
+    big = np.abs(expect32) >= 2.0 ** -6   # below that a bf16 step is < 3.1e-5 and the absolute bound rules
+    assert steps[big].max(initial=0) <= 1, f"{(steps[big] > 1).sum()} elements differ by more than one bf16 step"
+    return got, want
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (8, 8), (16, 1)])
+def test_small_edge_lengths(gpu_pool, hq, hkv):
+    # lengths straddling the 16-row tile, the 64-row wave stride and the 256-row partition
+    run_case(gpu_pool, 1, [1, 15, 16, 17, 63, 64, 65, 255, 256, 257, 511, 512, 513, 1025], hq, hkv)
+
+
+def test_config2_shape_llama8b(gpu_pool):
+    # batch 64, Hq 32, Hkv 8, ctx uniform in [512, 4096]
+    rng = np.random.default_rng(1001)
+    lens = rng.integers(512, 4097, 64).tolist()
+    run_case(gpu_pool, 1001, lens, 32, 8)
+
+
+@pytest.mark.parametrize("pt", [64, 128, 512, 1024])
+def test_partition_count_invariance(gpu_pool, pt):
+    # the result must not depend on how the rows are split (v1 == v2 in the reference's tests)
+    lens = [700, 64, 1500, 2049]
+    got, _ = run_case(gpu_pool, 7, lens, 32, 8, partition_tokens=pt)
+    base, _ = run_case(gpu_pool, 7, lens, 32, 8, partition_tokens=256)
+    assert np.abs(got - base).max() <= 2e-3
+
+
+def test_v2_entry_point(gpu_pool):
+    run_case(gpu_pool, 3, [513, 2000, 100], 32, 8, version="v2")
+
+
+def test_alibi(gpu_pool):
+    run_case(gpu_pool, 5, [33, 400, 1000], 32, 8, alibi=True)
+
+
+def test_single_token_returns_value_row(gpu_pool):
+    # T = 1: softmax over one logit is 1, so out = V[0] bit for bit
+    import torch
+
+    got, want = run_case(gpu_pool, 11, [1, 1, 1], 32, 8)
+    assert np.array_equal(got, want)  # fp32 result equals the (bf16-valued) V row exactly
