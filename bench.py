@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the vTensor KV-cache hot path on one MI355X.
+
+A step is one decode step of one layer over one batch: per-sequence range bookkeeping (map a
+2 MiB chunk where a sequence crosses a boundary), upload of the byte offsets and sequence
+lengths, `reshape_and_cache` of one new token per sequence, and decode attention over the whole
+context.  Inputs are synthetic (N(0,1) cast to the KV dtype) and resident in HBM before timing.
+
+Prints one JSON line: the BASELINE metric, a `roofline` object for the dominant kernel (HIP-event
+timed inside this process) and a `cpu_baseline` object (the reference's CPU attention timed on this
+host on a bounded sample of the same workload).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+
+CONFIGS = {
+    # BASELINE.json configs[1]: Llama-3-8B-shaped single-layer decode, bf16
+    "c2": dict(name="llama3-8b-decode-bf16 B=64 Hq=32 Hkv=8 D=128 ctx~U[512,4096]", batch=64, hq=32, hkv=8, d=128,
+               lo=512, hi=4096, seed=1001, kv="bf16"),
+    # configs[2]: long-context split-K decode
+    "c3": dict(name="long-context-decode-bf16 B=4 Hq=32 Hkv=8 D=128 ctx~U[32768,131072]", batch=4, hq=32, hkv=8,
+               d=128, lo=32768, hi=131072, seed=1002, kv="bf16"),
+    # configs[4] without its swap events: 256 sequences
+    "c5": dict(name="growth-bf16 B=256 Hq=32 Hkv=8 D=128 ctx~U[256,2048]", batch=256, hq=32, hkv=8, d=128, lo=256,
+               hi=2048, seed=1004, kv="bf16"),
+}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--partition-tokens", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (nothing in the KV-cache hot path communicates); "
+              "use --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from glake_amd import _C, _custom_ops as ops, vmm_allocator as vmm
+    from glake_amd.worker.cache_engine import CacheEngine
+
+    cfg = CONFIGS[args.config]
+    B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
+    K, W = args.steps, args.warmup
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda", 0)
+    gen = torch.Generator().manual_seed(cfg["seed"])
+    ctx0 = torch.randint(cfg["lo"], cfg["hi"] + 1, (B,), generator=gen).tolist()
+    total_steps = 2 * (K + W) + 4  # timed pass + kernel-timing pass, each with warm-up
+    row = Hkv * D * 2
+    max_tokens = max(ctx0) + total_steps + 1
+    chunks_per_range = (max_tokens * row + (2 << 20) - 1) // (2 << 20)
+    vmm.init_physical_handle(2 * B * chunks_per_range + 16, 0)
+    engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.bfloat16, max_num_seqs=B,
+                         max_num_batched_tokens=max_tokens, swap_space_bytes=1 << 30)
+    segs = engine.vmm_kvcache_segment
+
+    # ---- resident synthetic KV: N(0,1) -> bf16, written straight into the mapped ranges
+    ggen = torch.Generator(device=dev).manual_seed(cfg["seed"])
+    for b in range(B):
+        nbytes = ctx0[b] * row
+        segs[b].expandMultiSegment((nbytes + (2 << 20) - 1) // (2 << 20))
+        for base in (segs[b].getKeyDevicePtr(0), segs[b].getValueDevicePtr(0)):
+            t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            ops.swap_ranges([t.data_ptr()], [base], [nbytes], "d2d")
+            torch.cuda.synchronize()
+        segs[b].set_used_size(nbytes)
+    q = torch.randn(B, Hq * D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    new_k = torch.randn(B, Hkv * D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    new_v = torch.randn(B, Hkv * D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
+    slot_ids = list(range(B))
+    slot_t = torch.arange(B, dtype=torch.int64, device=dev)
+    scale = float(D) ** -0.5
+    kv_size = row
+
+    # pinned staging rows, one per step, so an async upload never races the next step's host writes
+    stage_m = torch.empty(total_steps, B, dtype=torch.int64).pin_memory()
+    stage_l = torch.empty(total_steps, B, dtype=torch.int32).pin_memory()
+    slot_m_t = torch.empty(B, dtype=torch.int64, device=dev)
+    lens_t = torch.empty(B, dtype=torch.int32, device=dev)
+    state = {"step": 0, "lens": list(ctx0)}
+    zeros = [0] * B
+    tok_bytes = [kv_size] * B
+
+    def step() -> int:
+        i = state["step"]
+        # 1. range bookkeeping (maps a chunk on a 2 MiB boundary), llama.py:340
+        slot_m = vmm.extend_kv_cache_batch(None, None, slot_ids, tok_bytes, segs, zeros, kv_size, True)
+        lens = state["lens"] = [n + 1 for n in state["lens"]]
+        stage_m[i].copy_(torch.tensor(slot_m, dtype=torch.int64))
+        stage_l[i].copy_(torch.tensor(lens, dtype=torch.int32))
+        slot_m_t.copy_(stage_m[i], non_blocking=True)
+        lens_t.copy_(stage_l[i], non_blocking=True)
+        max_len = max(lens)
+        # 2. append the new token's K/V rows
+        ops.reshape_and_cache(new_k, new_v, engine.k_cache_ptr[0], engine.v_cache_ptr[0], slot_m_t, slot_t, None,
+                              None, 1, Hkv, D)
+        # 3. decode attention over the whole context
+        ops.paged_attention_v1(out, q.view(B, Hq, D), engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hkv, scale,
+                               lens_t, 1, max_len, None, "auto", 1.0, slot_t,
+                               partition_tokens=args.partition_tokens)
+        state["step"] = i + 1
+        return sum(lens)
+
+    def attn_bytes(sum_ctx: int) -> int:
+        # K+V rows of every context token, plus q in and out out
+        return sum_ctx * 2 * Hkv * D * 2 + B * Hq * D * 2 + B * Hq * D * 2
+
+    # ---- timed region: exactly K steps, synchronised on both sides
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    bytes_total = 0
+    for _ in range(K):
+        bytes_total += attn_bytes(step()) + B * 2 * Hkv * D * (2 + 2)  # + reshape_and_cache in/out
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / K * 1e3
+    gbps = bytes_total / dt / 1e9
+    tokens_per_s = B * K / dt
+
+    # ---- per-kernel pass: HIP events around the split-K kernel on the stream it runs on
+    lib = _C.lib()
+    _C.check(lib.vtkv_set_kernel_timing(1))
+    part_ms, red_ms, kbytes = [], [], []
+    a, b_ = C.c_float(), C.c_float()
+    for i in range(W + K):
+        s = step()
+        _C.check(lib.vtkv_last_attention_kernel_ms(C.byref(a), C.byref(b_)))
+        if i >= W:
+            part_ms.append(a.value)
+            red_ms.append(b_.value)
+            kbytes.append(attn_bytes(s))
+    _C.check(lib.vtkv_set_kernel_timing(0))
+    avg_part_ms = float(np.mean(part_ms))
+    achieved = float(np.mean(kbytes)) / (avg_part_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                "kernel": "decode_attn_partial_kernel", "avg_kernel_us": round(avg_part_ms * 1e3, 2),
+                "avg_reduce_kernel_us": round(float(np.mean(red_ms)) * 1e3, 2),
+                "algorithmic_bytes_per_launch": int(np.mean(kbytes))}
+
+    # ---- swap: 25 % of the sequences out to pinned host memory and back
+    nswap = max(1, B // 4)
+    swap_slots = list(range(nswap))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    moved = engine.swap_out(swap_slots)
+    t1 = time.perf_counter()
+    engine.swap_in(swap_slots)
+    t2 = time.perf_counter()
+    swap = {"bytes_per_direction": moved, "out_gbps": round(moved / (t1 - t0) / 1e9, 2),
+            "in_gbps": round(moved / (t2 - t1) / 1e9, 2), "sequences": nswap}
+
+    result = {
+        "metric": "decode-attn HBM GB/s (% peak) + tokens/s @ Llama-3-8B shape B=64; swap GB/s",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": cfg["name"], "layers": 1, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
+                   "mean_ctx": round(float(np.mean(state["lens"])), 1)},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "tokens_per_s": round(tokens_per_s, 1),
+        "swap": swap,
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg, engine, state["lens"], q, scale, args.cpu_seconds)
+
+    print(json.dumps(result))
+    engine.close()
+    return 0
+
+
+def cpu_baseline(cfg, engine, lens, q, scale, budget_s: float):
+    """The reference's CPU paged attention v1 (compiled from the reference sources when that
+    build is present, otherwise the C restatement) on the first sequences of the same batch, in the
+    paged block-16 layout it requires."""
+    import torch
+
+    from glake_amd import _C
+    from oracle import oracle as O
+
+    B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
+    nsample = min(B, 16)
+    bs, x = 16, 8
+    lens = lens[:nsample]
+    nblk = [(n + bs - 1) // bs for n in lens]
+    k_cache = np.zeros((sum(nblk), Hkv, D // x, bs, x), np.uint16)
+    v_cache = np.zeros((sum(nblk), Hkv, D, bs), np.uint16)
+    block_tables = np.zeros((nsample, max(nblk)), np.int32)
+    blk0 = 0
+    for b in range(nsample):
+        seg = engine.vmm_kvcache_segment[b]
+        n = lens[b]
+        rows = np.zeros((nblk[b] * bs, Hkv, D), np.uint16)
+        for which, dst in ((0, k_cache), (1, v_cache)):
+            src = seg.getKeyDevicePtr(0) if which == 0 else seg.getValueDevicePtr(0)
+            _C.check(_C.lib().vtkv_memcpy_d2h(rows.ctypes.data_as(C.c_void_p), src, n * Hkv * D * 2))
+            blk = rows.reshape(nblk[b], bs, Hkv, D)
+            if which == 0:  # [blk, bs, H, D/x, x] -> [blk, H, D/x, bs, x]
+                dst[blk0:blk0 + nblk[b]] = blk.reshape(nblk[b], bs, Hkv, D // x, x).transpose(0, 2, 3, 1, 4)
+            else:           # [blk, bs, H, D] -> [blk, H, D, bs]
+                dst[blk0:blk0 + nblk[b]] = blk.transpose(0, 2, 3, 1)
+        block_tables[b, :nblk[b]] = np.arange(blk0, blk0 + nblk[b])
+        blk0 += nblk[b]
+    q_np = q.view(B, Hq, D)[:nsample].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    sl = np.array(lens, np.int32)
+    if O.ref_available():
+        kind = "reference"
+        run = lambda: O.ref_paged_attention(1, q_np, k_cache, v_cache, block_tables, sl, scale)
+        cores = int(O.ref().ref_num_threads())
+    else:
+        kind = "port"
+        pc = O.PagedCache(k_cache, v_cache, block_tables)
+        run = lambda: O.paged_attention_v1(q_np, pc, scale, sl)
+        cores = O.num_threads()
+    run()  # warm-up (thread pool, page faults)
+    t0 = time.perf_counter()
+    iters = 0
+    while True:
+        run()
+        iters += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or iters >= 1000:
+            break
+    per_call = el / iters
+    nbytes = sum(lens) * 2 * Hkv * D * 2 + 2 * nsample * Hq * D * 2
+    return {"value": round(nbytes / per_call / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind,
+            "tokens_per_s": round(nsample / per_call, 1), "ms_per_call": round(per_call * 1e3, 3),
+            "sample": f"paged_attention_v1 (block 16, bf16) on the first {nsample} of {B} sequences "
+                      f"({sum(lens)} context tokens), {iters} calls in {el:.1f} s"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,175 @@
+"""The attention backend of this package: same interface and metadata fields as the reference's
+one working backend (``vllm/attention/backends/xformers.py``: ``XFormersBackend`` :25-62,
+``XFormersMetadata`` :65-211, ``XFormersImpl`` :214-433), with the cache write and the decode
+attention served by the HIP kernels of ``libvtkv.so``.
+
+Decode is complete.  Prefill writes its rows into the cache; prefill attention itself belongs
+to a different kernel family and raises ``NotImplementedError``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple, Type
+
+import torch
+
+from ..ops.paged_attn import PagedAttention, PagedAttentionMetadata
+from .abstract import AttentionBackend, AttentionImpl, AttentionMetadata
+
+
+class VTensorBackend(AttentionBackend):
+    @staticmethod
+    def get_name() -> str:
+        return "vtensor-hip"
+
+    @staticmethod
+    def get_impl_cls() -> Type["VTensorImpl"]:
+        return VTensorImpl
+
+    @staticmethod
+    def make_metadata(*args, **kwargs) -> "VTensorMetadata":
+        return VTensorMetadata(*args, **kwargs)
+
+    @staticmethod
+    def get_kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int) -> Tuple[int, ...]:
+        return PagedAttention.get_kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size)
+
+    @staticmethod
+    def swap_blocks(src_kv_cache: torch.Tensor, dst_kv_cache: torch.Tensor, src_to_dst: torch.Tensor) -> None:
+        PagedAttention.swap_blocks(src_kv_cache, dst_kv_cache, src_to_dst)
+
+    @staticmethod
+    def copy_blocks(kv_caches: List[torch.Tensor], src_to_dists: torch.Tensor) -> None:
+        PagedAttention.copy_blocks(kv_caches, src_to_dists)
+
+
+@dataclass
+class VTensorMetadata(AttentionMetadata, PagedAttentionMetadata):
+    """Field for field the reference's XFormersMetadata (xformers.py:65-125)."""
+    seq_lens: Optional[List[int]]
+    seq_lens_tensor: Optional[torch.Tensor]
+    max_query_len: Optional[int]
+    max_prefill_seq_len: int
+    max_decode_seq_len: int
+    query_start_loc: Optional[torch.Tensor]
+    seq_start_loc: Optional[torch.Tensor]
+    context_lens_tensor: Optional[torch.Tensor]
+    is_extend: int
+    kv_batch_stride: int
+    kv_num_heads: int
+    kv_head_size: int
+    max_seq_len: int
+    slot_mapping_list: List[int]
+    set_used_size: List[int]
+    extend_seq_list: List[int]
+    use_cuda_graph: bool
+    cache_seq_lens: Optional[torch.Tensor] = None
+    slot_m: Optional[torch.Tensor] = None
+    k_cache_segment_ptr_list: Optional[List[torch.Tensor]] = None
+    v_cache_segment_ptr_list: Optional[List[torch.Tensor]] = None
+    kvcache_segment: Optional[list] = None
+    decode_seq_len: Optional[torch.Tensor] = None
+    _cached_prefill_metadata: Optional["VTensorMetadata"] = None
+    _cached_decode_metadata: Optional["VTensorMetadata"] = None
+
+    def _carry(self) -> Dict:
+        return dict(is_extend=self.is_extend, kv_batch_stride=self.kv_batch_stride, kv_num_heads=self.kv_num_heads,
+                    kv_head_size=self.kv_head_size, max_seq_len=self.max_seq_len,
+                    slot_mapping_list=self.slot_mapping_list, set_used_size=self.set_used_size,
+                    cache_seq_lens=self.cache_seq_lens, slot_m=self.slot_m,
+                    k_cache_segment_ptr_list=self.k_cache_segment_ptr_list,
+                    v_cache_segment_ptr_list=self.v_cache_segment_ptr_list, kvcache_segment=self.kvcache_segment)
+
+    @property
+    def prefill_metadata(self) -> Optional["VTensorMetadata"]:
+        # xformers.py:138-174
+        if self.num_prefills == 0:
+            return None
+        if self._cached_prefill_metadata is None:
+            self._cached_prefill_metadata = VTensorMetadata(
+                num_prefills=self.num_prefills, num_prefill_tokens=self.num_prefill_tokens, num_decode_tokens=0,
+                slot_mapping=self.slot_mapping[:self.num_prefill_tokens], seq_lens=self.seq_lens[:self.num_prefills],
+                seq_lens_tensor=self.seq_lens_tensor[:self.num_prefills], max_query_len=self.max_query_len,
+                max_prefill_seq_len=self.max_prefill_seq_len, max_decode_seq_len=0,
+                query_start_loc=None if self.query_start_loc is None else self.query_start_loc[:self.num_prefills + 1],
+                seq_start_loc=None,
+                context_lens_tensor=None if self.context_lens_tensor is None else self.context_lens_tensor[:self.num_prefills],
+                block_tables=None if self.block_tables is None else self.block_tables[:self.num_prefills],
+                use_cuda_graph=False, extend_seq_list=[], **self._carry())
+        return self._cached_prefill_metadata
+
+    @property
+    def decode_metadata(self) -> Optional["VTensorMetadata"]:
+        # xformers.py:176-211
+        if self.num_decode_tokens == 0:
+            return None
+        if self._cached_decode_metadata is None:
+            self._cached_decode_metadata = VTensorMetadata(
+                num_prefills=0, num_prefill_tokens=0, num_decode_tokens=self.num_decode_tokens,
+                slot_mapping=self.slot_mapping, seq_lens=None, seq_lens_tensor=self.seq_lens_tensor,
+                max_query_len=None, max_prefill_seq_len=0, max_decode_seq_len=self.max_decode_seq_len,
+                query_start_loc=None, seq_start_loc=None, context_lens_tensor=None,
+                block_tables=None if self.block_tables is None else self.block_tables[self.num_prefills:],
+                use_cuda_graph=self.use_cuda_graph, extend_seq_list=self.extend_seq_list, **self._carry())
+        return self._cached_decode_metadata
+
+
+class VTensorImpl(AttentionImpl[VTensorMetadata]):
+    """xformers.py:214-433 with the external flash-decoding call replaced by the in-tree kernel."""
+
+    def __init__(self, num_heads: int, head_size: int, scale: float, num_kv_heads: Optional[int] = None,
+                 alibi_slopes: Optional[List[float]] = None, sliding_window: Optional[int] = None,
+                 kv_cache_dtype: str = "auto") -> None:
+        self.num_heads = num_heads
+        self.head_size = head_size
+        self.scale = float(scale)
+        self.num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
+        if alibi_slopes is not None:
+            alibi_slopes = torch.tensor(alibi_slopes, dtype=torch.float32)
+        self.alibi_slopes = alibi_slopes
+        self.sliding_window = sliding_window
+        self.kv_cache_dtype = kv_cache_dtype
+        assert self.num_heads % self.num_kv_heads == 0
+        self.num_queries_per_kv = self.num_heads // self.num_kv_heads
+        supported = PagedAttention.get_supported_head_sizes()
+        if head_size not in supported:
+            raise ValueError(f"Head size {head_size} is not supported by PagedAttention. "
+                             f"Supported head sizes are: {supported}.")
+        if sliding_window is not None:
+            raise ValueError("sliding-window attention is not supported by the vtensor backend")
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, key_cache, value_cache,
+                attn_metadata: VTensorMetadata, kv_scale: float = 1.0, v_scale: Optional[float] = None) -> torch.Tensor:
+        """query [N, Hq*D], key/value [N, Hkv*D]; key_cache / value_cache are the per-layer
+        ``KV_cache`` handles (xformers.py:269-278); returns [N, Hq*D]."""
+        query = query.view(-1, self.num_heads, self.head_size)
+        key = key.view(-1, self.num_kv_heads, self.head_size)
+        value = value.view(-1, self.num_kv_heads, self.head_size)
+        vs = kv_scale if v_scale is None else v_scale
+
+        if key_cache is not None:
+            # xformers.py:290-312: one row per sequence in decode, max_query_len rows in prefill
+            max_seq_len = 1 if attn_metadata.num_prefill_tokens == 0 else attn_metadata.max_query_len
+            PagedAttention.write_to_paged_cache(
+                key, value, attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
+                attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], attn_metadata.slot_m,
+                attn_metadata.slot_mapping, attn_metadata.seq_lens_tensor, attn_metadata.cache_seq_lens, max_seq_len,
+                self.num_kv_heads, self.head_size, self.kv_cache_dtype, kv_scale, vs)
+
+        num_prefill_tokens = attn_metadata.num_prefill_tokens
+        num_decode_tokens = attn_metadata.num_decode_tokens
+        assert key.shape[0] == num_prefill_tokens + num_decode_tokens
+        if attn_metadata.prefill_metadata is not None:
+            raise NotImplementedError("prefill attention is outside the decode hot path of this backend")
+
+        output = None
+        if attn_metadata.decode_metadata is not None:
+            assert key_cache is not None, "decode needs a KV cache"
+            output = PagedAttention.forward_decode(
+                query[num_prefill_tokens:], attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
+                attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], attn_metadata.seq_lens_tensor,
+                attn_metadata.max_seq_len, self.kv_cache_dtype, self.num_kv_heads, self.scale, self.alibi_slopes,
+                kv_scale, attn_metadata.slot_mapping, vs)
+        if output is None:
+            output = torch.empty_like(query)
+        return output.view(-1, self.num_heads * self.head_size)

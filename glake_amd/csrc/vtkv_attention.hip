@@ -291,6 +291,15 @@ __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
     reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
 }
 
+// Optional per-kernel timing for benchmarks: when switched on, every vtkv_decode_attention call
+// records events around its two launches on the caller's stream.
+struct KernelTimer {
+  bool on = false;
+  hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+  bool recorded = false;
+};
+KernelTimer g_timer;
+
 int default_part_tokens(int max_seq_len) {
   (void)max_seq_len;
   return 256;
@@ -362,10 +371,34 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   (void)v_scale;
 
   hipStream_t st = (hipStream_t)stream;
+  const bool timed = g_timer.on;
+  if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[0], st));
   hipLaunchKernelGGL(decode_attn_partial_kernel<false>, dim3(num_kv_heads, (unsigned)parts, num_seqs),
                      dim3(kWaves * 64), 0, st, p);
+  if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[1], st));
   hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
+  if (timed) {
+    VTKV_HIP(hipEventRecord(g_timer.ev[2], st));
+    g_timer.recorded = true;
+  }
   VTKV_HIP(hipGetLastError());
+  return VTKV_OK;
+}
+
+int vtkv_set_kernel_timing(int on) {
+  if (on && !g_timer.ev[0])
+    for (auto &e : g_timer.ev) VTKV_HIP(hipEventCreate(&e));
+  g_timer.on = on != 0;
+  g_timer.recorded = false;
+  return VTKV_OK;
+}
+
+int vtkv_last_attention_kernel_ms(float *partial_ms, float *reduce_ms) {
+  VTKV_REQUIRE(partial_ms && reduce_ms, "null argument");
+  if (!g_timer.recorded) return vtkv::fail(VTKV_ESTATE, "no timed vtkv_decode_attention call to report");
+  VTKV_HIP(hipEventSynchronize(g_timer.ev[2]));
+  VTKV_HIP(hipEventElapsedTime(partial_ms, g_timer.ev[0], g_timer.ev[1]));
+  VTKV_HIP(hipEventElapsedTime(reduce_ms, g_timer.ev[1], g_timer.ev[2]));
   return VTKV_OK;
 }
 

@@ -1,0 +1,171 @@
+"""KV cache owner for the vTensor layout: one address-range segment per sequence slot, per-layer
+pointer tables, and the host arena that swapped-out sequences live in.
+
+Counterpart of the reference's ``CacheEngine`` (vllm/worker/cache_engine.py:19-142), taking plain
+sizes instead of vLLM config objects.  Swap works on whole sequences: the reference's block-wise
+``swap_in/swap_out`` (:131-139) is vestigial for vTensor (its ``gpu_cache`` holds pointer
+tables, not tensors, and it runs with zero CPU blocks), so the unit here is "the used bytes of a
+slot's K and V ranges in every layer", moved with chunked multi-stream copies.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .. import _C, _custom_ops as ops, vmm_allocator as vmm
+
+PHY_GRAN = 2 * 1024 * 1024  # cache_engine.py:54
+
+
+def _dtype_size(dtype: torch.dtype) -> int:
+    return torch.tensor([], dtype=dtype).element_size()
+
+
+class _HostArena:
+    """First-fit allocator over one pinned host buffer."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = nbytes
+        self.base = int(_C.check_ptr(_C.lib().vtkv_host_alloc(nbytes), "pinned host arena")) if nbytes > 0 else 0
+        self.free: List[Tuple[int, int]] = [(0, nbytes)] if nbytes > 0 else []
+
+    def alloc(self, n: int) -> int:
+        n = (n + 255) // 256 * 256
+        for i, (off, size) in enumerate(self.free):
+            if size >= n:
+                if size == n:
+                    self.free.pop(i)
+                else:
+                    self.free[i] = (off + n, size - n)
+                return off
+        raise _C.VtkvOutOfChunks(_C.ENOMEM, f"host swap arena exhausted: need {n} bytes")
+
+    def release(self, off: int, n: int) -> None:
+        n = (n + 255) // 256 * 256
+        self.free.append((off, n))
+        self.free.sort()
+        merged: List[Tuple[int, int]] = []
+        for o, s in self.free:
+            if merged and merged[-1][0] + merged[-1][1] == o:
+                merged[-1] = (merged[-1][0], merged[-1][1] + s)
+            else:
+                merged.append((o, s))
+        self.free = merged
+
+    def close(self) -> None:
+        if self.base:
+            _C.check(_C.lib().vtkv_host_free(C.c_void_p(self.base)))
+            self.base = 0
+
+
+class CacheEngine:
+    def __init__(self, num_layers: int, num_kv_heads: int, head_size: int, dtype: torch.dtype, max_num_seqs: int,
+                 max_num_batched_tokens: int, cache_seqs: int = 0, cache_tokens: int = 0,
+                 swap_space_bytes: int = 0, device: int = 0) -> None:
+        self.num_layers = num_layers
+        self.num_kv_heads = num_kv_heads
+        self.head_size = head_size
+        self.dtype = dtype
+        self.device = device
+        self.token_size = num_kv_heads * head_size * _dtype_size(dtype)  # bytes of one K (or V) row
+        # cache_engine.py:53-57: every slot reserves room for max_num_batched_tokens rows
+        ctx = max_num_batched_tokens * self.token_size
+        self.max_context_size = PHY_GRAN * ((ctx + PHY_GRAN - 1) // PHY_GRAN)
+        self.kv_batch_stride = self.max_context_size
+        # cache_engine.py:58-71: the first cache_seqs slots keep cache_tokens chunks mapped
+        keep = PHY_GRAN * cache_tokens if cache_seqs > 0 else 0
+        self.vmm_kvcache_segment = [
+            vmm.KVcacheSegment(num_layers, self.max_context_size, keep, cache_seqs > 0 and i < cache_seqs)
+            for i in range(max_num_seqs)
+        ]
+        # cache_engine.py:111-129: per layer one pointer table for K and one for V
+        self.gpu_cache = [(vmm.KV_cache(max_num_seqs, l), vmm.KV_cache(max_num_seqs, l)) for l in range(num_layers)]
+        vmm.copy_kv_cache([k.kv_cache for k, _ in self.gpu_cache], [v.kv_cache for _, v in self.gpu_cache],
+                          self.vmm_kvcache_segment)
+        # cache_engine.py:98-109: the same pointers as int64 device tensors, one per layer
+        self.k_cache_ptr: List[torch.Tensor] = []
+        self.v_cache_ptr: List[torch.Tensor] = []
+        dev = torch.device("cuda", device)
+        for l in range(num_layers):
+            self.k_cache_ptr.append(torch.tensor([s.getKeyDevicePtr(l) for s in self.vmm_kvcache_segment],
+                                                 dtype=torch.long, device=dev))
+            self.v_cache_ptr.append(torch.tensor([s.getValueDevicePtr(l) for s in self.vmm_kvcache_segment],
+                                                 dtype=torch.long, device=dev))
+        self._arena = _HostArena(swap_space_bytes)
+        self._swapped: Dict[int, Tuple[int, int]] = {}  # slot -> (arena offset, used bytes per range)
+
+    # ------------------------------------------------------------------ swap (whole sequences)
+    def swap_out(self, slots: Sequence[int]) -> int:
+        """Copy the used part of every K and V range of `slots` to pinned host memory on the current
+        stream, then unmap the slots (their chunks return to the pool).  Returns bytes moved."""
+        src, dst, nbytes = [], [], []
+        total = 0
+        for slot in slots:
+            if slot in self._swapped:
+                raise _C.VtkvError(_C.ESTATE, f"slot {slot} is already swapped out")
+            seg = self.vmm_kvcache_segment[slot]
+            used = seg.used_size
+            off = self._arena.alloc(2 * self.num_layers * used) if used else 0
+            self._swapped[slot] = (off, used)
+            for l in range(self.num_layers):
+                for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):
+                    if used:
+                        src.append(base)
+                        dst.append(self._arena.base + off + (2 * l + which) * used)
+                        nbytes.append(used)
+                        total += used
+        ops.swap_ranges(src, dst, nbytes, "out")
+        # the copies must have read the ranges before their chunks go back to the pool
+        torch.cuda.current_stream().synchronize()
+        for slot in slots:
+            self.vmm_kvcache_segment[slot].preempt_seq(slot)
+        return total
+
+    def swap_in(self, slots: Sequence[int]) -> int:
+        """Map chunks for `slots` again and copy their KV back from host memory."""
+        src, dst, nbytes = [], [], []
+        total = 0
+        for slot in slots:
+            if slot not in self._swapped:
+                raise _C.VtkvError(_C.ESTATE, f"slot {slot} is not swapped out")
+            off, used = self._swapped[slot]
+            seg = self.vmm_kvcache_segment[slot]
+            need = (used + PHY_GRAN - 1) // PHY_GRAN - seg.actual_size // PHY_GRAN
+            if need > 0:
+                seg.expandMultiSegment(need)
+            seg.set_used_size(used)
+            for l in range(self.num_layers):
+                for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):
+                    if used:
+                        src.append(self._arena.base + off + (2 * l + which) * used)
+                        dst.append(base)
+                        nbytes.append(used)
+                        total += used
+        ops.swap_ranges(src, dst, nbytes, "in")
+        torch.cuda.current_stream().synchronize()  # the arena space is reused after this
+        for slot in slots:
+            off, used = self._swapped.pop(slot)
+            if used:
+                self._arena.release(off, 2 * self.num_layers * used)
+        return total
+
+    # ------------------------------------------------------------------ block-wise API of the reference
+    def copy(self, src_to_dsts: torch.Tensor) -> None:
+        raise NotImplementedError("block copies have no meaning for per-sequence contiguous ranges; "
+                                  "use _custom_ops.copy_blocks on paged tensors")
+
+    @staticmethod
+    def get_cache_block_size(block_size: int, num_kv_heads: int, head_size: int, num_layers: int,
+                             dtype: torch.dtype) -> int:
+        # cache_engine.py:144-162
+        return _dtype_size(dtype) * num_layers * 2 * block_size * num_kv_heads * head_size
+
+    def close(self) -> None:
+        for seg in self.vmm_kvcache_segment:
+            seg.destroy()
+        for k, v in self.gpu_cache:
+            k.kv_cache.destroy()
+            v.kv_cache.destroy()
+        self._arena.close()

@@ -208,6 +208,14 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                           float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
                           void *stream);
 
+/* Benchmark aid without a counterpart in the reference (its kernel benchmark times from the host,
+ * benchmarks/kernels/benchmark_paged_attention.py:147-157): when switched on, each
+ * vtkv_decode_attention call records HIP events around its kernels on the caller's stream, and
+ * vtkv_last_attention_kernel_ms waits for the last such call and returns the duration of its split-K
+ * kernel and of its merge kernel in milliseconds. */
+int vtkv_set_kernel_timing(int on);
+int vtkv_last_attention_kernel_ms(float *partial_ms, float *reduce_ms);
+
 #ifdef __cplusplus
 }
 #endif
