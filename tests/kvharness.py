@@ -47,6 +47,18 @@ class GpuSeqs:
         _C.check(_C.lib().vtkv_memcpy_h2d(seg.getValueDevicePtr(layer), v_rows.ctypes.data_as(C.c_void_p), nbytes))
         seg.set_used_size(nbytes)
 
+    def map_zeroed(self, nbytes, layer=0):
+        """Map enough chunks for nbytes in every slot and clear them (fresh chunks hold stale data)."""
+        from glake_amd import _C
+
+        zeros = np.zeros(nbytes, np.uint8)
+        for seg in self.segs:
+            need = round_up(nbytes, CHUNK) - seg.actual_size
+            if need > 0:
+                seg.expandMultiSegment(need // CHUNK)
+            for dst in (seg.getKeyDevicePtr(layer), seg.getValueDevicePtr(layer)):
+                _C.check(_C.lib().vtkv_memcpy_h2d(dst, zeros.ctypes.data_as(C.c_void_p), nbytes))
+
     def download(self, slot, nbytes, layer=0, which="k", dtype=np.uint8):
         from glake_amd import _C
 

@@ -1,0 +1,120 @@
+"""Dynamic growth plus swap (BASELINE config 5): sequences append one token per step, map a new
+2 MiB chunk when they cross a boundary, and a seeded quarter of them is swapped out to pinned host
+memory and back every 16 steps.  Every KV byte is checked exactly; attention is checked against
+the oracle on a sample of sequences at the end."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+from kvharness import CHUNK, bits_from_torch_bf16, torch_bf16_from_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def download(seg, nbytes, which):
+    from glake_amd import _C
+
+    out = np.empty(nbytes // 2, np.uint16)
+    src = seg.getKeyDevicePtr(0) if which == 0 else seg.getValueDevicePtr(0)
+    _C.check(_C.lib().vtkv_memcpy_d2h(out.ctypes.data_as(C.c_void_p), src, nbytes))
+    return out
+
+
+@pytest.mark.parametrize("num_seqs,steps", [(32, 20), (256, 64)])
+def test_growth_and_swap_round_trips_are_bit_exact(gpu_pool, num_seqs, steps):
+    import torch
+
+    from glake_amd import _custom_ops as ops, vmm_allocator as vmm
+    from glake_amd.worker.cache_engine import CacheEngine
+
+    hq, hkv, d = 32, 8, 128
+    row = hkv * d * 2
+    gen = torch.Generator().manual_seed(1004)
+    ctx = torch.randint(256, 2049, (num_seqs,), generator=gen).tolist()
+    # make sure some sequences cross a chunk boundary (1024 rows) during the run
+    ctx[0], ctx[1], ctx[2] = 1024 - 3, 1024, 2048 - steps // 2
+    free0 = vmm.showFreeBlocks()
+    eng = CacheEngine(1, hkv, d, torch.bfloat16, num_seqs, 2048 + steps + 8, swap_space_bytes=num_seqs // 4 * 2 * 3 * CHUNK)
+    segs = eng.vmm_kvcache_segment
+    dev = torch.device("cuda")
+    ggen = torch.Generator(device=dev).manual_seed(7)
+    expect_k, expect_v = [], []
+    for b in range(num_seqs):
+        nbytes = ctx[b] * row
+        segs[b].expandMultiSegment((nbytes + CHUNK - 1) // CHUNK)
+        for which, keep in ((0, expect_k), (1, expect_v)):
+            t = torch.randn(ctx[b], hkv, d, generator=ggen, device=dev).to(torch.bfloat16)
+            base = segs[b].getKeyDevicePtr(0) if which == 0 else segs[b].getValueDevicePtr(0)
+            ops.swap_ranges([t.data_ptr()], [base], [nbytes], "d2d")
+            torch.cuda.synchronize()
+            keep.append([bits_from_torch_bf16(t).reshape(-1)])
+        segs[b].set_used_size(nbytes)
+    slot_t = torch.arange(num_seqs, dtype=torch.int64, device=dev)
+    lens = list(ctx)
+    moved_out = moved_in = 0
+    maps = 0
+    for step in range(1, steps + 1):
+        mapped_before = [s.actual_size for s in segs]
+        slot_m = vmm.extend_kv_cache_batch(None, None, list(range(num_seqs)), [row] * num_seqs, segs,
+                                           [0] * num_seqs, row, True)
+        assert slot_m == [n * row for n in lens]
+        maps += sum(a.actual_size > m for a, m in zip(segs, mapped_before))
+        nk = torch.randn(num_seqs, hkv, d, generator=ggen, device=dev).to(torch.bfloat16)
+        nv = torch.randn(num_seqs, hkv, d, generator=ggen, device=dev).to(torch.bfloat16)
+        ops.reshape_and_cache(nk, nv, eng.k_cache_ptr[0], eng.v_cache_ptr[0],
+                              torch.tensor(slot_m, dtype=torch.int64, device=dev), slot_t, None, None, 1, hkv, d)
+        hk, hv = bits_from_torch_bf16(nk), bits_from_torch_bf16(nv)
+        for b in range(num_seqs):
+            expect_k[b].append(hk[b].reshape(-1))
+            expect_v[b].append(hv[b].reshape(-1))
+        lens = [n + 1 for n in lens]
+        if step % 16 == 0 or (steps < 16 and step == steps // 2):
+            subset = torch.randperm(num_seqs, generator=gen)[:num_seqs // 4].tolist()
+            free_before = vmm.showFreeBlocks()
+            moved_out += eng.swap_out(subset)
+            assert all(segs[s].actual_size == 0 for s in subset)
+            assert vmm.showFreeBlocks() > free_before           # their chunks are back in the pool
+            moved_in += eng.swap_in(subset)
+            assert vmm.showFreeBlocks() == free_before
+            assert all(segs[s].used_size == lens[s] * row for s in subset)
+    assert maps >= 2 and moved_out == moved_in > 0
+    torch.cuda.synchronize()
+    for b in range(num_seqs):
+        want_k, want_v = np.concatenate(expect_k[b]), np.concatenate(expect_v[b])
+        assert np.array_equal(download(segs[b], lens[b] * row, 0), want_k), f"K of sequence {b} differs"
+        assert np.array_equal(download(segs[b], lens[b] * row, 1), want_v), f"V of sequence {b} differs"
+    # attention on a sample (sequence 0 and 1 crossed a chunk boundary) against the oracle
+    sample = [0, 1, 2, num_seqs // 2, num_seqs - 1]
+    q = O.f32_to_bf16(np.random.default_rng(0).standard_normal((num_seqs, hq, d)).astype(np.float32))
+    out = torch.empty(num_seqs, hq, d, dtype=torch.float32, device=dev)
+    ops.paged_attention_v1(out, torch_bf16_from_bits(q), eng.k_cache_ptr[0], eng.v_cache_ptr[0], hkv, d ** -0.5,
+                           torch.tensor(lens, dtype=torch.int32, device=dev), 1, max(lens), None, "auto", 1.0, slot_t)
+    got = out.cpu().numpy()[sample]
+    kb = [np.concatenate(expect_k[b]).reshape(-1, hkv, d) for b in sample]
+    vb = [np.concatenate(expect_v[b]).reshape(-1, hkv, d) for b in sample]
+    want = O.paged_attention_v1(O.bf16_to_f32(q[sample]), O.VTensorCache(kb, vb, np.arange(len(sample)), hkv, d),
+                                d ** -0.5, [lens[b] for b in sample])
+    assert np.all(np.abs(got - want) <= 2e-3 + 2e-3 * np.abs(want))
+    eng.close()
+    assert vmm.showFreeBlocks() == free0
+
+
+def test_swap_ranges_piece_and_stream_variants_are_exact(gpu_pool):
+    import torch
+
+    from glake_amd import _C, _custom_ops as ops
+
+    n = 37 * (1 << 20) + 4096 + 16
+    src = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda")
+    host = int(_C.check_ptr(_C.lib().vtkv_host_alloc(n), "host"))
+    for piece, streams in ((0, 0), (1 << 20, 4), (3 << 20, 8), (n, 1)):
+        back = torch.zeros_like(src)
+        ops.swap_ranges([src.data_ptr(), src.data_ptr() + n // 2], [host, host + n // 2], [n // 2, n - n // 2], "out",
+                        piece, streams)
+        ops.swap_ranges([host], [back.data_ptr()], [n], "in", piece, streams)
+        torch.cuda.synchronize()
+        assert torch.equal(src, back)
+    _C.check(_C.lib().vtkv_host_free(C.c_void_p(host)))

@@ -1,0 +1,141 @@
+"""The HIP virtual-memory chunk pool and per-sequence ranges: integer invariants of the reference's
+allocator (vmm_allocator/vmm_allocator.cpp:214-421) plus what it silently gets wrong (pool
+exhaustion, growth past the reserved range)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from kvharness import CHUNK
+
+pytestmark = pytest.mark.gpu
+
+
+def accounted(vmm, segs):
+    mapped = sum(2 * s.layer_num * (s.actual_size // CHUNK) for s in segs)
+    return vmm.showFreeBlocks() + mapped
+
+
+def test_grow_release_preempt_keep_the_books_balanced(gpu_pool):
+    vmm = gpu_pool
+    free0 = vmm.showFreeBlocks()
+    layers = 3
+    a = vmm.KVcacheSegment(layers, 8 * CHUNK, 2 * CHUNK, True)    # pre-mapped, keeps 2 chunks on release
+    b = vmm.KVcacheSegment(layers, 8 * CHUNK, 0, False)
+    assert a.actual_size == 2 * CHUNK and b.actual_size == 0
+    assert vmm.showFreeBlocks() == free0 - 2 * layers * 2
+    b.expandMultiSegment(3)
+    assert accounted(vmm, [a, b]) == free0
+    a.expandMultiSegment(4)
+    assert a.actual_size == 6 * CHUNK and accounted(vmm, [a, b]) == free0
+    a.set_used_size(5 * CHUNK + 17)
+    a.release_seq(0)                                               # keeps the first expand_size bytes
+    assert a.actual_size == 2 * CHUNK and a.used_size == 0 and accounted(vmm, [a, b]) == free0
+    a.release_seq(0)                                               # res == 0: nothing to do (cpp:393-396)
+    assert a.actual_size == 2 * CHUNK
+    b.release_seq(1)                                               # expand_size 0: everything goes back
+    assert b.actual_size == 0
+    a.preempt_seq(0)
+    assert a.actual_size == 0 and vmm.showFreeBlocks() == free0
+    c = vmm.KVcacheSegment(layers, 8 * CHUNK, 4 * CHUNK, False)
+    c.expandMultiSegment(1)
+    c.release_seq(2)                                               # fewer bytes mapped than expand_size: unmap all (cpp:391-392)
+    assert c.actual_size == 0
+    for s in (a, b, c):
+        s.destroy()
+    assert vmm.showFreeBlocks() == free0
+
+
+def test_pointers_are_stable_and_data_survives_growth(gpu_pool):
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    seg = vmm.KVcacheSegment(2, 6 * CHUNK, 0, False)
+    ptrs = [(seg.getKeyDevicePtr(l), seg.getValueDevicePtr(l)) for l in range(2)]
+    assert len({p for pair in ptrs for p in pair}) == 4 and all(p % CHUNK == 0 for pair in ptrs for p in pair)
+    seg.expandMultiSegment(1)
+    rng = np.random.default_rng(0)
+    blob = rng.integers(0, 256, CHUNK, dtype=np.uint8)
+    _C.check(_C.lib().vtkv_memcpy_h2d(ptrs[1][0], blob.ctypes.data_as(C.c_void_p), CHUNK))
+    seg.expandMultiSegment(2)
+    assert [(seg.getKeyDevicePtr(l), seg.getValueDevicePtr(l)) for l in range(2)] == ptrs
+    # a write spanning the old/new chunk boundary, then read everything back through one pointer
+    tail = rng.integers(0, 256, 2 * CHUNK, dtype=np.uint8)
+    _C.check(_C.lib().vtkv_memcpy_h2d(ptrs[1][0] + CHUNK, tail.ctypes.data_as(C.c_void_p), 2 * CHUNK))
+    got = np.empty(3 * CHUNK, np.uint8)
+    _C.check(_C.lib().vtkv_memcpy_d2h(got.ctypes.data_as(C.c_void_p), ptrs[1][0], 3 * CHUNK))
+    assert np.array_equal(got[:CHUNK], blob) and np.array_equal(got[CHUNK:], tail)
+    seg.destroy()
+
+
+def test_extend_kv_cache_batch_follows_the_reference_bookkeeping(gpu_pool):
+    vmm = gpu_pool
+    kv = 8 * 128 * 2
+    segs = [vmm.KVcacheSegment(1, 4 * CHUNK, 0, False) for _ in range(3)]
+    # prefill: used += prompt bytes, mapped covers prompt + 100 rows of slack (cpp:322-337)
+    prompt = [10 * kv, 1000 * kv, 1024 * kv]
+    slot_m = vmm.extend_kv_cache_batch(None, None, [0, 1, 2], prompt, segs, [0, 0, 0], kv, False)
+    assert slot_m == [0, 0, 0]
+    assert [s.used_size for s in segs] == prompt
+    assert [s.actual_size for s in segs] == [CHUNK, 2 * CHUNK, 2 * CHUNK]
+    # decode: returns the offset of the new row, then advances by one row (vmm_allocator.h:150-157)
+    slot_m = vmm.extend_kv_cache_batch(None, None, [0, 1, 2], [kv] * 3, segs, [0, 0, 0], kv, True)
+    assert slot_m == prompt and [s.used_size for s in segs] == [p + kv for p in prompt]
+    # set_used_size (in rows) rewinds a slot first (h:146-148)
+    slot_m = vmm.extend_kv_cache_batch(None, None, [0, 1, 2], [kv] * 3, segs, [0, 7, 0], kv, True)
+    assert slot_m[1] == 7 * kv and segs[1].used_size == 8 * kv
+    # a decode row that crosses the mapped size maps the next chunk by itself
+    segs[0].set_used_size(CHUNK)
+    free = vmm.showFreeBlocks()
+    slot_m = vmm.extend_kv_cache_batch(None, None, [0], [kv], segs[:1], [0], kv, True)
+    assert slot_m == [CHUNK] and segs[0].actual_size == 2 * CHUNK and vmm.showFreeBlocks() == free - 2
+    for s in segs:
+        s.destroy()
+
+
+def test_exhaustion_and_overflow_fail_cleanly(gpu_pool):
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    free0 = vmm.showFreeBlocks()
+    layers = 4
+    big = vmm.KVcacheSegment(layers, (free0 // (2 * layers) + 8) * CHUNK, 0, False)
+    with pytest.raises(_C.VtkvOutOfChunks):
+        big.expandMultiSegment(free0 // (2 * layers) + 1)          # more chunks than the pool holds
+    assert big.actual_size == 0 and vmm.showFreeBlocks() == free0  # nothing half-mapped
+    small = vmm.KVcacheSegment(1, 2 * CHUNK, 0, False)
+    small.expandMultiSegment(2)
+    with pytest.raises(_C.VtkvError):
+        small.expandMultiSegment(1)                                # beyond the reserved range
+    with pytest.raises(_C.VtkvError):
+        vmm.KVcacheSegment(1, CHUNK + 1, 0, False)                 # not a multiple of the chunk
+    small.destroy()
+    big.destroy()
+    with pytest.raises(_C.VtkvError):
+        small.getKeyDevicePtr(0)                                   # use after destroy is caught
+    assert vmm.showFreeBlocks() == free0
+
+
+def test_write_string_read_string_round_trip(gpu_pool):
+    # the reference's only self-check of the allocator (vmm_allocator/radix_cache.py:256-304)
+    seg = gpu_pool.KVcacheSegment(1, 2 * CHUNK, 0, False)
+    seg.write_string("hello ")
+    seg.write_string("contiguous world")
+    assert seg.read_string() == "hello contiguous world"
+    seg.destroy()
+
+
+def test_pointer_tables(gpu_pool):
+    vmm = gpu_pool
+    segs = [vmm.KVcacheSegment(2, 2 * CHUNK, 0, False) for _ in range(5)]
+    kt, vt = [vmm.KVCache(5) for _ in range(2)], [vmm.KVCache(5) for _ in range(2)]
+    vmm.copy_kv_cache(kt, vt, segs)
+    for l in range(2):
+        assert kt[l].to_numpy().tolist() == [s.getKeyDevicePtr(l) for s in segs]
+        assert vt[l].to_numpy().tolist() == [s.getValueDevicePtr(l) for s in segs]
+    kt[0].AddKVCache(3, 12345)
+    assert kt[0].to_numpy()[3] == 12345
+    for s in segs:
+        s.destroy()
+    for t in kt + vt:
+        t.destroy()
