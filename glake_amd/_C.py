@@ -10,7 +10,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libvtkv.so")
+# VTKV_LIBRARY_PATH selects another build of the same library (e.g. a tuning variant)
+LIB_PATH = os.environ.get("VTKV_LIBRARY_PATH") or os.path.join(_HERE, "lib", "libvtkv.so")
 
 F32, BF16, F16, FP8_E4M3 = 0, 1, 2, 3
 D2H, H2D, D2D = 0, 1, 2

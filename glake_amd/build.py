@@ -20,6 +20,9 @@ SOURCES = ["vtkv_vmm.cpp", "vtkv_cache.hip", "vtkv_attention.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # keep MFMA accumulators in ordinary VGPRs: the softmax rescale multiplies them on the VALU and
+    # the AGPR form would copy all of them back and forth every tile
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wall", "-Wno-unused-function",
 ]
 
@@ -31,15 +34,15 @@ def _hipcc() -> str:
     return exe
 
 
-def build_library(verbose: bool = False) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    obj_dir = os.path.join(_HERE, "build")
+def build_library(verbose: bool = False, out_path: str = LIB_PATH, extra_flags=()) -> str:
+    os.makedirs(os.path.dirname(out_path), exist_ok=True)
+    obj_dir = os.path.join(_HERE, "build", os.path.basename(out_path) + ".o")
     os.makedirs(obj_dir, exist_ok=True)
     hipcc = _hipcc()
 
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *HIP_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
         res = subprocess.run(cmd, capture_output=True, text=True)
         # the host pass does not know the device-only feature flag and says so: not an error
         err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
@@ -51,13 +54,13 @@ def build_library(verbose: bool = False) -> str:
 
     with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
         objs = list(ex.map(compile_one, SOURCES))
-    tmp = LIB_PATH + ".tmp"
+    tmp = out_path + ".tmp"
     res = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs, "-lpthread"],
                          capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("linking libvtkv.so failed:\n" + res.stderr)
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, out_path)
+    return out_path
 
 
 if __name__ == "__main__":

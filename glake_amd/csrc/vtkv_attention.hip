@@ -15,7 +15,7 @@
 //  * softmax statistics stay in registers: in the MFMA C layout a lane owns one head column and four
 //    rows, so a head's max/sum over the tile is an in-lane reduction plus two cross-row-group
 //    exchanges; an online (running-max) rescale keeps one pass.
-//  * O^T += V_tile^T . P^T runs on v_mfma_f32_16x16x16_bf16.  P^T is the C layout of S^T as is.  V is
+//  * O^T += V_tile^T . P^T runs on v_mfma_f32_16x16x32_bf16.  P^T is the C layout of S^T as is.  V is
 //    row-major but the A operand needs four rows per lane, so V tiles go through a wave-private,
 //    XOR-swizzled LDS tile and come back with ds_read_b64_tr_b16 (the transposing LDS read).
 //  * each wave keeps (m, l, O) for its rows; the four waves merge through LDS and the workgroup
@@ -32,6 +32,16 @@
 #include <algorithm>
 
 #include "vtkv_common.h"
+#ifndef VTKV_ATTN_STAGES
+#define VTKV_ATTN_STAGES 2
+#endif
+// register budget of the split-K kernel: N waves per SIMD (it fits 128 VGPRs with one register tile)
+#ifdef VTKV_ATTN_WAVES_PER_EU
+#define VTKV_ATTN_OCCUPANCY __attribute__((amdgpu_waves_per_eu(VTKV_ATTN_WAVES_PER_EU)))
+#else
+#define VTKV_ATTN_OCCUPANCY
+#endif
+static_assert(VTKV_ATTN_STAGES >= 1 && VTKV_ATTN_STAGES <= 4, "1 to 4 register tiles per wave");
 #include "vtkv_fp8.h"
 
 namespace {
@@ -45,6 +55,7 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kD = 128;            // head size
 constexpr int kTile = 16;          // rows per MFMA tile
 constexpr int kWaves = 4;          // waves per workgroup
+constexpr int kStages = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
 constexpr int kRowBytes = kD * 2;  // bf16 row of one head
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -77,8 +88,43 @@ __device__ __forceinline__ int v_lds_offset(int row, int piece16) {
   return row * kRowBytes + ((piece16 ^ ((row & 7) << 1)) << 4);
 }
 
-template <bool FP8>
-__global__ void __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnParams p) {
+// max over the four row groups (lanes l, l^16, l^32, l^48) with the gfx950 lane-swap instructions:
+// v_permlane16_swap exchanges odd 16-lane rows of its first operand with even rows of its second,
+// v_permlane32_swap does the same for 32-lane halves, so swapping a value with itself and taking the
+// max of the two results folds rows pairwise.
+// (the two results are copied to scalars before the bit cast: a bit cast applied directly to an
+// element of the returned vector reads element 0 both times with this compiler)
+__device__ __forceinline__ void swap_rows16(float x, float &a, float &b) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  a = __builtin_bit_cast(float, r0);
+  b = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ void swap_rows32(float x, float &a, float &b) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];
+  a = __builtin_bit_cast(float, r0);
+  b = __builtin_bit_cast(float, r1);
+}
+
+__device__ __forceinline__ float max_over_row_groups(float x) {
+  float a, b;
+  swap_rows16(x, a, b);
+  swap_rows32(fmaxf(a, b), a, b);
+  return fmaxf(a, b);
+}
+
+__device__ __forceinline__ float sum_over_row_groups(float x) {
+  float a, b;
+  swap_rows16(x, a, b);
+  swap_rows32(a + b, a, b);
+  return a + b;
+}
+
+template <bool ALIBI>
+__global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnParams p) {
   // wave-private V tiles (4 KiB each); reused after the main loop for the cross-wave merge
   __shared__ __attribute__((aligned(16))) char smem[kWaves * kTile * kRowBytes + 1024];
 
@@ -88,19 +134,22 @@ __global__ void __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnPa
   if (part_start >= seq_len) return;
   const int part_end = min(seq_len, part_start + p.part_tokens);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  // everything that decides control flow and base addresses is kept wave-uniform (scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 4;   // row group of the MFMA layouts
   const int n = lane & 15;   // column: query head inside the group (S^T, O^T), or row of the tile (A operand)
   const int G = p.group;
   const int Hkv = p.num_kv_heads;
 
+  // the table holds plain integers: say explicitly that they are global-memory addresses, otherwise
+  // the loads become flat loads that also count on the LDS wait counter and defeat the prefetch
+  typedef const __attribute__((address_space(1))) char *gptr;
+  typedef const __attribute__((address_space(1))) u32x4 *gvec;
   const int64_t slot = p.slot_ids[b];
-  const char *k_base = reinterpret_cast<const char *>(p.k_ptrs[slot]);
-  const char *v_base = reinterpret_cast<const char *>(p.v_ptrs[slot]);
-  constexpr int EB = FP8 ? 1 : 2;
-  const int64_t row_stride = (int64_t)Hkv * kD * EB;  // bytes between consecutive tokens
-  k_base += (int64_t)kvh * kD * EB;
-  v_base += (int64_t)kvh * kD * EB;
+  const uint32_t row_stride = (uint32_t)Hkv * kRowBytes;  // bytes between consecutive tokens
+  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kRowBytes;
+  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kRowBytes;
 
   // B operand of S^T = K.Q^T: lane (n, g) holds q[head n][32*ks + 8*g .. +8], zero for padded heads
   bf16x8 qop[4];
@@ -108,13 +157,17 @@ __global__ void __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnPa
     const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * kD;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
+#ifdef VTKV_DBG_NO_Q
+      u32x4 raw = {1u, 2u, 3u, (unsigned)lane};
+#else
       u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + ks * 32 + g * 8);
+#endif
       if (n >= G) raw = (u32x4){0, 0, 0, 0};
       qop[ks] = __builtin_bit_cast(bf16x8, raw);
     }
   }
-  const float slope_log2 =
-      (p.alibi_slopes != nullptr && n < G) ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
+  float slope_log2 = 0.f;
+  if (ALIBI) slope_log2 = n < G ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
 
   f32x4 acc[8];
 #pragma unroll
@@ -123,107 +176,178 @@ __global__ void __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnPa
   float l_run = 0.f;        // this lane's share of the running sum
 
   char *v_tile = smem + wave * (kTile * kRowBytes);
-  const int last_row = seq_len - 1;
 
-  // global -> register loads of one 16-row tile.
-  //   K: lane (n, g) takes row t0+n, bytes [64*ks + 16*g, +16): exactly its MFMA A operand.
-  //   V: lane l takes row t0 + 4*j + (l>>4), piece16 (l & 15): four full rows per load instruction.
-  // Rows past the end of the sequence are redirected to the last valid row (their logits are
-  // masked below) so no lane ever reads beyond the mapped part of the range.
-  u32x4 kreg[4], vreg[4];
-  auto load_tile = [&](int t0, u32x4 *kr, u32x4 *vr) {
-    const int krow = min(t0 + n, last_row);
-    const char *kp = k_base + (int64_t)krow * row_stride + g * 16;
+  // The partition's 16-row tiles are dealt round-robin to the four waves: this wave owns tiles
+  // wave, wave+4, ...  Only the last tile of a sequence can be ragged; its missing rows are redirected
+  // to the last valid row (their logits are masked) so no lane reads past the mapped part of a range.
+  const int n_tiles = (part_end - part_start + kTile - 1) / kTile;
+  const int my_tiles = (n_tiles - wave + kWaves - 1) / kWaves;
+  const int valid_last = part_end - (part_start + (n_tiles - 1) * kTile);  // rows in the last tile, 1..16
+  // per-lane byte offsets inside a tile: K lane (n, g) takes row n, bytes [16g, +16) of each 64-byte
+  // quarter (exactly its MFMA A operand); V lane takes row 4j+g, piece n: four full rows per load.
+  const uint32_t k_off = (uint32_t)n * row_stride + g * 16;
+  const uint32_t k_off_last = (uint32_t)min(n, valid_last - 1) * row_stride + g * 16;
+  uint32_t v_off[4], v_off_last[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) kr[ks] = *reinterpret_cast<const u32x4 *>(kp + ks * 64);
+  for (int j = 0; j < 4; ++j) {
+    v_off[j] = (uint32_t)(4 * j + g) * row_stride + n * 16;
+    v_off_last[j] = (uint32_t)min(4 * j + g, valid_last - 1) * row_stride + n * 16;
+  }
+
+  // Loads of the i-th tile of this wave.  Always issued, never predicated, so the wait counters the
+  // compiler derives are exact; past the wave's last tile the last tile is simply loaded again
+  // (it hits in cache and is not consumed).
+  auto load_k = [&](int i, u32x4 *kr) {
+    const int tile = wave + kWaves * min(i, my_tiles - 1);
+    const bool last = tile == n_tiles - 1;
+    gptr kp = k_base + (int64_t)(part_start + tile * kTile) * row_stride + (last ? k_off_last : k_off);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int vrow = min(t0 + 4 * j + g, last_row);
-      vr[j] = *reinterpret_cast<const u32x4 *>(v_base + (int64_t)vrow * row_stride + n * 16);
-    }
+    for (int ks = 0; ks < 4; ++ks) kr[ks] = *(gvec)(kp + ks * 64);
+  };
+  auto load_v = [&](int i, u32x4 *vr) {
+    const int tile = wave + kWaves * min(i, my_tiles - 1);
+    const bool last = tile == n_tiles - 1;
+    const int64_t row0 = (int64_t)(part_start + tile * kTile) * row_stride;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) vr[j] = *(gvec)(v_base + row0 + (last ? v_off_last[j] : v_off[j]));
   };
 
-  int t0 = part_start + wave * kTile;
-  if (t0 < part_end) load_tile(t0, kreg, vreg);
-
-  for (; t0 < part_end; t0 += kWaves * kTile) {
-    // prefetch the wave's next tile while this one is consumed
-    u32x4 knext[4], vnext[4];
-    const int t_next = t0 + kWaves * kTile;
-    if (t_next < part_end) load_tile(t_next, knext, vnext);
-
+  // one 16-row tile: logits, online softmax update, P.V
+  auto consume = [&](int i, u32x4 *kreg, u32x4 *vreg) {
+#ifdef VTKV_ATTN_NOCOMPUTE
+    for (int j = 0; j < 4; ++j) { u32x4 t = kreg[j] ^ vreg[j]; acc[j][0] += __builtin_bit_cast(float, t[0] ^ t[1] ^ t[2] ^ t[3]); }
+    return;
+#endif
+    const int tile = wave + kWaves * i;
+    const int t0 = part_start + tile * kTile;
     // S^T[row, head] = sum_d K[row, d] q[head, d]
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks)
       s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kreg[ks]), qop[ks], s, 0, 0, 0);
+    if (kStages == 1) load_k(i + 1, kreg);  // the K registers are free again: refill them for the next tile
 
     // stage V for the transposing read
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(4 * j + g, n)) = vreg[j];
+    if (kStages == 1) load_v(i + 1, vreg);  // likewise the V registers once they are in LDS
 
     // logits in log2 units; lane owns rows t0 + 4*g + i of head n
     float x[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int t = t0 + 4 * g + i;
-      x[i] = s[i] * p.scale_log2 + slope_log2 * (float)(t - seq_len + 1);
-      if (t >= seq_len) x[i] = -INFINITY;
+    for (int r = 0; r < 4; ++r) {
+      x[r] = s[r] * p.scale_log2;
+      if (ALIBI) x[r] += slope_log2 * (float)(t0 + 4 * g + r - seq_len + 1);
     }
-    float tmax = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+    if (tile == n_tiles - 1 && valid_last < kTile) {  // wave-uniform: only a sequence's ragged last tile
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (4 * g + r >= valid_last) x[r] = -INFINITY;
+    }
+    const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
     const float m_new = fmaxf(m_run, tmax);
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
     m_run = m_new;
     float pr[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pr[i] = __builtin_amdgcn_exp2f(x[i] - m_new);
+    for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
     l_run = l_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+      for (int d = 0; d < 8; ++d) acc[d] *= alpha;
     }
-    // P^T as B operand (row 4g+i, head n), split into a bf16 head and a bf16 tail so that P.V keeps
-    // ~16 mantissa bits of P: the result then tracks an fp32-P reference, not just a bf16-P one.
+    // P^T as B operand, split into a bf16 head and a bf16 tail so that P.V keeps ~16 mantissa bits of
+    // P (the result then tracks an fp32-P reference, not just a bf16-P one).  Head and tail share one
+    // K=32 MFMA: reduction slot (g, j) of v_mfma_f32_16x16x32_bf16 stands for row 4g+j with the head of
+    // P for j < 4 and for row 4g+j-4 with the tail for j >= 4, so the B operand is [head(4), tail(4)]
+    // straight from this lane's four logits and the A operand is the lane's V^T quad twice.
     float plo[4];
-    u32x2 pb_hi = {pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3])};
+    u32x4 pb;
+    pb[0] = pack_bf16x2(pr[0], pr[1]);
+    pb[1] = pack_bf16x2(pr[2], pr[3]);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const unsigned hi_bits = (i & 1) ? (pb_hi[i >> 1] & 0xffff0000u) : (pb_hi[i >> 1] << 16);
-      plo[i] = pr[i] - __builtin_bit_cast(float, hi_bits);
+    for (int r = 0; r < 4; ++r) {
+      const unsigned hi_bits = (r & 1) ? (pb[r >> 1] & 0xffff0000u) : (pb[r >> 1] << 16);
+      plo[r] = pr[r] - __builtin_bit_cast(float, hi_bits);
     }
-    u32x2 pb_lo = {pack_bf16x2(plo[0], plo[1]), pack_bf16x2(plo[2], plo[3])};
-    const s16x4 pop_hi = __builtin_bit_cast(s16x4, pb_hi);
-    const s16x4 pop_lo = __builtin_bit_cast(s16x4, pb_lo);
+    pb[2] = pack_bf16x2(plo[0], plo[1]);
+    pb[3] = pack_bf16x2(plo[2], plo[3]);
+    const bf16x8 pop = __builtin_bit_cast(bf16x8, pb);
 
     // O^T[d, head] += sum_row V[row, d] P[row, head], 16 d per MFMA.  LDS operations of one wave
     // execute in order, so the fences only pin the compiler's ordering of tile writes and reads.
+    // The reads are issued four at a time ahead of the MFMAs that use them.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-#pragma unroll
-    for (int db = 0; db < 8; ++db) {
+    {
       const int row = 4 * g + (n >> 2);
-      const int off = row * kRowBytes + (((2 * db + ((n >> 1) & 1)) ^ ((row & 7) << 1)) << 4) + ((n & 1) << 3);
-      const s16x4 vop = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) s16x4 *)(v_tile + off));
-      acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop, pop_hi, acc[db], 0, 0, 0);
-      acc[db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop, pop_lo, acc[db], 0, 0, 0);
+      const int base = row * kRowBytes + ((n & 1) << 3);
+      const int swz = (row & 7) << 1;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        u32x4 vop[4];
+#pragma unroll
+        for (int d4 = 0; d4 < 4; ++d4) {
+          const int db = 4 * half + d4;
+          const int off = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
+          const s16x4 quad =
+              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(v_tile + off));
+          const u32x2 qd = __builtin_bit_cast(u32x2, quad);
+          vop[d4] = (u32x4){qd[0], qd[1], qd[0], qd[1]};
+        }
+#pragma unroll
+        for (int d4 = 0; d4 < 4; ++d4)
+          acc[4 * half + d4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[d4]), pop,
+                                                                       acc[4 * half + d4], 0, 0, 0);
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
 
-    if (t_next < part_end) {
+  // A ring of kStages register tiles per wave: while one tile is consumed the loads of the wave's next
+  // kStages-1 tiles are in flight.  The steady-state path has no join after a load, only exits.
+  if (my_tiles > 0) {
+    u32x4 kbuf[kStages][4], vbuf[kStages][4];
+    if constexpr (kStages == 1) {
+      // one register tile per wave, refilled inside consume() as soon as its contents have been used:
+      // the loads of tile i+1 fly during the softmax and P.V of tile i at no extra register cost
+      load_k(0, kbuf[0]);
+      load_v(0, vbuf[0]);
+      for (int i = 0; i < my_tiles; ++i) consume(i, kbuf[0], vbuf[0]);
+    } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        kreg[j] = knext[j];
-        vreg[j] = vnext[j];
+      for (int st = 0; st < kStages - 1; ++st) {
+        load_k(st, kbuf[st]);
+        load_v(st, vbuf[st]);
       }
+      int i = 0;
+#define VTKV_STAGE(ST)                                                           \
+  {                                                                              \
+    load_k(i + kStages - 1, kbuf[((ST) + kStages - 1) % kStages]);               \
+    load_v(i + kStages - 1, vbuf[((ST) + kStages - 1) % kStages]);               \
+    consume(i, kbuf[(ST)], vbuf[(ST)]);                                          \
+    if (++i >= my_tiles) break;                                                  \
+  }
+      for (;;) {
+        VTKV_STAGE(0)
+        if constexpr (kStages > 1) VTKV_STAGE(1)
+        if constexpr (kStages > 2) VTKV_STAGE(2)
+        if constexpr (kStages > 3) VTKV_STAGE(3)
+      }
+#undef VTKV_STAGE
     }
   }
 
+#ifdef VTKV_DBG_SKIP_EPILOGUE
+  {
+    float t = l_run + m_run;
+    for (int d = 0; d < 8; ++d) t += acc[d][0] + acc[d][1] + acc[d][2] + acc[d][3];
+    if (t == 1.2345f) p.part_max[0] = t;
+  }
+  return;
+#endif
   // ---- merge the four waves.  l_run is still split over the four row groups of a lane column.
-  l_run += __shfl_xor(l_run, 16);
-  l_run += __shfl_xor(l_run, 32);
+  l_run = sum_over_row_groups(l_run);
   __syncthreads();  // every wave is done with its V tile: smem is free for the merge
   float *sm_m = reinterpret_cast<float *>(smem + kWaves * kTile * kRowBytes);  // [4][16]
   float *sm_l = sm_m + kWaves * 16;                                               // [4][16]
@@ -300,9 +424,11 @@ struct KernelTimer {
 };
 KernelTimer g_timer;
 
+// 512 rows per workgroup (the reference's PARTITION_SIZE, csrc/attention/attention_kernels.cu:37):
+// measured best on MI355X between per-workgroup fixed cost and balance across the 256 CUs.
 int default_part_tokens(int max_seq_len) {
   (void)max_seq_len;
-  return 256;
+  return 512;
 }
 
 }  // namespace
@@ -334,6 +460,9 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0,
                "q rows must be 16-byte aligned and at least num_heads*head_size apart");
   VTKV_REQUIRE(max_seq_len > 0, "max_seq_len must be > 0");
+  // the kernel addresses rows of a range with 32-bit byte offsets
+  VTKV_REQUIRE((int64_t)max_seq_len * num_kv_heads * head_size * 2 < (1ll << 31),
+               "a sequence range of %d rows exceeds 2 GiB", max_seq_len);
   if (num_seqs == 0) return VTKV_OK;
   const int pt = partition_tokens > 0 ? partition_tokens : default_part_tokens(max_seq_len);
   VTKV_REQUIRE(pt % (kWaves * kTile) == 0, "partition_tokens must be a multiple of %d", kWaves * kTile);
@@ -373,8 +502,12 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   hipStream_t st = (hipStream_t)stream;
   const bool timed = g_timer.on;
   if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[0], st));
-  hipLaunchKernelGGL(decode_attn_partial_kernel<false>, dim3(num_kv_heads, (unsigned)parts, num_seqs),
-                     dim3(kWaves * 64), 0, st, p);
+  if (alibi_slopes)
+    hipLaunchKernelGGL(decode_attn_partial_kernel<true>, dim3(num_kv_heads, (unsigned)parts, num_seqs),
+                       dim3(kWaves * 64), 0, st, p);
+  else
+    hipLaunchKernelGGL(decode_attn_partial_kernel<false>, dim3(num_kv_heads, (unsigned)parts, num_seqs),
+                       dim3(kWaves * 64), 0, st, p);
   if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[1], st));
   hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
   if (timed) {
