@@ -33,6 +33,9 @@ CONFIGS = {
     # configs[2]: long-context split-K decode
     "c3": dict(name="long-context-decode-bf16 B=4 Hq=32 Hkv=8 D=128 ctx~U[32768,131072]", batch=4, hq=32, hkv=8,
                d=128, lo=32768, hi=131072, seed=1002, kv="bf16"),
+    # configs[3]: fp8-e4m3 KV at the Llama-3-70B per-layer shape
+    "c4": dict(name="llama3-70b-layer-decode-fp8kv B=128 Hq=64 Hkv=8 D=128 ctx~U[1024,8192]", batch=128, hq=64,
+               hkv=8, d=128, lo=1024, hi=8192, seed=1003, kv="fp8"),
     # configs[4] without its swap events: 256 sequences
     "c5": dict(name="growth-bf16 B=256 Hq=32 Hkv=8 D=128 ctx~U[256,2048]", batch=256, hq=32, hkv=8, d=128, lo=256,
                hi=2048, seed=1004, kv="bf16"),
@@ -67,21 +70,31 @@ def main() -> int:
     gen = torch.Generator().manual_seed(cfg["seed"])
     ctx0 = torch.randint(cfg["lo"], cfg["hi"] + 1, (B,), generator=gen).tolist()
     total_steps = 2 * (K + W) + 4  # timed pass + kernel-timing pass, each with warm-up
-    row = Hkv * D * 2
+    fp8 = cfg["kv"] == "fp8"
+    eb = 1 if fp8 else 2            # bytes per KV element
+    kv_dtype = "fp8" if fp8 else "auto"
+    row = Hkv * D * eb
     max_tokens = max(ctx0) + total_steps + 1
     chunks_per_range = (max_tokens * row + (2 << 20) - 1) // (2 << 20)
     vmm.init_physical_handle(2 * B * chunks_per_range + 16, 0)
-    engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.bfloat16, max_num_seqs=B,
+    engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.uint8 if fp8 else torch.bfloat16,
+                         max_num_seqs=B,
                          max_num_batched_tokens=max_tokens, swap_space_bytes=1 << 30)
     segs = engine.vmm_kvcache_segment
 
     # ---- resident synthetic KV: N(0,1) -> bf16, written straight into the mapped ranges
     ggen = torch.Generator(device=dev).manual_seed(cfg["seed"])
+    # fp8: one scale per tensor; N(0,1) over ~1e8 draws peaks near 5.7, use amax = 6 -> scale = 6/448
+    k_scale = v_scale = 6.0 / 448.0 if fp8 else 1.0
     for b in range(B):
         nbytes = ctx0[b] * row
         segs[b].expandMultiSegment((nbytes + (2 << 20) - 1) // (2 << 20))
         for base in (segs[b].getKeyDevicePtr(0), segs[b].getValueDevicePtr(0)):
             t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            if fp8:
+                codes = torch.empty(t.shape, dtype=torch.uint8, device=dev)
+                ops.convert_fp8(codes, t, k_scale)
+                t = codes
             ops.swap_ranges([t.data_ptr()], [base], [nbytes], "d2d")
             torch.cuda.synchronize()
         segs[b].set_used_size(nbytes)
@@ -115,17 +128,17 @@ def main() -> int:
         max_len = max(lens)
         # 2. append the new token's K/V rows
         ops.reshape_and_cache(new_k, new_v, engine.k_cache_ptr[0], engine.v_cache_ptr[0], slot_m_t, slot_t, None,
-                              None, 1, Hkv, D)
+                              None, 1, Hkv, D, kv_dtype, k_scale, v_scale)
         # 3. decode attention over the whole context
         ops.paged_attention_v1(out, q.view(B, Hq, D), engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hkv, scale,
-                               lens_t, 1, max_len, None, "auto", 1.0, slot_t,
+                               lens_t, 1, max_len, None, kv_dtype, k_scale, slot_t, v_scale=v_scale,
                                partition_tokens=args.partition_tokens)
         state["step"] = i + 1
         return sum(lens)
 
     def attn_bytes(sum_ctx: int) -> int:
         # K+V rows of every context token, plus q in and out out
-        return sum_ctx * 2 * Hkv * D * 2 + B * Hq * D * 2 + B * Hq * D * 2
+        return sum_ctx * 2 * Hkv * D * eb + B * Hq * D * 2 + B * Hq * D * 2
 
     # ---- timed region: exactly K steps, synchronised on both sides
     for _ in range(W):
@@ -134,7 +147,7 @@ def main() -> int:
     t0 = time.perf_counter()
     bytes_total = 0
     for _ in range(K):
-        bytes_total += attn_bytes(step()) + B * 2 * Hkv * D * (2 + 2)  # + reshape_and_cache in/out
+        bytes_total += attn_bytes(step()) + B * 2 * Hkv * D * (2 + eb)  # + reshape_and_cache in/out
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / K * 1e3
@@ -178,7 +191,7 @@ def main() -> int:
         "metric": "decode-attn HBM GB/s (% peak) + tokens/s @ Llama-3-8B shape B=64; swap GB/s",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "bf16 (fp8-e4m3 KV)" if fp8 else "bf16", "data": "synthetic",
         "config": {"workload": cfg["name"], "layers": 1, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
                    "mean_ctx": round(float(np.mean(state["lens"])), 1)},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
@@ -187,7 +200,7 @@ def main() -> int:
         "roofline": roofline,
     }
 
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not fp8:
         result["cpu_baseline"] = cpu_baseline(cfg, engine, state["lens"], q, scale, args.cpu_seconds)
 
     print(json.dumps(result))

@@ -123,7 +123,21 @@ __device__ __forceinline__ float sum_over_row_groups(float x) {
   return a + b;
 }
 
-template <bool ALIBI>
+// eight e4m3fn codes (two dwords) -> eight bf16 values; exact, every e4m3fn value is a bf16 value
+__device__ __forceinline__ u32x4 fp8x8_to_bf16x8(unsigned lo, unsigned hi) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  u32x4 r;
+  r[0] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false));
+  r[1] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true));
+  r[2] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false));
+  r[3] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true));
+  return r;
+}
+
+// FP8: K and V rows hold one e4m3fn code per element (128 bytes per head row).  They are widened to
+// bf16 in registers (K) or on the way into the LDS tile (V); the per-tensor scales are folded into the
+// logit scale (K) and into the final normalisation (V), so dequantisation costs no multiply per element.
+template <bool ALIBI, bool FP8>
 __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnParams p) {
   // wave-private V tiles (4 KiB each); reused after the main loop for the cross-wave merge
   __shared__ __attribute__((aligned(16))) char smem[kWaves * kTile * kRowBytes + 1024];
@@ -147,11 +161,15 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_p
   typedef const __attribute__((address_space(1))) char *gptr;
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
   const int64_t slot = p.slot_ids[b];
-  const uint32_t row_stride = (uint32_t)Hkv * kRowBytes;  // bytes between consecutive tokens
-  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kRowBytes;
-  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kRowBytes;
+  constexpr int kKvRowBytes = FP8 ? kD : kRowBytes;  // bytes of one head row in global memory
+  constexpr int kLoads = FP8 ? 2 : 4;                // 16-byte loads per lane for a K (or V) tile
+  const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;  // bytes between consecutive tokens
+  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
+  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
 
-  // B operand of S^T = K.Q^T: lane (n, g) holds q[head n][32*ks + 8*g .. +8], zero for padded heads
+  // B operand of S^T = K.Q^T: for MFMA step ks lane (n, g) holds the eight q[head n][d] whose K elements
+  // the lane's 16-byte K loads deliver: d = 32*ks + 8*g + j for bf16 rows; for fp8 rows one load carries
+  // 16 elements, so steps 2c and 2c+1 take d = 64*c + 16*g + j and + 8.  Zero for padded heads.
   bf16x8 qop[4];
   {
     const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * kD;
@@ -160,7 +178,8 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_p
 #ifdef VTKV_DBG_NO_Q
       u32x4 raw = {1u, 2u, 3u, (unsigned)lane};
 #else
-      u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + ks * 32 + g * 8);
+      const int d0 = FP8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
+      u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + d0);
 #endif
       if (n >= G) raw = (u32x4){0, 0, 0, 0};
       qop[ks] = __builtin_bit_cast(bf16x8, raw);
@@ -187,11 +206,14 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_p
   // quarter (exactly its MFMA A operand); V lane takes row 4j+g, piece n: four full rows per load.
   const uint32_t k_off = (uint32_t)n * row_stride + g * 16;
   const uint32_t k_off_last = (uint32_t)min(n, valid_last - 1) * row_stride + g * 16;
-  uint32_t v_off[4], v_off_last[4];
+  // (fp8 rows are 128 bytes: a V load then covers eight rows, lane l takes row 8j + l/8, piece l%8)
+  uint32_t v_off[kLoads], v_off_last[kLoads];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    v_off[j] = (uint32_t)(4 * j + g) * row_stride + n * 16;
-    v_off_last[j] = (uint32_t)min(4 * j + g, valid_last - 1) * row_stride + n * 16;
+  for (int j = 0; j < kLoads; ++j) {
+    const int row = FP8 ? 8 * j + (lane >> 3) : 4 * j + g;
+    const int col = FP8 ? (lane & 7) * 16 : n * 16;
+    v_off[j] = (uint32_t)row * row_stride + col;
+    v_off_last[j] = (uint32_t)min(row, valid_last - 1) * row_stride + col;
   }
 
   // Loads of the i-th tile of this wave.  Always issued, never predicated, so the wait counters the
@@ -202,35 +224,42 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_p
     const bool last = tile == n_tiles - 1;
     gptr kp = k_base + (int64_t)(part_start + tile * kTile) * row_stride + (last ? k_off_last : k_off);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) kr[ks] = *(gvec)(kp + ks * 64);
+    for (int ks = 0; ks < kLoads; ++ks) kr[ks] = *(gvec)(kp + ks * 64);
   };
   auto load_v = [&](int i, u32x4 *vr) {
     const int tile = wave + kWaves * min(i, my_tiles - 1);
     const bool last = tile == n_tiles - 1;
     const int64_t row0 = (int64_t)(part_start + tile * kTile) * row_stride;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) vr[j] = *(gvec)(v_base + row0 + (last ? v_off_last[j] : v_off[j]));
+    for (int j = 0; j < kLoads; ++j) vr[j] = *(gvec)(v_base + row0 + (last ? v_off_last[j] : v_off[j]));
   };
 
   // one 16-row tile: logits, online softmax update, P.V
   auto consume = [&](int i, u32x4 *kreg, u32x4 *vreg) {
-#ifdef VTKV_ATTN_NOCOMPUTE
-    for (int j = 0; j < 4; ++j) { u32x4 t = kreg[j] ^ vreg[j]; acc[j][0] += __builtin_bit_cast(float, t[0] ^ t[1] ^ t[2] ^ t[3]); }
-    return;
-#endif
     const int tile = wave + kWaves * i;
     const int t0 = part_start + tile * kTile;
     // S^T[row, head] = sum_d K[row, d] q[head, d]
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kreg[ks]), qop[ks], s, 0, 0, 0);
+    for (int ks = 0; ks < 4; ++ks) {
+      const u32x4 kop = FP8 ? fp8x8_to_bf16x8(kreg[ks >> 1][2 * (ks & 1)], kreg[ks >> 1][2 * (ks & 1) + 1]) : kreg[ks];
+      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kop), qop[ks], s, 0, 0, 0);
+    }
     if (kStages == 1) load_k(i + 1, kreg);  // the K registers are free again: refill them for the next tile
 
-    // stage V for the transposing read
+    // stage V (as bf16) for the transposing read
+    if constexpr (FP8) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(4 * j + g, n)) = vreg[j];
+      for (int j = 0; j < 2; ++j) {
+        const int row = 8 * j + (lane >> 3), piece = 2 * (lane & 7);
+        *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece)) = fp8x8_to_bf16x8(vreg[j][0], vreg[j][1]);
+        *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece + 1)) = fp8x8_to_bf16x8(vreg[j][2], vreg[j][3]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(4 * j + g, n)) = vreg[j];
+    }
     if (kStages == 1) load_v(i + 1, vreg);  // likewise the V registers once they are in LDS
 
     // logits in log2 units; lane owns rows t0 + 4*g + i of head n
@@ -454,14 +483,16 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
   VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
   VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
-  VTKV_REQUIRE(kv_dtype == VTKV_BF16, "kv_dtype must be BF16");
+  VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be BF16 or FP8_E4M3");
+  if (kv_dtype == VTKV_FP8_E4M3)
+    VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
   const int group = num_heads / num_kv_heads;
   VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0,
                "q rows must be 16-byte aligned and at least num_heads*head_size apart");
   VTKV_REQUIRE(max_seq_len > 0, "max_seq_len must be > 0");
   // the kernel addresses rows of a range with 32-bit byte offsets
-  VTKV_REQUIRE((int64_t)max_seq_len * num_kv_heads * head_size * 2 < (1ll << 31),
+  VTKV_REQUIRE((int64_t)max_seq_len * num_kv_heads * head_size * vtkv::elem_bytes(kv_dtype) < (1ll << 31),
                "a sequence range of %d rows exceeds 2 GiB", max_seq_len);
   if (num_seqs == 0) return VTKV_OK;
   const int pt = partition_tokens > 0 ? partition_tokens : default_part_tokens(max_seq_len);
@@ -474,7 +505,6 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
     return vtkv::fail(VTKV_ENOMEM, "workspace of %lld bytes is smaller than the %lld needed",
                       (long long)workspace_bytes, (long long)need);
   VTKV_REQUIRE((uintptr_t)workspace % 16 == 0, "workspace must be 16-byte aligned");
-  (void)k_scale;
 
   AttnParams p;
   p.q = (const uint16_t *)q;
@@ -495,19 +525,23 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   p.group = group;
   p.part_tokens = pt;
   p.max_parts = (int)parts;
-  p.scale_log2 = scale * kLog2e;
-  p.v_scale = 1.f;
-  (void)v_scale;
+  // x = code * scale: the K scale multiplies every logit, the V scale the whole output
+  p.scale_log2 = scale * kLog2e * (kv_dtype == VTKV_FP8_E4M3 ? k_scale : 1.f);
+  p.v_scale = kv_dtype == VTKV_FP8_E4M3 ? v_scale : 1.f;
 
   hipStream_t st = (hipStream_t)stream;
   const bool timed = g_timer.on;
   if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[0], st));
-  if (alibi_slopes)
-    hipLaunchKernelGGL(decode_attn_partial_kernel<true>, dim3(num_kv_heads, (unsigned)parts, num_seqs),
-                       dim3(kWaves * 64), 0, st, p);
+  const dim3 grid(num_kv_heads, (unsigned)parts, num_seqs), block(kWaves * 64);
+  const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
+  if (alibi_slopes && fp8)
+    hipLaunchKernelGGL((decode_attn_partial_kernel<true, true>), grid, block, 0, st, p);
+  else if (alibi_slopes)
+    hipLaunchKernelGGL((decode_attn_partial_kernel<true, false>), grid, block, 0, st, p);
+  else if (fp8)
+    hipLaunchKernelGGL((decode_attn_partial_kernel<false, true>), grid, block, 0, st, p);
   else
-    hipLaunchKernelGGL(decode_attn_partial_kernel<false>, dim3(num_kv_heads, (unsigned)parts, num_seqs),
-                       dim3(kWaves * 64), 0, st, p);
+    hipLaunchKernelGGL((decode_attn_partial_kernel<false, false>), grid, block, 0, st, p);
   if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[1], st));
   hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
   if (timed) {

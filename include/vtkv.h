@@ -200,7 +200,7 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  *   alibi_slopes device float[num_heads] or NULL
  *   kv_dtype     q_dtype, or VTKV_FP8_E4M3 with k_scale / v_scale (x = code * scale)
  *   workspace    device scratch of at least vtkv_decode_attention_workspace_bytes(...) bytes
- * Supported: q_dtype VTKV_BF16, head_size 128, num_heads/num_kv_heads in 1..16. */
+ * Supported: q_dtype VTKV_BF16, kv_dtype VTKV_BF16 or VTKV_FP8_E4M3, head_size 128, num_heads/num_kv_heads in 1..16. */
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                           const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,

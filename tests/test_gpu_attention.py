@@ -115,3 +115,11 @@ def test_single_token_returns_value_row(gpu_pool):
 
     got, want = run_case(gpu_pool, 11, [1, 1, 1], 32, 8)
     assert np.array_equal(got, want)  # fp32 result equals the (bf16-valued) V row exactly
+
+
+def test_config3_long_context_split_k(gpu_pool):
+    """BASELINE config 3 at reduced batch: contexts of 32k-131k rows, hundreds of partitions per
+    sequence, so the cross-partition log-sum-exp merge carries the result."""
+    rng = np.random.default_rng(1002)
+    lens = [int(rng.integers(32768, 131073)), 131072, 40000]
+    run_case(gpu_pool, 1002, lens, 32, 8)
