@@ -107,6 +107,15 @@ def main() -> int:
     scale = float(D) ** -0.5
     kv_size = row
 
+    # A plain copy of known size (256 MiB read, 256 MiB written: 1024 blocks of 128 KiB for K and for V)
+    # outside the timed region: under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its `copy_blocks_kernel`
+    # dispatch calibrates the counters.
+    cal = [torch.zeros(2048, 128 << 10, dtype=torch.uint8, device=dev) for _ in range(2)]
+    pairs = torch.stack([torch.arange(1024), torch.arange(1024) + 1024], dim=1).to(device=dev, dtype=torch.int64)
+    ops.copy_blocks([cal[0]], [cal[1]], pairs)
+    torch.cuda.synchronize()
+    del cal, pairs
+
     # pinned staging rows, one per step, so an async upload never races the next step's host writes
     stage_m = torch.empty(total_steps, B, dtype=torch.int64).pin_memory()
     stage_l = torch.empty(total_steps, B, dtype=torch.int32).pin_memory()
