@@ -3,39 +3,48 @@
 // One query token per sequence attends to the first seq_len rows of that sequence's K and V
 // ranges, both token-major [T, Hkv, D].  The work is bound by HBM reads of K and V
 // (2*Hkv*D*e bytes per token, 2*G/e flop per byte with G = Hq/Hkv), so the design goal is to read
-// every K/V byte exactly once and keep many 16-byte loads in flight:
+// every K/V byte exactly once, keep many 16-byte loads in flight on every CU for the whole launch,
+// and spend as little time as possible outside the streaming loop:
 //
-//  * split-K: grid (Hkv, partitions, sequences); a workgroup of four wave64 handles one kv head
-//    over one partition of `part_tokens` rows and ALL G query heads of that kv head's group
-//    share the pass (the reference launches one block per query head and re-reads KV G times,
-//    csrc/attention/attention_kernels.cu:625 grid(num_heads, num_seqs, 1)).
-//  * inside a wave a tile is 16 rows.  S^T = K_tile . Q^T runs on v_mfma_f32_16x16x32_bf16 with the
-//    G query heads padded to the 16 columns: K rows are the A operand, and a lane's 16-byte
-//    global load of one row piece already IS its A operand, so K never touches LDS.
+//  * work is counted in tiles of 16 rows of one kv head.  All tiles of the batch form one sequence
+//    ordered (sequence, kv head, tile); it is cut into gridDim.x equal contiguous spans, one per
+//    workgroup, whatever the sequence lengths are ("stream-K" split).  Every CU therefore gets the
+//    same number of bytes, a workgroup streams a long contiguous run of rows, and the fixed cost of
+//    starting and finishing a (sequence, kv head) segment is paid once or twice per workgroup instead
+//    of once per 512 rows.  The grid is the number of workgroups the device holds at once.
+//  * ALL G query heads of a kv head's group share the pass over its rows (the reference launches one
+//    block per query head and re-reads KV G times, csrc/attention/attention_kernels.cu:625).
+//  * inside a workgroup the tiles of a segment are dealt round-robin to four wave64.
+//    S^T = K_tile . Q^T runs on v_mfma_f32_16x16x32_bf16 with the G query heads padded to the 16
+//    columns: K rows are the A operand, and a lane's 16-byte global load of one row piece already IS
+//    its A operand, so K never touches LDS.
 //  * softmax statistics stay in registers: in the MFMA C layout a lane owns one head column and four
 //    rows, so a head's max/sum over the tile is an in-lane reduction plus two cross-row-group
 //    exchanges; an online (running-max) rescale keeps one pass.
 //  * O^T += V_tile^T . P^T runs on v_mfma_f32_16x16x32_bf16.  P^T is the C layout of S^T as is.  V is
 //    row-major but the A operand needs four rows per lane, so V tiles go through a wave-private,
 //    XOR-swizzled LDS tile and come back with ds_read_b64_tr_b16 (the transposing LDS read).
-//  * each wave keeps (m, l, O) for its rows; the four waves merge through LDS and the workgroup
-//    writes one normalised partial (max, sum, O/sum) per head; a second small kernel merges the
-//    partitions of each sequence with the log-sum-exp rule of the reference's split kernel
-//    (csrc/attention/attention_kernels.cu:486-583; CPU twin csrc/cpu/attention.cpp:583-644).
+//  * each wave keeps (m, l, O) for its rows; at the end of a segment the four waves merge through LDS
+//    and the workgroup writes one normalised partial (max, sum, O/sum) per head into slot
+//    (workgroup + segment id), which is unique because both only ever increase along the tile order.
+//    A second small kernel merges the few partials of each (sequence, head) with the log-sum-exp rule
+//    of the reference's split kernel (csrc/attention/attention_kernels.cu:486-583; CPU twin
+//    csrc/cpu/attention.cpp:583-644).
 //
 // Numerics: bf16 q.k products accumulated in fp32 and softmax in fp32 as in the reference
 // (csrc/attention/attention_kernels.cu:226-283).  The reference CUDA kernel rounds P to bf16
 // before P.V (:326-327) while its CPU twin keeps P in fp32 (csrc/cpu/attention.cpp:197-211); here P
-// enters the MFMA as a bf16 head plus a bf16 tail (two MFMAs), which is as good as fp32 P for the
-// tolerance in force.  fp32 accumulation, output rounded to bf16 once.  No epsilon is added to the softmax denominator (the
-// CPU twin has none, csrc/cpu/attention.cpp:43-67).
+// enters the MFMA as a bf16 head plus a bf16 tail, which is as good as fp32 P for the tolerance in
+// force.  fp32 accumulation, output rounded to bf16 once.  No epsilon is added to the softmax
+// denominator (the CPU twin has none, csrc/cpu/attention.cpp:43-67).
 #include <algorithm>
+#include <mutex>
 
 #include "vtkv_common.h"
 #ifndef VTKV_ATTN_STAGES
 #define VTKV_ATTN_STAGES 2
 #endif
-// register budget of the split-K kernel: N waves per SIMD (it fits 128 VGPRs with one register tile)
+// register budget of the streaming kernel: N waves per SIMD (it fits 128 VGPRs with one register tile)
 #ifdef VTKV_ATTN_WAVES_PER_EU
 #define VTKV_ATTN_OCCUPANCY __attribute__((amdgpu_waves_per_eu(VTKV_ATTN_WAVES_PER_EU)))
 #else
@@ -55,8 +64,12 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kD = 128;            // head size
 constexpr int kTile = 16;          // rows per MFMA tile
 constexpr int kWaves = 4;          // waves per workgroup
+constexpr int kThreads = kWaves * 64;
 constexpr int kStages = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
 constexpr int kRowBytes = kD * 2;  // bf16 row of one head
+constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
+constexpr int kMinSpan = 4;        // a workgroup takes at least one tile per wave
+constexpr int kDefaultMaxGrid = 4096;  // upper bound of the resident-workgroup grid, sizes the scratch
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct AttnParams {
@@ -64,12 +77,17 @@ struct AttnParams {
   const int64_t *k_ptrs, *v_ptrs, *slot_ids;
   const int32_t *seq_lens;
   const float *alibi_slopes;
-  float *part_max, *part_sum, *part_out;  // [B,Hq,P], [B,Hq,P], [B,Hq,P,D]
-  void *out;                              // [B,Hq,D] bf16, or fp32 when out_f32
+  // scratch: partial results per slot, and the prefix sums of per-sequence tile counts
+  float *part_out;  // [slots][G][D]
+  float *part_max;  // [slots][G]   (log2 units)
+  float *part_sum;  // [slots][G]
+  int32_t *cum_tiles;  // [num_seqs + 1]
+  void *out;           // [B,Hq,D] bf16, or fp32 when out_f32
   int out_f32;
   int64_t q_stride;
-  int num_heads, num_kv_heads, group;  // Hq, Hkv, G
-  int part_tokens, max_parts;
+  int num_seqs, num_heads, num_kv_heads, group;  // B, Hq, Hkv, G
+  int span_tiles;   // tiles per workgroup; 0 = all tiles / gridDim.x
+  int grid;         // workgroups of the streaming kernel
   float scale_log2;  // scale * log2(e) [* k_scale for fp8 K]
   float v_scale;
 };
@@ -88,10 +106,10 @@ __device__ __forceinline__ int v_lds_offset(int row, int piece16) {
   return row * kRowBytes + ((piece16 ^ ((row & 7) << 1)) << 4);
 }
 
-// max over the four row groups (lanes l, l^16, l^32, l^48) with the gfx950 lane-swap instructions:
-// v_permlane16_swap exchanges odd 16-lane rows of its first operand with even rows of its second,
-// v_permlane32_swap does the same for 32-lane halves, so swapping a value with itself and taking the
-// max of the two results folds rows pairwise.
+// max / sum over the four row groups (lanes l, l^16, l^32, l^48) with the gfx950 lane-swap
+// instructions: v_permlane16_swap exchanges odd 16-lane rows of its first operand with even rows of its
+// second, v_permlane32_swap does the same for 32-lane halves, so swapping a value with itself and
+// combining the two results folds rows pairwise.
 // (the two results are copied to scalars before the bit cast: a bit cast applied directly to an
 // element of the returned vector reads element 0 both times with this compiler)
 __device__ __forceinline__ void swap_rows16(float x, float &a, float &b) {
@@ -134,222 +152,287 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(unsigned lo, unsigned hi) {
   return r;
 }
 
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// Tiles per workgroup span, the same rule in both kernels.
+__device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
+  if (p.span_tiles > 0) return p.span_tiles;
+  return max((total_tiles + p.grid - 1) / p.grid, kMinSpan);
+}
+
 // FP8: K and V rows hold one e4m3fn code per element (128 bytes per head row).  They are widened to
 // bf16 in registers (K) or on the way into the LDS tile (V); the per-tensor scales are folded into the
 // logit scale (K) and into the final normalisation (V), so dequantisation costs no multiply per element.
 template <bool ALIBI, bool FP8>
-__global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_partial_kernel(AttnParams p) {
-  // wave-private V tiles (4 KiB each); reused after the main loop for the cross-wave merge
+__global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stream_kernel(AttnParams p) {
+  // wave-private V tiles (4 KiB each); reused at the end of a segment for the cross-wave merge
   __shared__ __attribute__((aligned(16))) char smem[kWaves * kTile * kRowBytes + 1024];
-
-  const int kvh = blockIdx.x, part = blockIdx.y, b = blockIdx.z;
-  const int seq_len = p.seq_lens[b];
-  const int part_start = part * p.part_tokens;
-  if (part_start >= seq_len) return;
-  const int part_end = min(seq_len, part_start + p.part_tokens);
+  __shared__ int s_cum[kMaxSeqs + 1];  // s_cum[b] = tiles (of one kv head) of sequences before b
+  __shared__ int s_wave_tot[kWaves];
 
   const int lane = threadIdx.x & 63;
   // everything that decides control flow and base addresses is kept wave-uniform (scalar registers)
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = uniform(threadIdx.x >> 6);
   const int g = lane >> 4;   // row group of the MFMA layouts
   const int n = lane & 15;   // column: query head inside the group (S^T, O^T), or row of the tile (A operand)
   const int G = p.group;
   const int Hkv = p.num_kv_heads;
+  const int B = p.num_seqs;
 
-  // the table holds plain integers: say explicitly that they are global-memory addresses, otherwise
-  // the loads become flat loads that also count on the LDS wait counter and defeat the prefetch
+  // ---- exclusive prefix sums of the per-sequence tile counts (every workgroup computes its own copy)
+  {
+    constexpr int kPer = kMaxSeqs / kThreads;
+    int local[kPer], sum = 0;
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      const int idx = threadIdx.x * kPer + k;
+      const int len = idx < B ? p.seq_lens[idx] : 0;
+      local[k] = sum;
+      sum += len > 0 ? (len + kTile - 1) / kTile : 0;
+    }
+    int incl = sum;  // inclusive scan over the wave
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int t = __shfl_up(incl, d);
+      if (lane >= d) incl += t;
+    }
+    if (lane == 63) s_wave_tot[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += s_wave_tot[w];
+    const int excl = base + incl - sum;
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      const int idx = threadIdx.x * kPer + k;
+      if (idx <= B) s_cum[idx] = excl + local[k];
+    }
+    if (threadIdx.x == 0) s_cum[B] = s_wave_tot[0] + s_wave_tot[1] + s_wave_tot[2] + s_wave_tot[3];
+    __syncthreads();
+  }
+  const int seq_tiles_total = uniform(s_cum[B]);
+  const int total_tiles = seq_tiles_total * Hkv;
+  if (blockIdx.x == 0)
+    for (int i = threadIdx.x; i <= B; i += kThreads) p.cum_tiles[i] = s_cum[i];
+
+  // ---- this workgroup's span [g_cur, g_end) of the global tile order
+  const int span = span_of(p, total_tiles);
+  int g_cur = blockIdx.x * span;
+  if (g_cur >= total_tiles) return;
+  const int g_end = min(total_tiles, g_cur + span);
+
+  // first sequence of the span: the last b with Hkv*cum[b] <= g_cur (sequences without rows own no tile)
+  int b;
+  {
+    int lo = 0, hi = B;  // invariant: Hkv*cum[lo] <= g_cur < Hkv*cum[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (uniform(s_cum[mid]) * Hkv <= g_cur) lo = mid; else hi = mid;
+    }
+    b = lo;
+  }
+  int nt_b = uniform(s_cum[b + 1]) - uniform(s_cum[b]);
+  int kvh = (g_cur - uniform(s_cum[b]) * Hkv) / nt_b;
+  int tile0 = g_cur - uniform(s_cum[b]) * Hkv - kvh * nt_b;
+
   typedef const __attribute__((address_space(1))) char *gptr;
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
-  const int64_t slot = p.slot_ids[b];
   constexpr int kKvRowBytes = FP8 ? kD : kRowBytes;  // bytes of one head row in global memory
   constexpr int kLoads = FP8 ? 2 : 4;                // 16-byte loads per lane for a K (or V) tile
   const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;  // bytes between consecutive tokens
-  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
-  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
-
-  // B operand of S^T = K.Q^T: for MFMA step ks lane (n, g) holds the eight q[head n][d] whose K elements
-  // the lane's 16-byte K loads deliver: d = 32*ks + 8*g + j for bf16 rows; for fp8 rows one load carries
-  // 16 elements, so steps 2c and 2c+1 take d = 64*c + 16*g + j and + 8.  Zero for padded heads.
-  bf16x8 qop[4];
-  {
-    const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * kD;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-#ifdef VTKV_DBG_NO_Q
-      u32x4 raw = {1u, 2u, 3u, (unsigned)lane};
-#else
-      const int d0 = FP8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
-      u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + d0);
-#endif
-      if (n >= G) raw = (u32x4){0, 0, 0, 0};
-      qop[ks] = __builtin_bit_cast(bf16x8, raw);
-    }
-  }
-  float slope_log2 = 0.f;
-  if (ALIBI) slope_log2 = n < G ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
-
-  f32x4 acc[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY;  // running max of scaled logits (log2 units) of head n
-  float l_run = 0.f;        // this lane's share of the running sum
-
   char *v_tile = smem + wave * (kTile * kRowBytes);
 
-  // The partition's 16-row tiles are dealt round-robin to the four waves: this wave owns tiles
-  // wave, wave+4, ...  Only the last tile of a sequence can be ragged; its missing rows are redirected
-  // to the last valid row (their logits are masked) so no lane reads past the mapped part of a range.
-  const int n_tiles = (part_end - part_start + kTile - 1) / kTile;
-  const int my_tiles = (n_tiles - wave + kWaves - 1) / kWaves;
-  const int valid_last = part_end - (part_start + (n_tiles - 1) * kTile);  // rows in the last tile, 1..16
-  // per-lane byte offsets inside a tile: K lane (n, g) takes row n, bytes [16g, +16) of each 64-byte
-  // quarter (exactly its MFMA A operand); V lane takes row 4j+g, piece n: four full rows per load.
-  const uint32_t k_off = (uint32_t)n * row_stride + g * 16;
-  const uint32_t k_off_last = (uint32_t)min(n, valid_last - 1) * row_stride + g * 16;
-  // (fp8 rows are 128 bytes: a V load then covers eight rows, lane l takes row 8j + l/8, piece l%8)
-  uint32_t v_off[kLoads], v_off_last[kLoads];
-#pragma unroll
-  for (int j = 0; j < kLoads; ++j) {
-    const int row = FP8 ? 8 * j + (lane >> 3) : 4 * j + g;
-    const int col = FP8 ? (lane & 7) * 16 : n * 16;
-    v_off[j] = (uint32_t)row * row_stride + col;
-    v_off_last[j] = (uint32_t)min(row, valid_last - 1) * row_stride + col;
-  }
+  // ---- one segment = the part of the span that lies in one (sequence, kv head)
+  while (g_cur < g_end) {
+    const int seg_tiles = min(g_end - g_cur, nt_b - tile0);
+    const int seq_len = p.seq_lens[b];
+    const int seg_start = tile0 * kTile;                               // first row of the segment
+    const int seg_end = min(seq_len, (tile0 + seg_tiles) * kTile);     // one past its last row
 
-  // Loads of the i-th tile of this wave.  Always issued, never predicated, so the wait counters the
-  // compiler derives are exact; past the wave's last tile the last tile is simply loaded again
-  // (it hits in cache and is not consumed).
-  auto load_k = [&](int i, u32x4 *kr) {
-    const int tile = wave + kWaves * min(i, my_tiles - 1);
-    const bool last = tile == n_tiles - 1;
-    gptr kp = k_base + (int64_t)(part_start + tile * kTile) * row_stride + (last ? k_off_last : k_off);
-#pragma unroll
-    for (int ks = 0; ks < kLoads; ++ks) kr[ks] = *(gvec)(kp + ks * 64);
-  };
-  auto load_v = [&](int i, u32x4 *vr) {
-    const int tile = wave + kWaves * min(i, my_tiles - 1);
-    const bool last = tile == n_tiles - 1;
-    const int64_t row0 = (int64_t)(part_start + tile * kTile) * row_stride;
-#pragma unroll
-    for (int j = 0; j < kLoads; ++j) vr[j] = *(gvec)(v_base + row0 + (last ? v_off_last[j] : v_off[j]));
-  };
+    // the tables hold plain integers: say explicitly that they are global-memory addresses, otherwise
+    // the loads become flat loads that also count on the LDS wait counter and defeat the prefetch
+    const int64_t slot = p.slot_ids[b];
+    gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
+    gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
 
-  // one 16-row tile: logits, online softmax update, P.V
-  auto consume = [&](int i, u32x4 *kreg, u32x4 *vreg) {
-    const int tile = wave + kWaves * i;
-    const int t0 = part_start + tile * kTile;
-    // S^T[row, head] = sum_d K[row, d] q[head, d]
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const u32x4 kop = FP8 ? fp8x8_to_bf16x8(kreg[ks >> 1][2 * (ks & 1)], kreg[ks >> 1][2 * (ks & 1) + 1]) : kreg[ks];
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kop), qop[ks], s, 0, 0, 0);
-    }
-    if (kStages == 1) load_k(i + 1, kreg);  // the K registers are free again: refill them for the next tile
-
-    // stage V (as bf16) for the transposing read
-    if constexpr (FP8) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int row = 8 * j + (lane >> 3), piece = 2 * (lane & 7);
-        *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece)) = fp8x8_to_bf16x8(vreg[j][0], vreg[j][1]);
-        *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece + 1)) = fp8x8_to_bf16x8(vreg[j][2], vreg[j][3]);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(4 * j + g, n)) = vreg[j];
-    }
-    if (kStages == 1) load_v(i + 1, vreg);  // likewise the V registers once they are in LDS
-
-    // logits in log2 units; lane owns rows t0 + 4*g + i of head n
-    float x[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      x[r] = s[r] * p.scale_log2;
-      if (ALIBI) x[r] += slope_log2 * (float)(t0 + 4 * g + r - seq_len + 1);
-    }
-    if (tile == n_tiles - 1 && valid_last < kTile) {  // wave-uniform: only a sequence's ragged last tile
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (4 * g + r >= valid_last) x[r] = -INFINITY;
-    }
-    const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
-    const float m_new = fmaxf(m_run, tmax);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
-    m_run = m_new;
-    float pr[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
-    l_run = l_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
-#pragma unroll
-      for (int d = 0; d < 8; ++d) acc[d] *= alpha;
-    }
-    // P^T as B operand, split into a bf16 head and a bf16 tail so that P.V keeps ~16 mantissa bits of
-    // P (the result then tracks an fp32-P reference, not just a bf16-P one).  Head and tail share one
-    // K=32 MFMA: reduction slot (g, j) of v_mfma_f32_16x16x32_bf16 stands for row 4g+j with the head of
-    // P for j < 4 and for row 4g+j-4 with the tail for j >= 4, so the B operand is [head(4), tail(4)]
-    // straight from this lane's four logits and the A operand is the lane's V^T quad twice.
-    float plo[4];
-    u32x4 pb;
-    pb[0] = pack_bf16x2(pr[0], pr[1]);
-    pb[1] = pack_bf16x2(pr[2], pr[3]);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const unsigned hi_bits = (r & 1) ? (pb[r >> 1] & 0xffff0000u) : (pb[r >> 1] << 16);
-      plo[r] = pr[r] - __builtin_bit_cast(float, hi_bits);
-    }
-    pb[2] = pack_bf16x2(plo[0], plo[1]);
-    pb[3] = pack_bf16x2(plo[2], plo[3]);
-    const bf16x8 pop = __builtin_bit_cast(bf16x8, pb);
-
-    // O^T[d, head] += sum_row V[row, d] P[row, head], 16 d per MFMA.  LDS operations of one wave
-    // execute in order, so the fences only pin the compiler's ordering of tile writes and reads.
-    // The reads are issued four at a time ahead of the MFMAs that use them.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    // B operand of S^T = K.Q^T: for MFMA step ks lane (n, g) holds the eight q[head n][d] whose K
+    // elements the lane's 16-byte K loads deliver: d = 32*ks + 8*g + j for bf16 rows; for fp8 rows one
+    // load carries 16 elements, so steps 2c and 2c+1 take d = 64*c + 16*g + j and + 8.  Zero for
+    // padded heads.
+    bf16x8 qop[4];
     {
-      const int row = 4 * g + (n >> 2);
-      const int base = row * kRowBytes + ((n & 1) << 3);
-      const int swz = (row & 7) << 1;
+      const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * kD;
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        u32x4 vop[4];
-#pragma unroll
-        for (int d4 = 0; d4 < 4; ++d4) {
-          const int db = 4 * half + d4;
-          const int off = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
-          const s16x4 quad =
-              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(v_tile + off));
-          const u32x2 qd = __builtin_bit_cast(u32x2, quad);
-          vop[d4] = (u32x4){qd[0], qd[1], qd[0], qd[1]};
-        }
-#pragma unroll
-        for (int d4 = 0; d4 < 4; ++d4)
-          acc[4 * half + d4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[d4]), pop,
-                                                                       acc[4 * half + d4], 0, 0, 0);
+      for (int ks = 0; ks < 4; ++ks) {
+        const int d0 = FP8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
+        u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + d0);
+        if (n >= G) raw = (u32x4){0, 0, 0, 0};
+        qop[ks] = __builtin_bit_cast(bf16x8, raw);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  };
+    float slope_log2 = 0.f;
+    if (ALIBI) slope_log2 = n < G ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
 
-  // A ring of kStages register tiles per wave: while one tile is consumed the loads of the wave's next
-  // kStages-1 tiles are in flight.  The steady-state path has no join after a load, only exits.
-  if (my_tiles > 0) {
-    u32x4 kbuf[kStages][4], vbuf[kStages][4];
-    if constexpr (kStages == 1) {
-      // one register tile per wave, refilled inside consume() as soon as its contents have been used:
-      // the loads of tile i+1 fly during the softmax and P.V of tile i at no extra register cost
-      load_k(0, kbuf[0]);
-      load_v(0, vbuf[0]);
-      for (int i = 0; i < my_tiles; ++i) consume(i, kbuf[0], vbuf[0]);
-    } else {
+    f32x4 acc[8];
 #pragma unroll
-      for (int st = 0; st < kStages - 1; ++st) {
-        load_k(st, kbuf[st]);
-        load_v(st, vbuf[st]);
+    for (int i = 0; i < 8; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY;  // running max of scaled logits (log2 units) of head n
+    float l_run = 0.f;        // this lane's share of the running sum
+
+    // The segment's tiles are dealt round-robin to the four waves: this wave owns tiles wave, wave+4, ...
+    // Only the last tile of a sequence can be ragged; its missing rows are redirected to the last valid
+    // row (their logits are masked) so no lane reads past the mapped part of a range.
+    const int n_tiles = seg_tiles;
+    const int my_tiles = (n_tiles - wave + kWaves - 1) / kWaves;
+    const int valid_last = seg_end - (seg_start + (n_tiles - 1) * kTile);  // rows in the last tile, 1..16
+    // per-lane byte offsets inside a tile: K lane (n, g) takes row n, bytes [16g, +16) of each 64-byte
+    // quarter (exactly its MFMA A operand); V lane takes row 4j+g, piece n: four full rows per load
+    // (fp8 rows are 128 bytes: a V load then covers eight rows, lane l takes row 8j + l/8, piece l%8).
+    const uint32_t k_off = (uint32_t)n * row_stride + g * 16;
+    const uint32_t k_off_last = (uint32_t)min(n, valid_last - 1) * row_stride + g * 16;
+    uint32_t v_off[kLoads], v_off_last[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      const int row = FP8 ? 8 * j + (lane >> 3) : 4 * j + g;
+      const int col = FP8 ? (lane & 7) * 16 : n * 16;
+      v_off[j] = (uint32_t)row * row_stride + col;
+      v_off_last[j] = (uint32_t)min(row, valid_last - 1) * row_stride + col;
+    }
+
+    // Loads of the i-th tile of this wave.  Always issued, never predicated, so the wait counters the
+    // compiler derives are exact; past the wave's last tile the last tile is simply loaded again
+    // (it hits in cache and is not consumed).
+    auto load_k = [&](int i, u32x4 *kr) {
+      const int tile = wave + kWaves * min(i, my_tiles - 1);
+      const bool last = tile == n_tiles - 1;
+      gptr kp = k_base + (int64_t)(seg_start + tile * kTile) * row_stride + (last ? k_off_last : k_off);
+#pragma unroll
+      for (int ks = 0; ks < kLoads; ++ks) kr[ks] = *(gvec)(kp + ks * 64);
+    };
+    auto load_v = [&](int i, u32x4 *vr) {
+      const int tile = wave + kWaves * min(i, my_tiles - 1);
+      const bool last = tile == n_tiles - 1;
+      const int64_t row0 = (int64_t)(seg_start + tile * kTile) * row_stride;
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) vr[j] = *(gvec)(v_base + row0 + (last ? v_off_last[j] : v_off[j]));
+    };
+
+    // one 16-row tile: logits, online softmax update, P.V
+    auto consume = [&](int i, u32x4 *kreg, u32x4 *vreg) {
+      const int tile = wave + kWaves * i;
+      const int t0 = seg_start + tile * kTile;
+      // S^T[row, head] = sum_d K[row, d] q[head, d]
+      f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const u32x4 kop =
+            FP8 ? fp8x8_to_bf16x8(kreg[ks >> 1][2 * (ks & 1)], kreg[ks >> 1][2 * (ks & 1) + 1]) : kreg[ks];
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kop), qop[ks], s, 0, 0, 0);
       }
-      int i = 0;
+      if (kStages == 1) load_k(i + 1, kreg);  // the K registers are free again: refill them for the next tile
+
+      // stage V (as bf16) for the transposing read
+      if constexpr (FP8) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int row = 8 * j + (lane >> 3), piece = 2 * (lane & 7);
+          *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece)) = fp8x8_to_bf16x8(vreg[j][0], vreg[j][1]);
+          *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece + 1)) = fp8x8_to_bf16x8(vreg[j][2], vreg[j][3]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(4 * j + g, n)) = vreg[j];
+      }
+      if (kStages == 1) load_v(i + 1, vreg);  // likewise the V registers once they are in LDS
+
+      // logits in log2 units; lane owns rows t0 + 4*g + r of head n
+      float x[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        x[r] = s[r] * p.scale_log2;
+        if (ALIBI) x[r] += slope_log2 * (float)(t0 + 4 * g + r - seq_len + 1);
+      }
+      if (tile == n_tiles - 1 && valid_last < kTile) {  // wave-uniform: only a sequence's ragged last tile
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (4 * g + r >= valid_last) x[r] = -INFINITY;
+      }
+      const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
+      const float m_new = fmaxf(m_run, tmax);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
+      m_run = m_new;
+      float pr[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+      l_run = l_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+        for (int d = 0; d < 8; ++d) acc[d] *= alpha;
+      }
+      // P^T as B operand, split into a bf16 head and a bf16 tail so that P.V keeps ~16 mantissa bits of
+      // P (the result then tracks an fp32-P reference, not just a bf16-P one).  Head and tail share one
+      // K=32 MFMA: reduction slot (g, j) of v_mfma_f32_16x16x32_bf16 stands for row 4g+j with the head of
+      // P for j < 4 and for row 4g+j-4 with the tail for j >= 4, so the B operand is [head(4), tail(4)]
+      // straight from this lane's four logits and the A operand is the lane's V^T quad twice.
+      float plo[4];
+      u32x4 pb;
+      pb[0] = pack_bf16x2(pr[0], pr[1]);
+      pb[1] = pack_bf16x2(pr[2], pr[3]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const unsigned hi_bits = (r & 1) ? (pb[r >> 1] & 0xffff0000u) : (pb[r >> 1] << 16);
+        plo[r] = pr[r] - __builtin_bit_cast(float, hi_bits);
+      }
+      pb[2] = pack_bf16x2(plo[0], plo[1]);
+      pb[3] = pack_bf16x2(plo[2], plo[3]);
+      const bf16x8 pop = __builtin_bit_cast(bf16x8, pb);
+
+      // O^T[d, head] += sum_row V[row, d] P[row, head], 16 d per MFMA.  LDS operations of one wave
+      // execute in order, so the fences only pin the compiler's ordering of tile writes and reads.
+      // The reads are issued four at a time ahead of the MFMAs that use them.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      {
+        const int row = 4 * g + (n >> 2);
+        const int base = row * kRowBytes + ((n & 1) << 3);
+        const int swz = (row & 7) << 1;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          u32x4 vop[4];
+#pragma unroll
+          for (int d4 = 0; d4 < 4; ++d4) {
+            const int db = 4 * half + d4;
+            const int off = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
+            const s16x4 quad =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(v_tile + off));
+            const u32x2 qd = __builtin_bit_cast(u32x2, quad);
+            vop[d4] = (u32x4){qd[0], qd[1], qd[0], qd[1]};
+          }
+#pragma unroll
+          for (int d4 = 0; d4 < 4; ++d4)
+            acc[4 * half + d4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[d4]), pop,
+                                                                         acc[4 * half + d4], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    // A ring of kStages register tiles per wave: while one tile is consumed the loads of the wave's next
+    // kStages-1 tiles are in flight.  The steady-state path has no join after a load, only exits.
+    if (my_tiles > 0) {
+      u32x4 kbuf[kStages][4], vbuf[kStages][4];
+      if constexpr (kStages == 1) {
+        // one register tile per wave, refilled inside consume() as soon as its contents have been used:
+        // the loads of tile i+1 fly during the softmax and P.V of tile i at no extra register cost
+        load_k(0, kbuf[0]);
+        load_v(0, vbuf[0]);
+        for (int i = 0; i < my_tiles; ++i) consume(i, kbuf[0], vbuf[0]);
+      } else {
+#pragma unroll
+        for (int st = 0; st < kStages - 1; ++st) {
+          load_k(st, kbuf[st]);
+          load_v(st, vbuf[st]);
+        }
+        int i = 0;
 #define VTKV_STAGE(ST)                                                           \
   {                                                                              \
     load_k(i + kStages - 1, kbuf[((ST) + kStages - 1) % kStages]);               \
@@ -357,84 +440,104 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kWaves * 64) decode_attn_p
     consume(i, kbuf[(ST)], vbuf[(ST)]);                                          \
     if (++i >= my_tiles) break;                                                  \
   }
-      for (;;) {
-        VTKV_STAGE(0)
-        if constexpr (kStages > 1) VTKV_STAGE(1)
-        if constexpr (kStages > 2) VTKV_STAGE(2)
-        if constexpr (kStages > 3) VTKV_STAGE(3)
-      }
+        for (;;) {
+          VTKV_STAGE(0)
+          if constexpr (kStages > 1) VTKV_STAGE(1)
+          if constexpr (kStages > 2) VTKV_STAGE(2)
+          if constexpr (kStages > 3) VTKV_STAGE(3)
+        }
 #undef VTKV_STAGE
+      }
     }
-  }
 
-#ifdef VTKV_DBG_SKIP_EPILOGUE
-  {
-    float t = l_run + m_run;
-    for (int d = 0; d < 8; ++d) t += acc[d][0] + acc[d][1] + acc[d][2] + acc[d][3];
-    if (t == 1.2345f) p.part_max[0] = t;
-  }
-  return;
-#endif
-  // ---- merge the four waves.  l_run is still split over the four row groups of a lane column.
-  l_run = sum_over_row_groups(l_run);
-  __syncthreads();  // every wave is done with its V tile: smem is free for the merge
-  float *sm_m = reinterpret_cast<float *>(smem + kWaves * kTile * kRowBytes);  // [4][16]
-  float *sm_l = sm_m + kWaves * 16;                                               // [4][16]
-  float *sm_o = reinterpret_cast<float *>(smem);                                  // [4][G][128] (<= 16 KiB at G<=8)
-  if (g == 0) {
-    sm_m[wave * 16 + n] = m_run;
-    sm_l[wave * 16 + n] = l_run;
-  }
-  __syncthreads();
-  float m_wg = fmaxf(fmaxf(sm_m[n], sm_m[16 + n]), fmaxf(sm_m[32 + n], sm_m[48 + n]));
-  const float f = __builtin_amdgcn_exp2f(m_run - m_wg);  // 0 for a wave that saw no row
-  // G <= 8 fits the 16 KiB; for larger groups the merge runs in two halves of 8 heads
-  for (int h0 = 0; h0 < G; h0 += 8) {
-    if (h0 > 0) __syncthreads();
-    if (n >= h0 && n < min(G, h0 + 8)) {
-#pragma unroll
-      for (int db = 0; db < 8; ++db)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          sm_o[(wave * 8 + (n - h0)) * kD + db * 16 + 4 * g + i] = acc[db][i] * f;
+    // ---- merge the four waves.  l_run is still split over the four row groups of a lane column.
+    l_run = sum_over_row_groups(l_run);
+    __syncthreads();  // every wave is done with its V tile: smem is free for the merge
+    float *sm_m = reinterpret_cast<float *>(smem + kWaves * kTile * kRowBytes);  // [4][16]
+    float *sm_l = sm_m + kWaves * 16;                                               // [4][16]
+    float *sm_o = reinterpret_cast<float *>(smem);                                  // [4][8][128] = 16 KiB
+    if (g == 0) {
+      sm_m[wave * 16 + n] = m_run;
+      sm_l[wave * 16 + n] = l_run;
     }
     __syncthreads();
-    const int nh = min(G, h0 + 8) - h0;
-    for (int idx = threadIdx.x; idx < nh * kD; idx += kWaves * 64) {
-      const int hh = idx / kD, d = idx % kD;
-      const int head = h0 + hh;
-      const float mw = fmaxf(fmaxf(sm_m[head], sm_m[16 + head]), fmaxf(sm_m[32 + head], sm_m[48 + head]));
-      float lsum = 0.f, o = 0.f;
+    const float m_wg = fmaxf(fmaxf(sm_m[n], sm_m[16 + n]), fmaxf(sm_m[32 + n], sm_m[48 + n]));
+    const float f = __builtin_amdgcn_exp2f(m_run - m_wg);  // 0 for a wave that saw no row
+    // slot of this (workgroup, segment): both indices only grow along the tile order, so the sum is unique
+    const int64_t slot_idx = (int64_t)blockIdx.x + (int64_t)b * Hkv + kvh;
+    // G <= 8 fits the 16 KiB; for larger groups the merge runs in two halves of 8 heads
+    for (int h0 = 0; h0 < G; h0 += 8) {
+      if (h0 > 0) __syncthreads();
+      if (n >= h0 && n < min(G, h0 + 8)) {
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) {
-        lsum += sm_l[w * 16 + head] * __builtin_amdgcn_exp2f(sm_m[w * 16 + head] - mw);
-        o += sm_o[(w * 8 + hh) * kD + d];
+        for (int db = 0; db < 8; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            sm_o[(wave * 8 + (n - h0)) * kD + db * 16 + 4 * g + i] = acc[db][i] * f;
       }
-      const int64_t pidx = ((int64_t)b * p.num_heads + kvh * G + head) * p.max_parts + part;
-      p.part_out[pidx * kD + d] = o / lsum;
-      if (d == 0) {
-        p.part_max[pidx] = mw;   // log2 units
-        p.part_sum[pidx] = lsum;
+      __syncthreads();
+      const int nh = min(G, h0 + 8) - h0;
+      for (int idx = threadIdx.x; idx < nh * kD; idx += kThreads) {
+        const int hh = idx / kD, d = idx % kD;
+        const int head = h0 + hh;
+        const float mw = fmaxf(fmaxf(sm_m[head], sm_m[16 + head]), fmaxf(sm_m[32 + head], sm_m[48 + head]));
+        float lsum = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+          lsum += sm_l[w * 16 + head] * __builtin_amdgcn_exp2f(sm_m[w * 16 + head] - mw);
+          o += sm_o[(w * 8 + hh) * kD + d];
+        }
+        const int64_t pidx = slot_idx * G + head;
+        p.part_out[pidx * kD + d] = o / lsum;
+        if (d == 0) {
+          p.part_max[pidx] = mw;  // log2 units
+          p.part_sum[pidx] = lsum;
+        }
       }
+    }
+
+    // ---- next segment of the span
+    g_cur += seg_tiles;
+    tile0 += seg_tiles;
+    if (g_cur < g_end) {
+      if (tile0 == nt_b) {
+        tile0 = 0;
+        if (++kvh == Hkv) {
+          kvh = 0;
+          do {
+            ++b;
+            nt_b = uniform(s_cum[b + 1]) - uniform(s_cum[b]);
+          } while (nt_b == 0);  // g_cur < total_tiles guarantees a later sequence with rows
+        }
+      }
+      __syncthreads();  // the merge area is the next segment's V tiles
     }
   }
 }
 
-// Merge the partitions of one (sequence, head): out = sum_j o_j w_j / sum_j w_j with
-// w_j = l_j * 2^(m_j - max m)  (csrc/attention/attention_kernels.cu:515-582).
+// Merge the partials of one (sequence, head): out = sum_j o_j w_j / sum_j w_j with
+// w_j = l_j * 2^(m_j - max m)  (csrc/attention/attention_kernels.cu:515-582).  The segment's tiles
+// [first, first + nt) of the global order were handled by workgroups first/span .. (first+nt-1)/span.
 __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
   const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-  const int seq_len = p.seq_lens[b];
-  if (seq_len <= 0) return;
-  const int nparts = (seq_len + p.part_tokens - 1) / p.part_tokens;
-  const int64_t base = ((int64_t)b * p.num_heads + head) * p.max_parts;
+  const int G = p.group, Hkv = p.num_kv_heads;
+  const int cum_b = p.cum_tiles[b];
+  const int nt = p.cum_tiles[b + 1] - cum_b;
+  if (nt <= 0) return;
+  const int total_tiles = p.cum_tiles[p.num_seqs] * Hkv;
+  const int span = span_of(p, total_tiles);
+  const int kvh = head / G, hg = head % G;
+  const int first = cum_b * Hkv + kvh * nt;
+  const int w0 = first / span, w1 = (first + nt - 1) / span;
+  const int64_t seg = (int64_t)b * Hkv + kvh;
   float m = -INFINITY;
-  for (int j = 0; j < nparts; ++j) m = fmaxf(m, p.part_max[base + j]);
+  for (int w = w0; w <= w1; ++w) m = fmaxf(m, p.part_max[(w + seg) * G + hg]);
   float wsum = 0.f, o = 0.f;
-  for (int j = 0; j < nparts; ++j) {
-    const float w = p.part_sum[base + j] * __builtin_amdgcn_exp2f(p.part_max[base + j] - m);
-    wsum += w;
-    o += p.part_out[(base + j) * kD + d] * w;
+  for (int w = w0; w <= w1; ++w) {
+    const int64_t pidx = (w + seg) * G + hg;
+    const float wt = p.part_sum[pidx] * __builtin_amdgcn_exp2f(p.part_max[pidx] - m);
+    wsum += wt;
+    o += p.part_out[pidx * kD + d] * wt;
   }
   const float r = o / wsum * p.v_scale;
   const int64_t oi = ((int64_t)b * p.num_heads + head) * kD + d;
@@ -453,11 +556,42 @@ struct KernelTimer {
 };
 KernelTimer g_timer;
 
-// 512 rows per workgroup (the reference's PARTITION_SIZE, csrc/attention/attention_kernels.cu:37):
-// measured best on MI355X between per-workgroup fixed cost and balance across the 256 CUs.
-int default_part_tokens(int max_seq_len) {
-  (void)max_seq_len;
-  return 512;
+// Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
+struct Residency {
+  std::mutex mu;
+  int device = -1;
+  int grid[4] = {0, 0, 0, 0};
+};
+Residency g_res;
+
+template <typename K>
+int resident_grid(K kernel, int variant) {
+  std::lock_guard<std::mutex> lk(g_res.mu);
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (g_res.device != dev) {
+    g_res.device = dev;
+    for (int &v : g_res.grid) v = 0;
+  }
+  if (g_res.grid[variant] == 0) {
+    int per_cu = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, 0) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    g_res.grid[variant] = std::min(std::max(per_cu, 1) * cus, kDefaultMaxGrid);
+  }
+  return g_res.grid[variant];
+}
+
+// Upper bound of the number of partial slots: one per workgroup plus one per (sequence, kv head);
+// each slot holds `group` heads, and num_seqs*num_kv_heads*group = num_seqs*num_heads.
+int64_t scratch_floats(int64_t grid, int num_seqs, int num_heads, int head_size) {
+  return (grid * 16 + (int64_t)num_seqs * num_heads) * (head_size + 2);
+}
+
+int64_t fixed_span_grid(int num_seqs, int num_kv_heads_bound, int max_seq_len, int partition_tokens) {
+  const int64_t tiles = (int64_t)num_seqs * num_kv_heads_bound * ((max_seq_len + kTile - 1) / kTile);
+  const int64_t span = partition_tokens / kTile;
+  return (tiles + span - 1) / span;
 }
 
 }  // namespace
@@ -467,25 +601,27 @@ extern "C" {
 int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_seq_len,
                                               int partition_tokens) {
   if (num_seqs <= 0 || num_heads <= 0 || head_size <= 0 || max_seq_len <= 0) return 0;
-  const int pt = partition_tokens > 0 ? partition_tokens : default_part_tokens(max_seq_len);
-  const int64_t parts = (max_seq_len + pt - 1) / pt;
-  return (int64_t)num_seqs * num_heads * parts * (head_size + 2) * (int64_t)sizeof(float);
+  const int64_t grid = partition_tokens >= kTile ? fixed_span_grid(num_seqs, num_heads, max_seq_len, partition_tokens)
+                                                 : kDefaultMaxGrid;
+  const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
+  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes;
 }
 
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                           const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
                           const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
-                          float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream) {
+                          float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
+                          void *stream) {
   VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids && seq_lens, "null argument");
   VTKV_REQUIRE(num_seqs >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
+  VTKV_REQUIRE(num_seqs <= kMaxSeqs, "at most %d sequences per call, got %d", kMaxSeqs, num_seqs);
   VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
   VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
   VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
   VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be BF16 or FP8_E4M3");
-  if (kv_dtype == VTKV_FP8_E4M3)
-    VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
+  if (kv_dtype == VTKV_FP8_E4M3) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
   const int group = num_heads / num_kv_heads;
   VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0,
@@ -494,13 +630,28 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   // the kernel addresses rows of a range with 32-bit byte offsets
   VTKV_REQUIRE((int64_t)max_seq_len * num_kv_heads * head_size * vtkv::elem_bytes(kv_dtype) < (1ll << 31),
                "a sequence range of %d rows exceeds 2 GiB", max_seq_len);
+  VTKV_REQUIRE(partition_tokens == 0 || (partition_tokens >= kWaves * kTile && partition_tokens % kTile == 0),
+               "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
   if (num_seqs == 0) return VTKV_OK;
-  const int pt = partition_tokens > 0 ? partition_tokens : default_part_tokens(max_seq_len);
-  VTKV_REQUIRE(pt % (kWaves * kTile) == 0, "partition_tokens must be a multiple of %d", kWaves * kTile);
-  const int64_t parts = (max_seq_len + pt - 1) / pt;
-  VTKV_REQUIRE(parts <= 65535 && num_seqs <= 65535, "grid too large: %lld partitions, %d sequences",
-               (long long)parts, num_seqs);
-  const int64_t need = vtkv_decode_attention_workspace_bytes(num_seqs, num_heads, head_size, max_seq_len, pt);
+
+  const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
+  const bool alibi = alibi_slopes != nullptr;
+  int64_t grid;
+  if (partition_tokens > 0) {
+    grid = fixed_span_grid(num_seqs, num_kv_heads, max_seq_len, partition_tokens);
+    VTKV_REQUIRE(grid <= (1ll << 24), "partition_tokens %d gives %lld workgroups", partition_tokens, (long long)grid);
+  } else {
+    int g = 0;
+    if (alibi && fp8) g = resident_grid(decode_attn_stream_kernel<true, true>, 3);
+    else if (alibi) g = resident_grid(decode_attn_stream_kernel<true, false>, 2);
+    else if (fp8) g = resident_grid(decode_attn_stream_kernel<false, true>, 1);
+    else g = resident_grid(decode_attn_stream_kernel<false, false>, 0);
+    if (g <= 0) return vtkv::fail(VTKV_EHIP, "cannot query the kernel's occupancy");
+    grid = g;
+  }
+  const int64_t n_float = scratch_floats(grid, num_seqs, num_heads, head_size);
+  const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
+  const int64_t need = n_float * (int64_t)sizeof(float) + cum_bytes;
   if (!workspace || workspace_bytes < need)
     return vtkv::fail(VTKV_ENOMEM, "workspace of %lld bytes is smaller than the %lld needed",
                       (long long)workspace_bytes, (long long)need);
@@ -513,35 +664,36 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   p.slot_ids = slot_ids;
   p.seq_lens = seq_lens;
   p.alibi_slopes = alibi_slopes;
-  const int64_t n_stat = (int64_t)num_seqs * num_heads * parts;
-  p.part_out = (float *)workspace;
+  const int64_t n_stat = grid * 16 + (int64_t)num_seqs * num_heads;  // (slot, head) pairs
+  p.cum_tiles = (int32_t *)workspace;
+  p.part_out = (float *)((char *)workspace + cum_bytes);
   p.part_max = p.part_out + n_stat * kD;
   p.part_sum = p.part_max + n_stat;
   p.out = out;
   p.out_f32 = out_dtype == VTKV_F32;
   p.q_stride = q_stride;
+  p.num_seqs = num_seqs;
   p.num_heads = num_heads;
   p.num_kv_heads = num_kv_heads;
   p.group = group;
-  p.part_tokens = pt;
-  p.max_parts = (int)parts;
+  p.span_tiles = partition_tokens > 0 ? partition_tokens / kTile : 0;
+  p.grid = (int)grid;
   // x = code * scale: the K scale multiplies every logit, the V scale the whole output
-  p.scale_log2 = scale * kLog2e * (kv_dtype == VTKV_FP8_E4M3 ? k_scale : 1.f);
-  p.v_scale = kv_dtype == VTKV_FP8_E4M3 ? v_scale : 1.f;
+  p.scale_log2 = scale * kLog2e * (fp8 ? k_scale : 1.f);
+  p.v_scale = fp8 ? v_scale : 1.f;
 
   hipStream_t st = (hipStream_t)stream;
   const bool timed = g_timer.on;
   if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[0], st));
-  const dim3 grid(num_kv_heads, (unsigned)parts, num_seqs), block(kWaves * 64);
-  const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
-  if (alibi_slopes && fp8)
-    hipLaunchKernelGGL((decode_attn_partial_kernel<true, true>), grid, block, 0, st, p);
-  else if (alibi_slopes)
-    hipLaunchKernelGGL((decode_attn_partial_kernel<true, false>), grid, block, 0, st, p);
+  const dim3 grid3((unsigned)grid), block(kThreads);
+  if (alibi && fp8)
+    hipLaunchKernelGGL((decode_attn_stream_kernel<true, true>), grid3, block, 0, st, p);
+  else if (alibi)
+    hipLaunchKernelGGL((decode_attn_stream_kernel<true, false>), grid3, block, 0, st, p);
   else if (fp8)
-    hipLaunchKernelGGL((decode_attn_partial_kernel<false, true>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((decode_attn_stream_kernel<false, true>), grid3, block, 0, st, p);
   else
-    hipLaunchKernelGGL((decode_attn_partial_kernel<false, false>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((decode_attn_stream_kernel<false, false>), grid3, block, 0, st, p);
   if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[1], st));
   hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
   if (timed) {

@@ -54,7 +54,10 @@ def test_version_and_constants_without_a_gpu():
     lib = _C.lib()
     assert lib.vtkv_version() >= 100
     assert lib.vtkv_chunk_bytes() == 2 * 1024 * 1024
-    assert lib.vtkv_decode_attention_workspace_bytes(64, 32, 128, 4096, 256) == 64 * 32 * 16 * 130 * 4
+    ws = lib.vtkv_decode_attention_workspace_bytes
+    assert ws(64, 32, 128, 4096, 0) > 64 * 32 * 130 * 4       # at least one partial per (sequence, head)
+    assert ws(64, 32, 128, 4096, 256) > ws(64, 32, 128, 4096, 1024) > 0   # smaller spans, more partials
+    assert ws(0, 32, 128, 4096, 0) == 0
 
 
 def test_host_arena_first_fit_and_coalescing():
