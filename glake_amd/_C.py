@@ -62,6 +62,7 @@ SIGNATURES = {
     "vtkv_ptr_table_fill": (_i, [_u64, _p, _i, _i, _i]),
     "vtkv_memcpy_h2d": (_i, [_u64, _p, _i64]),
     "vtkv_memcpy_d2h": (_i, [_p, _u64, _i64]),
+    "vtkv_memcpy_h2d_async": (_i, [_u64, _p, _i64, _p]),
     "vtkv_reshape_and_cache": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i, _i, _f, _f, _p]),
     "vtkv_reshape_and_cache_paged": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i, _p]),
     "vtkv_swap_blocks": (_i, [_p, _p, _i64, _p, _i, _i, _p]),

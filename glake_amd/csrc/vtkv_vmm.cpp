@@ -427,6 +427,13 @@ int vtkv_memcpy_h2d(uint64_t dst, const void *src, int64_t bytes) {
   return VTKV_OK;
 }
 
+int vtkv_memcpy_h2d_async(uint64_t dst, const void *src, int64_t bytes, void *stream) {
+  VTKV_REQUIRE(bytes >= 0 && (bytes == 0 || (dst && src)), "null argument");
+  if (bytes)
+    VTKV_HIP(hipMemcpyAsync((void *)(uintptr_t)dst, src, (size_t)bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+  return VTKV_OK;
+}
+
 int vtkv_memcpy_d2h(void *dst, uint64_t src, int64_t bytes) {
   VTKV_REQUIRE(bytes >= 0 && (bytes == 0 || (dst && src)), "null argument");
   if (bytes) VTKV_HIP(hipMemcpy(dst, (const void *)(uintptr_t)src, (size_t)bytes, hipMemcpyDeviceToHost));

@@ -37,3 +37,105 @@ def prepare_step(attn_metadata, kv_caches: Sequence) -> None:
                                        attn_metadata.kvcache_segment, attn_metadata.set_used_size, kv_size,
                                        attn_metadata.num_prefills == 0)  # llama.py:340
     attn_metadata.slot_m = torch.tensor(slot_m, dtype=torch.int64, device=attn_metadata.slot_mapping.device)
+
+
+class DecodeStepPlan:
+    """One decode step of one layer for a fixed set of sequences, with the per-step host work cut down.
+
+    ``run`` does what the reference does per step and layer through separate Python calls
+    (vllm/model_executor/models/llama.py:307-341 then vllm/attention/backends/xformers.py:301-371):
+    advance each sequence's range by one token row (mapping a chunk at a 2 MiB boundary), upload the
+    byte offsets and the new sequence lengths, append the step's K/V rows and run decode attention
+    over the whole context.  The same C entry points are used as by the separate ops
+    (``vtkv_extend_kv_cache_batch``, ``vtkv_reshape_and_cache``, ``vtkv_decode_attention``); what the
+    plan saves is per-call Python: argument arrays, the device tables and the pinned staging ring are
+    made once, the bookkeeping writes its offsets straight into pinned memory, and both metadata arrays
+    travel in one asynchronous copy.  Build a new plan when the set of running sequences changes.
+    """
+
+    def __init__(self, segments: Sequence, slot_ids: Sequence[int], key_cache, value_cache, num_heads: int,
+                 num_kv_heads: int, head_size: int, scale: float, kv_cache_dtype: str = "auto", k_scale: float = 1.0,
+                 v_scale: float = 1.0, model_dtype: torch.dtype = torch.bfloat16, device=None, ring: int = 128):
+        import ctypes as C
+
+        import numpy as np
+
+        from .. import _C, _custom_ops as ops
+
+        if len(segments) != len(slot_ids) or not segments:
+            raise _C.VtkvError(_C.EINVAL, "DecodeStepPlan: one slot id per segment, at least one sequence")
+        if ring < 2 or ring % 2:
+            raise _C.VtkvError(_C.EINVAL, "DecodeStepPlan: ring must be even and at least 2")
+        self._C, self._lib, self._np = _C, _C.lib(), np
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        n = self.n = len(segments)
+        self.num_heads, self.num_kv_heads, self.head_size = int(num_heads), int(num_kv_heads), int(head_size)
+        self.scale = float(scale)
+        self._src_dt = ops._DTYPES[model_dtype]
+        self._kv_dt = ops._kv_dtype(kv_cache_dtype, self._src_dt)
+        self.k_scale, self.v_scale = float(k_scale), float(v_scale)
+        self.kv_size = self.num_kv_heads * self.head_size * (1 if self._kv_dt == _C.FP8_E4M3 else 2)  # bytes per row
+        self._segments = list(segments)  # keeps the handles alive
+        self._segs = (C.c_void_p * n)(*[s._h for s in segments])
+        self._tok = (C.c_int64 * n)(*([self.kv_size] * n))
+        self._k_table, self._v_table = ops._ptr(key_cache), ops._ptr(value_cache)
+        self._tables = (key_cache, value_cache)
+        self._slot_t = torch.tensor(list(slot_ids), dtype=torch.int64, device=self.device)
+        self._slot_p = C.c_void_p(self._slot_t.data_ptr())
+        # per step: n int64 byte offsets then n int32 lengths; a ring of pinned rows, guarded by one event
+        # per half so that a row is rewritten only after its previous upload has run
+        self._ring = ring
+        self._stage = torch.empty(ring, 3 * n, dtype=torch.int32).pin_memory()
+        stage_np = self._stage.numpy()
+        self._offs = [stage_np[i, :2 * n].view(np.int64) for i in range(ring)]
+        self._lens = [stage_np[i, 2 * n:] for i in range(ring)]
+        self._row_p = [C.c_void_p(self._stage[i].data_ptr()) for i in range(ring)]
+        self._meta = torch.empty(3 * n, dtype=torch.int32, device=self.device)
+        self._meta_addr = self._meta.data_ptr()
+        self._offs_p = C.c_void_p(self._meta_addr)
+        self._lens_p = C.c_void_p(self._meta_addr + 8 * n)
+        self._events = [torch.cuda.Event(), torch.cuda.Event()]
+        self._recorded = [False, False]
+        self._row = 0
+        need = self._lib.vtkv_decode_attention_workspace_bytes(n, self.num_heads, self.head_size, 1, 0)
+        self._ws = ops._workspace(need, self.device)
+        self._ws_p, self._ws_n = C.c_void_p(self._ws.data_ptr()), self._ws.numel()
+        self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
+
+    def run(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
+            alibi_slopes=None) -> int:
+        """query [n, num_heads, head_size]; key/value [n, num_kv_heads*head_size] (or 3-d), the step's new
+        rows; out like query (or float32).  Returns the longest sequence length after the step."""
+        C_void_p = type(self._slot_p)
+        lib, check, n = self._lib, self._C.check, self.n
+        i, half = self._row, self._ring // 2
+        if i == 0 or i == half:
+            h = 0 if i == 0 else 1
+            if self._recorded[h]:
+                self._events[h].synchronize()
+        check(lib.vtkv_extend_kv_cache_batch(self._segs, n, self._tok, None, self.kv_size, 1, self._row_p[i]))
+        lens = self._lens[i]
+        self._np.floor_divide(self._offs[i], self.kv_size, out=lens, casting="unsafe")
+        lens += 1
+        max_len = int(lens.max())
+        stream = C_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        check(lib.vtkv_memcpy_h2d_async(self._meta_addr, self._row_p[i], 12 * n, stream))
+        if i == half - 1 or i == self._ring - 1:
+            h = 0 if i == half - 1 else 1
+            self._events[h].record()
+            self._recorded[h] = True
+        self._row = (i + 1) % self._ring
+        self.seq_lens = lens
+        kstride = key.stride(0)
+        vstride = value.stride(0)
+        check(lib.vtkv_reshape_and_cache(
+            C_void_p(key.data_ptr()), C_void_p(value.data_ptr()), self._k_table, self._v_table, self._offs_p,
+            self._slot_p, None, None, n, 1, self.num_kv_heads, self.head_size, kstride, vstride, self._src_dt,
+            self._kv_dt, self.k_scale, self.v_scale, stream))
+        out_dt = self._C.F32 if out.dtype == torch.float32 else self._C.BF16
+        check(lib.vtkv_decode_attention(
+            C_void_p(out.data_ptr()), C_void_p(query.data_ptr()), self._k_table, self._v_table, self._slot_p,
+            self._lens_p, n, self.num_heads, self.num_kv_heads, self.head_size, query.stride(0), self.scale, max_len,
+            None if alibi_slopes is None else C_void_p(alibi_slopes.data_ptr()), self._src_dt, out_dt, self._kv_dt,
+            self.k_scale, self.v_scale, self._ws_p, self._ws_n, 0, stream))
+        return max_len

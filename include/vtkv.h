@@ -118,6 +118,11 @@ int vtkv_ptr_table_fill(uint64_t table, vtkv_segment *const *segs, int n, int la
  * For tests and debugging; replaces write_string / read_string (vmm_allocator.cpp:423-446). */
 int vtkv_memcpy_h2d(uint64_t dst, const void *src, int64_t bytes);
 int vtkv_memcpy_d2h(void *dst, uint64_t src, int64_t bytes);
+/* Asynchronous upload on `stream` from pinned host memory (vtkv_host_alloc, or any hipHostMalloc'ed
+ * buffer), which must stay untouched until the copy has run.  Carries a step's byte offsets and sequence
+ * lengths to the device; replaces the torch.tensor(..., device="cuda") uploads of
+ * vllm/model_executor/models/llama.py:340-341. */
+int vtkv_memcpy_h2d_async(uint64_t dst, const void *src, int64_t bytes, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Cache ops.  Replace vllm._C.cache_ops (csrc/pybind.cpp:88-117, csrc/cache.h:8-44).
