@@ -75,7 +75,7 @@ SIGNATURES = {
     "vtkv_decode_attention": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f, _i, _p, _i, _i, _i, _f, _f, _p,
                                     _i64, _i, _p]),
     "vtkv_set_kernel_timing": (_i, [_i]),
-    "vtkv_last_attention_kernel_ms": (_i, [_p, _p]),
+    "vtkv_attention_kernel_times": (_i, [_p, _p, _i]),
 }
 
 _lib = None

@@ -44,6 +44,7 @@
 // denominator (the CPU twin has none, csrc/cpu/attention.cpp:43-67).
 #include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "vtkv_common.h"
 #ifndef VTKV_ATTN_STAGES
@@ -314,15 +315,18 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stre
     }
 
     // Loads of the i-th tile of this wave.  Always issued, never predicated, so the wait counters the
-    // compiler derives are exact; past the wave's last tile the last tile is simply loaded again
-    // (it hits in cache and is not consumed).
+    // compiler derives are exact; past the wave's last tile every lane loads the segment's first 16
+    // bytes instead (one cache line per load, not consumed).
     auto load_tile = [&](gptr base, int i, u32x4 *regs) {
-      const int tile = wave + kWaves * min(i, my_tiles - 1);
+      const bool live = i < my_tiles;
+      const int tile = wave + kWaves * i;
       const bool last = tile == n_tiles - 1;
-      const int64_t row0 = (int64_t)(seg_start + tile * kTile) * row_stride;
+      // (a mask, not a select: selects here end up as branches around separate copies of the loads)
+      const uint32_t mask = uniform(live ? ~0u : 0u);
+      const int64_t row0 = (int64_t)((uint32_t)(seg_start + tile * kTile) & mask) * row_stride;
 #pragma unroll
       for (int j = 0; j < kLoads; ++j)
-        regs[j] = __builtin_nontemporal_load((gvec)(base + row0 + (last ? t_off_last[j] : t_off[j])));
+        regs[j] = __builtin_nontemporal_load((gvec)(base + row0 + ((last ? t_off_last[j] : t_off[j]) & mask)));
     };
     auto load_k = [&](int i, u32x4 *kr) { load_tile(k_base, i, kr); };
     auto load_v = [&](int i, u32x4 *vr) { load_tile(v_base, i, vr); };
@@ -574,11 +578,13 @@ __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
 }
 
 // Optional per-kernel timing for benchmarks: when switched on, every vtkv_decode_attention call
-// records events around its two launches on the caller's stream.
+// records events around its two launches on the caller's stream, without waiting for them, so the
+// calls stay queued back to back as they are in production.  Up to kTimedCalls calls are kept.
+constexpr int kTimedCalls = 1024;
 struct KernelTimer {
   bool on = false;
-  hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
-  bool recorded = false;
+  std::vector<hipEvent_t> ev;  // three per call, created on first use
+  int calls = 0;
 };
 KernelTimer g_timer;
 
@@ -709,8 +715,17 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   p.v_scale = fp8 ? v_scale : 1.f;
 
   hipStream_t st = (hipStream_t)stream;
-  const bool timed = g_timer.on;
-  if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[0], st));
+  const bool timed = g_timer.on && g_timer.calls < kTimedCalls;
+  hipEvent_t *ev = nullptr;
+  if (timed) {
+    if ((int)g_timer.ev.size() < 3 * (g_timer.calls + 1)) {
+      hipEvent_t e3[3];
+      for (auto &e : e3) VTKV_HIP(hipEventCreate(&e));
+      g_timer.ev.insert(g_timer.ev.end(), e3, e3 + 3);
+    }
+    ev = &g_timer.ev[3 * g_timer.calls];
+    VTKV_HIP(hipEventRecord(ev[0], st));
+  }
   const dim3 grid3((unsigned)grid), block(kThreads);
   if (alibi && fp8)
     hipLaunchKernelGGL((decode_attn_stream_kernel<true, true>), grid3, block, 0, st, p);
@@ -720,31 +735,32 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
     hipLaunchKernelGGL((decode_attn_stream_kernel<false, true>), grid3, block, 0, st, p);
   else
     hipLaunchKernelGGL((decode_attn_stream_kernel<false, false>), grid3, block, 0, st, p);
-  if (timed) VTKV_HIP(hipEventRecord(g_timer.ev[1], st));
+  if (timed) VTKV_HIP(hipEventRecord(ev[1], st));
   hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
   if (timed) {
-    VTKV_HIP(hipEventRecord(g_timer.ev[2], st));
-    g_timer.recorded = true;
+    VTKV_HIP(hipEventRecord(ev[2], st));
+    ++g_timer.calls;
   }
   VTKV_HIP(hipGetLastError());
   return VTKV_OK;
 }
 
 int vtkv_set_kernel_timing(int on) {
-  if (on && !g_timer.ev[0])
-    for (auto &e : g_timer.ev) VTKV_HIP(hipEventCreate(&e));
   g_timer.on = on != 0;
-  g_timer.recorded = false;
+  if (on) g_timer.calls = 0;
   return VTKV_OK;
 }
 
-int vtkv_last_attention_kernel_ms(float *partial_ms, float *reduce_ms) {
-  VTKV_REQUIRE(partial_ms && reduce_ms, "null argument");
-  if (!g_timer.recorded) return vtkv::fail(VTKV_ESTATE, "no timed vtkv_decode_attention call to report");
-  VTKV_HIP(hipEventSynchronize(g_timer.ev[2]));
-  VTKV_HIP(hipEventElapsedTime(partial_ms, g_timer.ev[0], g_timer.ev[1]));
-  VTKV_HIP(hipEventElapsedTime(reduce_ms, g_timer.ev[1], g_timer.ev[2]));
-  return VTKV_OK;
+int vtkv_attention_kernel_times(float *stream_ms, float *reduce_ms, int capacity) {
+  VTKV_REQUIRE(stream_ms && reduce_ms && capacity >= 0, "null argument");
+  const int n = std::min(capacity, g_timer.calls);
+  for (int i = 0; i < n; ++i) {
+    hipEvent_t *ev = &g_timer.ev[3 * i];
+    VTKV_HIP(hipEventSynchronize(ev[2]));
+    VTKV_HIP(hipEventElapsedTime(&stream_ms[i], ev[0], ev[1]));
+    VTKV_HIP(hipEventElapsedTime(&reduce_ms[i], ev[1], ev[2]));
+  }
+  return n;
 }
 
 }  // extern "C"

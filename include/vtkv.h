@@ -214,12 +214,13 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                           void *stream);
 
 /* Benchmark aid without a counterpart in the reference (its kernel benchmark times from the host,
- * benchmarks/kernels/benchmark_paged_attention.py:147-157): when switched on, each
- * vtkv_decode_attention call records HIP events around its kernels on the caller's stream, and
- * vtkv_last_attention_kernel_ms waits for the last such call and returns the duration of its split-K
- * kernel and of its merge kernel in milliseconds. */
+ * benchmarks/kernels/benchmark_paged_attention.py:147-157): while switched on, each vtkv_decode_attention
+ * call (up to 1024 of them) records HIP events around its kernels on the caller's stream without waiting
+ * for them.  vtkv_attention_kernel_times waits for the recorded calls and writes, for the first
+ * min(capacity, calls) of them in call order, the duration of the streaming kernel and of the merge
+ * kernel in milliseconds; it returns that count.  Switching timing on again starts a new series. */
 int vtkv_set_kernel_timing(int on);
-int vtkv_last_attention_kernel_ms(float *partial_ms, float *reduce_ms);
+int vtkv_attention_kernel_times(float *stream_ms, float *reduce_ms, int capacity);
 
 #ifdef __cplusplus
 }
