@@ -191,7 +191,7 @@ int vtkv_convert_fp8(void *dst, const void *src, int64_t n, float scale, int to_
  * call (vllm/attention/backends/xformers.py:407-430).
  * ---------------------------------------------------------------------------------------- */
 
-/* Bytes of scratch vtkv_decode_attention needs for these sizes (partition_tokens: 0 = library default). */
+/* Bytes of scratch vtkv_decode_attention needs for these sizes (partition_tokens as below). */
 int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_seq_len,
                                               int partition_tokens);
 
@@ -204,7 +204,13 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  *   max_seq_len  host upper bound of seq_lens (sizes the grid, as in the reference launcher)
  *   alibi_slopes device float[num_heads] or NULL
  *   kv_dtype     q_dtype, or VTKV_FP8_E4M3 with k_scale / v_scale (x = code * scale)
- *   workspace    device scratch of at least vtkv_decode_attention_workspace_bytes(...) bytes
+ *   workspace    device scratch of at least vtkv_decode_attention_workspace_bytes(...) bytes; calls that
+ *                share a workspace must be ordered on one stream
+ *   partition_tokens  0: the rows of the whole batch are cut into equal contiguous spans, one per
+ *                workgroup of a grid that fills the device once, whatever the sequence lengths are;
+ *                > 0 (a multiple of 16, at least 64): every workgroup takes that many rows, the
+ *                reference's fixed partitions (512 in paged_attention_v2, csrc/attention/attention_kernels.cu:739-914).
+ *                The result does not depend on the choice beyond fp32 summation order.
  * Supported: q_dtype VTKV_BF16, kv_dtype VTKV_BF16 or VTKV_FP8_E4M3, head_size 128, num_heads/num_kv_heads in 1..16. */
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                           const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
