@@ -59,6 +59,8 @@ def main() -> int:
     ap.add_argument("--partition-tokens", type=int, default=0)
     ap.add_argument("--host-path", default="plan", choices=["plan", "ops"],
                     help="plan: DecodeStepPlan (arguments prepared once); ops: the separate reference-style op calls")
+    ap.add_argument("--unfused", action="store_true",
+                    help="plan path: separate reshape_and_cache and attention launches instead of the fused one")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -139,7 +141,8 @@ def main() -> int:
 
     from glake_amd.worker.step import DecodeStepPlan
     plan = DecodeStepPlan(segs, slot_ids, engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hq, Hkv, D, scale,
-                          kv_cache_dtype=kv_dtype, k_scale=k_scale, v_scale=v_scale, device=dev)
+                          kv_cache_dtype=kv_dtype, k_scale=k_scale, v_scale=v_scale, device=dev,
+                          fused=not args.unfused)
     q3 = q.view(B, Hq, D)
 
     def step_plan() -> int:
@@ -239,7 +242,8 @@ def main() -> int:
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 (fp8-e4m3 KV)" if fp8 else "bf16", "data": "synthetic",
         "config": {"workload": cfg["name"], "layers": 1, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
-                   "mean_ctx": round(float(np.mean(final_lens)), 1), "host_path": args.host_path},
+                   "mean_ctx": round(float(np.mean(final_lens)), 1), "host_path": args.host_path,
+                   "fused_append": bool(plan.fused) and step is step_plan},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "host_issue_ms_per_step": round(host_dt / K * 1e3, 4),

@@ -112,6 +112,61 @@ def paged_attention_v1(
         float(kv_scale if v_scale is None else v_scale), _ptr(ws), ws.numel(), int(partition_tokens), _stream()))
 
 
+def decode_append_attention(
+    out: torch.Tensor,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    key_cache: Union[int, torch.Tensor],
+    value_cache: Union[int, torch.Tensor],
+    num_kv_heads: int,
+    scale: float,
+    seq_lens: Union[torch.Tensor, Sequence[int]],
+    max_seq_len: int,
+    alibi_slopes: Optional[torch.Tensor],
+    slot_mapping: torch.Tensor,
+    partition_tokens: int = 0,
+) -> None:
+    """One launch for the two calls a decode step makes per layer, ``reshape_and_cache`` then
+    ``paged_attention_v1`` (vllm/attention/backends/xformers.py:310-312 and :357-371): ``key`` /
+    ``value`` hold one new row per sequence, ``seq_lens`` counts it, the row lands at position
+    ``seq_lens[b] - 1`` of sequence b's ranges and attention runs over all ``seq_lens[b]`` rows.
+    ``seq_lens`` is an int32 GPU tensor, or a host sequence of at most 512 ints (then nothing is
+    uploaded).  bf16 cache only.  No counterpart as a single op in the reference."""
+    _require_cuda(out, query, key, value, slot_mapping)
+    num_seqs, num_heads, head_size = query.shape
+    if not out.is_contiguous():
+        raise _C.VtkvError(_C.EINVAL, "out must be contiguous")
+    if slot_mapping.dtype != torch.int64:
+        raise _C.VtkvError(_C.EINVAL, "slot_mapping must be int64")
+    key = key.view(-1, num_kv_heads, head_size)
+    value = value.view(-1, num_kv_heads, head_size)
+    if key.shape[0] != num_seqs or value.shape[0] != num_seqs:
+        raise _C.VtkvError(_C.EINVAL, "key/value must hold one row per sequence")
+    if key.stride(2) != 1 or key.stride(1) != head_size or value.stride(2) != 1 or value.stride(1) != head_size:
+        raise _C.VtkvError(_C.EINVAL, "key/value rows must be contiguous in (head, dim)")
+    if isinstance(seq_lens, torch.Tensor):
+        _require_cuda(seq_lens)
+        if seq_lens.dtype != torch.int32:
+            raise _C.VtkvError(_C.EINVAL, "seq_lens must be int32")
+        dev_lens, host_lens = _ptr(seq_lens), None
+    else:
+        if len(seq_lens) != num_seqs:
+            raise _C.VtkvError(_C.EINVAL, "one sequence length per query row")
+        dev_lens, host_lens = None, (C.c_int32 * num_seqs)(*[int(x) for x in seq_lens])
+    qd = _dt(query)
+    lib = _C.lib()
+    need = lib.vtkv_decode_attention_workspace_bytes(num_seqs, num_heads, head_size, max_seq_len, partition_tokens)
+    ws = _workspace(need, query.device)
+    if alibi_slopes is not None:
+        alibi_slopes = alibi_slopes.to(device=query.device, dtype=torch.float32)
+    _C.check(lib.vtkv_decode_append_attention(
+        _ptr(out), _ptr(query), _ptr(key), _ptr(value), key.stride(0), value.stride(0), _ptr(key_cache),
+        _ptr(value_cache), _ptr(slot_mapping), dev_lens, host_lens, num_seqs, num_heads, num_kv_heads, head_size,
+        query.stride(0), float(scale), int(max_seq_len), _ptr(alibi_slopes), qd, _dt(out), _dt(key), _ptr(ws),
+        ws.numel(), int(partition_tokens), _stream()))
+
+
 def paged_attention_v2(
     out: torch.Tensor,
     exp_sum: Optional[torch.Tensor],

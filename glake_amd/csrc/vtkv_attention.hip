@@ -43,6 +43,7 @@
 // force.  fp32 accumulation, output rounded to bf16 once.  No epsilon is added to the softmax
 // denominator (the CPU twin has none, csrc/cpu/attention.cpp:43-67).
 #include <algorithm>
+#include <cstring>
 #include <mutex>
 #include <vector>
 
@@ -76,6 +77,7 @@ constexpr int kRowBytes = kD * 2;  // bf16 row of one head
 constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
 constexpr int kMinSpan = 4;        // a workgroup takes at least one tile per wave
 constexpr int kDefaultMaxGrid = 4096;  // upper bound of the resident-workgroup grid, sizes the scratch
+constexpr int kInlineLens = 512;       // sequence lengths that fit the kernel argument block
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct AttnParams {
@@ -96,6 +98,15 @@ struct AttnParams {
   int grid;         // workgroups of the streaming kernel
   float scale_log2;  // scale * log2(e) [* k_scale for fp8 K]
   float v_scale;
+  // fused append: the step's new K/V rows, one per sequence, row b at new_k + b * new_k_stride (bytes)
+  const char *new_k, *new_v;
+  int64_t new_k_stride, new_v_stride;
+  int inline_lens;  // sequence lengths come with the kernel arguments instead of from seq_lens
+};
+
+// Sequence lengths passed by value (no upload, no dependent global load at the start of the kernel).
+struct InlineLens {
+  int32_t v[kInlineLens];
 };
 
 __device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
@@ -179,8 +190,16 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // FP8: K and V rows hold one e4m3fn code per element (128 bytes per head row).  They are widened to
 // bf16 in registers (K) or on the way into the LDS tile (V); the per-tensor scales are folded into the
 // logit scale (K) and into the final normalisation (V), so dequantisation costs no multiply per element.
-template <bool ALIBI, bool FP8>
-__global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stream_kernel(AttnParams p) {
+//
+// APPEND: seq_lens count the step's new token, whose K/V row is not in the cache yet but in new_k /
+// new_v.  The rows before it are read from the cache as usual; the new row forms one more tile of its
+// own at the end of the sequence's tile list, loaded from new_k / new_v, and the wave that handles it
+// also stores the row into the cache.  One launch then does reshape_and_cache and attention, and each
+// byte of the new rows is read once.
+template <bool ALIBI, bool FP8, bool APPEND>
+__global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
+    decode_attn_stream_kernel(AttnParams p, InlineLens il) {
+  static_assert(!(FP8 && APPEND), "the fused append copies bf16 rows");
   // wave-private V tiles (4 KiB each); reused at the end of a segment for the cross-wave merge
   // then the merge statistics (1 KiB) and the wave-private K tiles
   __shared__ __attribute__((aligned(16))) char smem[2 * kWaves * kTile * kRowBytes + 1024];
@@ -195,6 +214,12 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stre
   const int G = p.group;
   const int Hkv = p.num_kv_heads;
   const int B = p.num_seqs;
+  auto len_of = [&](int idx) { return p.inline_lens ? il.v[idx] : p.seq_lens[idx]; };
+  // tiles of one kv head of a sequence: its cached rows in 16s, plus the new row's own tile
+  auto tiles_of = [](int len) {
+    if (len <= 0) return 0;
+    return APPEND ? (len - 1 + kTile - 1) / kTile + 1 : (len + kTile - 1) / kTile;
+  };
 
   // ---- exclusive prefix sums of the per-sequence tile counts (every workgroup computes its own copy)
   {
@@ -203,9 +228,9 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stre
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
       const int idx = threadIdx.x * kPer + k;
-      const int len = idx < B ? p.seq_lens[idx] : 0;
+      const int len = idx < B ? len_of(idx) : 0;
       local[k] = sum;
-      sum += len > 0 ? (len + kTile - 1) / kTile : 0;
+      sum += tiles_of(len);
     }
     int incl = sum;  // inclusive scan over the wave
 #pragma unroll
@@ -262,15 +287,22 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stre
   // ---- one segment = the part of the span that lies in one (sequence, kv head)
   while (g_cur < g_end) {
     const int seg_tiles = min(g_end - g_cur, nt_b - tile0);
-    const int seq_len = p.seq_lens[b];
+    const int seq_len = uniform(len_of(b));
+    const int ctx_len = APPEND ? seq_len - 1 : seq_len;                // rows read from the cache
+    const bool has_new = APPEND && tile0 + seg_tiles == nt_b;          // the segment ends with the new row's tile
     const int seg_start = tile0 * kTile;                               // first row of the segment
-    const int seg_end = min(seq_len, (tile0 + seg_tiles) * kTile);     // one past its last row
+    const int seg_end = min(ctx_len, (tile0 + seg_tiles) * kTile);     // one past its last cached row
 
     // the tables hold plain integers: say explicitly that they are global-memory addresses, otherwise
     // the loads become flat loads that also count on the LDS wait counter and defeat the prefetch
     const int64_t slot = p.slot_ids[b];
     gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
     gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
+    gptr nk_base = k_base, nv_base = v_base;
+    if (APPEND) {
+      nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kvh * kRowBytes;
+      nv_base = (gptr)(uintptr_t)p.new_v + (int64_t)b * p.new_v_stride + kvh * kRowBytes;
+    }
 
     // B operand of S^T = K.Q^T: for MFMA step ks lane (n, g) holds the eight q[head n][d] whose K
     // elements the lane's 16-byte K operand pieces hold: d = 32*ks + 8*g + j for bf16 rows; for fp8 rows one
@@ -299,13 +331,15 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stre
     // The segment's tiles are dealt round-robin to the four waves: this wave owns tiles wave, wave+4, ...
     // Only the last tile of a sequence can be ragged; its missing rows are redirected to the last valid
     // row (their logits are masked) so no lane reads past the mapped part of a range.
-    const int n_tiles = seg_tiles;
-    const int my_tiles = (n_tiles - wave + kWaves - 1) / kWaves;
-    const int valid_last = seg_end - (seg_start + (n_tiles - 1) * kTile);  // rows in the last tile, 1..16
+    const int n_tiles = seg_tiles - (has_new ? 1 : 0);  // tiles of cached rows; the new row's tile comes last
+    const int my_tiles = (seg_tiles - wave + kWaves - 1) / kWaves;
+    // rows in the last tile of cached rows, 1..16
+    const int valid_last = n_tiles > 0 ? seg_end - (seg_start + (n_tiles - 1) * kTile) : kTile;
     // per-lane byte offsets inside a K or V tile: load j of a lane takes row 4j+g, piece n, i.e. four
     // whole rows per load (fp8 rows are 128 bytes: a load then covers eight rows, lane l takes row
     // 8j + l/8, piece l%8).
     uint32_t t_off[kLoads], t_off_last[kLoads];
+    const uint32_t t_off_new = n * 16;  // the new row's tile: every row slot holds the one new row
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       const int row = FP8 ? 8 * j + (lane >> 3) : 4 * j + g;
@@ -317,24 +351,40 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stre
     // Loads of the i-th tile of this wave.  Always issued, never predicated, so the wait counters the
     // compiler derives are exact; past the wave's last tile every lane loads the segment's first 16
     // bytes instead (one cache line per load, not consumed).
-    auto load_tile = [&](gptr base, int i, u32x4 *regs) {
+    auto load_tile = [&](gptr base, gptr new_base, int i, u32x4 *regs) {
       const bool live = i < my_tiles;
       const int tile = wave + kWaves * i;
       const bool last = tile == n_tiles - 1;
-      // (a mask, not a select: selects here end up as branches around separate copies of the loads)
-      const uint32_t mask = uniform(live ? ~0u : 0u);
+      const bool is_new = APPEND && has_new && live && tile == seg_tiles - 1;
+      // (masks, not selects: selects here end up as branches around separate copies of the loads)
+      const uint32_t mask = uniform(live && !is_new ? ~0u : 0u);
+      const uint32_t mask_new = uniform(is_new ? ~0u : 0u);
       const int64_t row0 = (int64_t)((uint32_t)(seg_start + tile * kTile) & mask) * row_stride;
+      gptr src = base;
+      if (APPEND) src = (gptr)((uintptr_t)base + (((uintptr_t)new_base - (uintptr_t)base) & (uintptr_t)(int64_t)(int32_t)mask_new));  // base or new_base
 #pragma unroll
-      for (int j = 0; j < kLoads; ++j)
-        regs[j] = __builtin_nontemporal_load((gvec)(base + row0 + ((last ? t_off_last[j] : t_off[j]) & mask)));
+      for (int j = 0; j < kLoads; ++j) {
+        uint32_t off = (last ? t_off_last[j] : t_off[j]) & mask;
+        if (APPEND) off |= t_off_new & mask_new;
+        regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off));
+      }
     };
-    auto load_k = [&](int i, u32x4 *kr) { load_tile(k_base, i, kr); };
-    auto load_v = [&](int i, u32x4 *vr) { load_tile(v_base, i, vr); };
+    auto load_k = [&](int i, u32x4 *kr) { load_tile(k_base, nk_base, i, kr); };
+    auto load_v = [&](int i, u32x4 *vr) { load_tile(v_base, nv_base, i, vr); };
 
     // one 16-row tile: logits, online softmax update, P.V
     auto consume = [&](int i, u32x4 *kreg, u32x4 *vreg) {
       const int tile = wave + kWaves * i;
-      const int t0 = seg_start + tile * kTile;
+      const bool is_new = APPEND && has_new && tile == seg_tiles - 1;
+      const int t0 = is_new ? seq_len - 1 : seg_start + tile * kTile;                  // position of the tile's row 0
+      const int valid = is_new ? 1 : (tile == n_tiles - 1 ? valid_last : kTile);       // rows that count
+      if (APPEND && is_new && g == 0) {
+        // lanes 0..15 hold the sixteen 16-byte pieces of the new K and V rows: append them to the cache
+        typedef __attribute__((address_space(1))) u32x4 *gvec_rw;
+        const int64_t dst = (int64_t)(seq_len - 1) * row_stride + n * 16;
+        *(gvec_rw)((uintptr_t)k_base + dst) = kreg[0];
+        *(gvec_rw)((uintptr_t)v_base + dst) = vreg[0];
+      }
       // S^T[row, head] = sum_d K[row, d] q[head, d]
       f32x4 s = {0.f, 0.f, 0.f, 0.f};
       // K tile through LDS: in as loaded, out as A operand (lane (n, g): row n, bytes [16g, +16) of
@@ -382,10 +432,10 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads) decode_attn_stre
         x[r] = s[r] * p.scale_log2;
         if (ALIBI) x[r] += slope_log2 * (float)(t0 + 4 * g + r - seq_len + 1);
       }
-      if (tile == n_tiles - 1 && valid_last < kTile) {  // wave-uniform: only a sequence's ragged last tile
+      if (valid < kTile) {  // wave-uniform: only a sequence's ragged last tile, or the new row's tile
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (4 * g + r >= valid_last) x[r] = -INFINITY;
+          if (4 * g + r >= valid) x[r] = -INFINITY;
       }
       const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
       const float m_new = fmaxf(m_run, tmax);
@@ -592,7 +642,7 @@ KernelTimer g_timer;
 struct Residency {
   std::mutex mu;
   int device = -1;
-  int grid[4] = {0, 0, 0, 0};
+  int grid[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 };
 Residency g_res;
 
@@ -626,29 +676,21 @@ int64_t fixed_span_grid(int num_seqs, int num_kv_heads_bound, int max_seq_len, i
   return (tiles + span - 1) / span;
 }
 
-}  // namespace
-
-extern "C" {
-
-int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_seq_len,
-                                              int partition_tokens) {
-  if (num_seqs <= 0 || num_heads <= 0 || head_size <= 0 || max_seq_len <= 0) return 0;
-  const int64_t grid = partition_tokens >= kTile ? fixed_span_grid(num_seqs, num_heads, max_seq_len, partition_tokens)
-                                                 : kDefaultMaxGrid;
-  const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
-  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes;
-}
-
-int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
-                          const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
-                          int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
-                          const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
-                          float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
-                          void *stream) {
-  VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids && seq_lens, "null argument");
+// Shared by both entry points.  new_key == nullptr: attention only.
+int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
+                   const int32_t *seq_lens, const int32_t *host_seq_lens, int num_seqs, int num_heads,
+                   int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                   const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale, float v_scale,
+                   void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream, const void *new_key,
+                   const void *new_value, int64_t key_stride, int64_t value_stride) {
+  const bool append = new_key != nullptr;
+  VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids, "null argument");
+  VTKV_REQUIRE((seq_lens != nullptr) != (host_seq_lens != nullptr), "pass either device or host sequence lengths");
   VTKV_REQUIRE(num_seqs >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
   VTKV_REQUIRE(num_seqs <= kMaxSeqs, "at most %d sequences per call, got %d", kMaxSeqs, num_seqs);
+  VTKV_REQUIRE(!host_seq_lens || num_seqs <= kInlineLens, "at most %d sequence lengths can be passed from the host, got %d",
+               kInlineLens, num_seqs);
   VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
   VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
   VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
@@ -664,20 +706,36 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                "a sequence range of %d rows exceeds 2 GiB", max_seq_len);
   VTKV_REQUIRE(partition_tokens == 0 || (partition_tokens >= kWaves * kTile && partition_tokens % kTile == 0),
                "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
+  if (append) {
+    VTKV_REQUIRE(new_value != nullptr, "null argument");
+    VTKV_REQUIRE(kv_dtype == VTKV_BF16, "the fused append needs a bf16 cache (use vtkv_reshape_and_cache for fp8)");
+    const int64_t row = (int64_t)num_kv_heads * head_size;
+    VTKV_REQUIRE(key_stride >= row && value_stride >= row && key_stride % 8 == 0 && value_stride % 8 == 0 &&
+                     (uintptr_t)new_key % 16 == 0 && (uintptr_t)new_value % 16 == 0,
+                 "key/value rows must be 16-byte aligned and at least num_kv_heads*head_size apart");
+  }
   if (num_seqs == 0) return VTKV_OK;
 
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   const bool alibi = alibi_slopes != nullptr;
+  // kernel variant: bit 0 fp8, bit 1 alibi, 4 + alibi for the fused append
+  const int variant = append ? 4 + (alibi ? 1 : 0) : (alibi ? 2 : 0) + (fp8 ? 1 : 0);
+  void (*kernel)(AttnParams, InlineLens) = nullptr;
+  switch (variant) {
+    case 0: kernel = decode_attn_stream_kernel<false, false, false>; break;
+    case 1: kernel = decode_attn_stream_kernel<false, true, false>; break;
+    case 2: kernel = decode_attn_stream_kernel<true, false, false>; break;
+    case 3: kernel = decode_attn_stream_kernel<true, true, false>; break;
+    case 4: kernel = decode_attn_stream_kernel<false, false, true>; break;
+    default: kernel = decode_attn_stream_kernel<true, false, true>; break;
+  }
   int64_t grid;
   if (partition_tokens > 0) {
-    grid = fixed_span_grid(num_seqs, num_kv_heads, max_seq_len, partition_tokens);
+    // (the fused append adds one tile per sequence and kv head)
+    grid = fixed_span_grid(num_seqs, num_kv_heads, max_seq_len + (append ? kTile : 0), partition_tokens);
     VTKV_REQUIRE(grid <= (1ll << 24), "partition_tokens %d gives %lld workgroups", partition_tokens, (long long)grid);
   } else {
-    int g = 0;
-    if (alibi && fp8) g = resident_grid(decode_attn_stream_kernel<true, true>, 3);
-    else if (alibi) g = resident_grid(decode_attn_stream_kernel<true, false>, 2);
-    else if (fp8) g = resident_grid(decode_attn_stream_kernel<false, true>, 1);
-    else g = resident_grid(decode_attn_stream_kernel<false, false>, 0);
+    const int g = resident_grid(kernel, variant);
     if (g <= 0) return vtkv::fail(VTKV_EHIP, "cannot query the kernel's occupancy");
     grid = g;
   }
@@ -713,6 +771,13 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   // x = code * scale: the K scale multiplies every logit, the V scale the whole output
   p.scale_log2 = scale * kLog2e * (fp8 ? k_scale : 1.f);
   p.v_scale = fp8 ? v_scale : 1.f;
+  p.new_k = (const char *)new_key;
+  p.new_v = (const char *)new_value;
+  p.new_k_stride = key_stride * 2;
+  p.new_v_stride = value_stride * 2;
+  p.inline_lens = host_seq_lens != nullptr;
+  InlineLens il;
+  if (host_seq_lens) memcpy(il.v, host_seq_lens, (size_t)num_seqs * sizeof(int32_t));
 
   hipStream_t st = (hipStream_t)stream;
   const bool timed = g_timer.on && g_timer.calls < kTimedCalls;
@@ -726,15 +791,7 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
     ev = &g_timer.ev[3 * g_timer.calls];
     VTKV_HIP(hipEventRecord(ev[0], st));
   }
-  const dim3 grid3((unsigned)grid), block(kThreads);
-  if (alibi && fp8)
-    hipLaunchKernelGGL((decode_attn_stream_kernel<true, true>), grid3, block, 0, st, p);
-  else if (alibi)
-    hipLaunchKernelGGL((decode_attn_stream_kernel<true, false>), grid3, block, 0, st, p);
-  else if (fp8)
-    hipLaunchKernelGGL((decode_attn_stream_kernel<false, true>), grid3, block, 0, st, p);
-  else
-    hipLaunchKernelGGL((decode_attn_stream_kernel<false, false>), grid3, block, 0, st, p);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, p, il);
   if (timed) VTKV_HIP(hipEventRecord(ev[1], st));
   hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
   if (timed) {
@@ -743,6 +800,45 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   }
   VTKV_HIP(hipGetLastError());
   return VTKV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_seq_len,
+                                              int partition_tokens) {
+  if (num_seqs <= 0 || num_heads <= 0 || head_size <= 0 || max_seq_len <= 0) return 0;
+  const int64_t grid = partition_tokens >= kTile
+                           ? fixed_span_grid(num_seqs, num_heads, max_seq_len + kTile, partition_tokens)
+                           : kDefaultMaxGrid;
+  const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
+  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes;
+}
+
+int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                          const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
+                          int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                          const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                          float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
+                          void *stream) {
+  VTKV_REQUIRE(seq_lens, "null argument");
+  return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, nullptr, num_seqs, num_heads, num_kv_heads,
+                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
+                        v_scale, workspace, workspace_bytes, partition_tokens, stream, nullptr, nullptr, 0, 0);
+}
+
+int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,
+                                 int64_t value_stride, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                                 const int64_t *slot_ids, const int32_t *seq_lens, const int32_t *host_seq_lens,
+                                 int num_seqs, int num_heads, int num_kv_heads, int head_size, int64_t q_stride,
+                                 float scale, int max_seq_len, const float *alibi_slopes, int q_dtype, int out_dtype,
+                                 int kv_dtype, void *workspace, int64_t workspace_bytes, int partition_tokens,
+                                 void *stream) {
+  VTKV_REQUIRE(key && value, "null argument");
+  return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, host_seq_lens, num_seqs, num_heads, num_kv_heads,
+                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, 1.f, 1.f,
+                        workspace, workspace_bytes, partition_tokens, stream, key, value, key_stride, value_stride);
 }
 
 int vtkv_set_kernel_timing(int on) {

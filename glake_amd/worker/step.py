@@ -50,12 +50,16 @@ class DecodeStepPlan:
     (``vtkv_extend_kv_cache_batch``, ``vtkv_reshape_and_cache``, ``vtkv_decode_attention``); what the
     plan saves is per-call Python: argument arrays, the device tables and the pinned staging ring are
     made once, the bookkeeping writes its offsets straight into pinned memory, and both metadata arrays
-    travel in one asynchronous copy.  Build a new plan when the set of running sequences changes.
+    travel in one asynchronous copy.  With a bf16 cache and ``fused=True`` the append and the attention
+    are one launch (``vtkv_decode_append_attention``) and, up to 512 sequences, the lengths travel with the
+    kernel arguments, so a step is two kernels (attention and its merge) and no copy.  Build a new plan
+    when the set of running sequences changes.
     """
 
     def __init__(self, segments: Sequence, slot_ids: Sequence[int], key_cache, value_cache, num_heads: int,
                  num_kv_heads: int, head_size: int, scale: float, kv_cache_dtype: str = "auto", k_scale: float = 1.0,
-                 v_scale: float = 1.0, model_dtype: torch.dtype = torch.bfloat16, device=None, ring: int = 128):
+                 v_scale: float = 1.0, model_dtype: torch.dtype = torch.bfloat16, device=None, ring: int = 128,
+                 fused: bool = True):
         import ctypes as C
 
         import numpy as np
@@ -101,6 +105,9 @@ class DecodeStepPlan:
         self._ws = ops._workspace(need, self.device)
         self._ws_p, self._ws_n = C.c_void_p(self._ws.data_ptr()), self._ws.numel()
         self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
+        self.fused = bool(fused) and self._kv_dt == _C.BF16 and self._src_dt == _C.BF16
+        self._inline = self.fused and n <= 512
+        self._host_lens_p = [C.c_void_p(self._stage[i].data_ptr() + 8 * n) for i in range(ring)]
 
     def run(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, out: torch.Tensor,
             alibi_slopes=None) -> int:
@@ -119,23 +126,41 @@ class DecodeStepPlan:
         lens += 1
         max_len = int(lens.max())
         stream = C_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        self._row = (i + 1) % self._ring
+        self.seq_lens = lens
+        out_dt = self._C.F32 if out.dtype == torch.float32 else self._C.BF16
+        alibi_p = None if alibi_slopes is None else C_void_p(alibi_slopes.data_ptr())
+        if self._inline:
+            # nothing on the GPU reads the staging row: the lengths are copied into the kernel arguments
+            check(lib.vtkv_decode_append_attention(
+                C_void_p(out.data_ptr()), C_void_p(query.data_ptr()), C_void_p(key.data_ptr()),
+                C_void_p(value.data_ptr()), key.stride(0), value.stride(0), self._k_table, self._v_table,
+                self._slot_p, None, self._host_lens_p[i], n, self.num_heads, self.num_kv_heads, self.head_size,
+                query.stride(0), self.scale, max_len, alibi_p, self._src_dt, out_dt, self._kv_dt, self._ws_p,
+                self._ws_n, 0, stream))
+            return max_len
         check(lib.vtkv_memcpy_h2d_async(self._meta_addr, self._row_p[i], 12 * n, stream))
         if i == half - 1 or i == self._ring - 1:
             h = 0 if i == half - 1 else 1
             self._events[h].record()
             self._recorded[h] = True
-        self._row = (i + 1) % self._ring
-        self.seq_lens = lens
+        if self.fused:
+            check(lib.vtkv_decode_append_attention(
+                C_void_p(out.data_ptr()), C_void_p(query.data_ptr()), C_void_p(key.data_ptr()),
+                C_void_p(value.data_ptr()), key.stride(0), value.stride(0), self._k_table, self._v_table,
+                self._slot_p, self._lens_p, None, n, self.num_heads, self.num_kv_heads, self.head_size,
+                query.stride(0), self.scale, max_len, alibi_p, self._src_dt, out_dt, self._kv_dt, self._ws_p,
+                self._ws_n, 0, stream))
+            return max_len
         kstride = key.stride(0)
         vstride = value.stride(0)
         check(lib.vtkv_reshape_and_cache(
             C_void_p(key.data_ptr()), C_void_p(value.data_ptr()), self._k_table, self._v_table, self._offs_p,
             self._slot_p, None, None, n, 1, self.num_kv_heads, self.head_size, kstride, vstride, self._src_dt,
             self._kv_dt, self.k_scale, self.v_scale, stream))
-        out_dt = self._C.F32 if out.dtype == torch.float32 else self._C.BF16
         check(lib.vtkv_decode_attention(
             C_void_p(out.data_ptr()), C_void_p(query.data_ptr()), self._k_table, self._v_table, self._slot_p,
             self._lens_p, n, self.num_heads, self.num_kv_heads, self.head_size, query.stride(0), self.scale, max_len,
-            None if alibi_slopes is None else C_void_p(alibi_slopes.data_ptr()), self._src_dt, out_dt, self._kv_dt,
+            alibi_p, self._src_dt, out_dt, self._kv_dt,
             self.k_scale, self.v_scale, self._ws_p, self._ws_n, 0, stream))
         return max_len

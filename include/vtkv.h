@@ -219,6 +219,24 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                           float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
                           void *stream);
 
+/* reshape_and_cache (decode form: one new row per sequence) fused into the attention launch; replaces
+ * the pair of calls at vllm/attention/backends/xformers.py:310-312 and :357-371 for a decode step.
+ * seq_lens[b] counts the new token: key[b] / value[b] ([num_seqs, num_kv_heads, head_size] bf16, row strides
+ * in elements) are appended at row seq_lens[b]-1 of sequence b's ranges, which must be mapped that far, and
+ * attention runs over all seq_lens[b] rows.  The cache contents and the result are those of
+ * vtkv_reshape_and_cache followed by vtkv_decode_attention (the result up to fp32 summation order).
+ * Lengths come either from the device (seq_lens) or from the host (host_seq_lens, at most 512 sequences;
+ * copied into the kernel arguments during the call, so no upload is needed and the array may be reused
+ * at once); pass NULL for the other.  kv_dtype must be VTKV_BF16.  Other arguments as for
+ * vtkv_decode_attention. */
+int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,
+                                 int64_t value_stride, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                                 const int64_t *slot_ids, const int32_t *seq_lens, const int32_t *host_seq_lens,
+                                 int num_seqs, int num_heads, int num_kv_heads, int head_size, int64_t q_stride,
+                                 float scale, int max_seq_len, const float *alibi_slopes, int q_dtype, int out_dtype,
+                                 int kv_dtype, void *workspace, int64_t workspace_bytes, int partition_tokens,
+                                 void *stream);
+
 /* Benchmark aid without a counterpart in the reference (its kernel benchmark times from the host,
  * benchmarks/kernels/benchmark_paged_attention.py:147-157): while switched on, each vtkv_decode_attention
  * call (up to 1024 of them) records HIP events around its kernels on the caller's stream without waiting

@@ -1,0 +1,126 @@
+"""The fused decode-step launch (vtkv_decode_append_attention, through the C ABI): the new K/V rows
+land in the cache bit for bit where reshape_and_cache would put them, and the attention output over
+old rows + new row is within 2e-3 abs + 2e-3 rel of the oracle (fp32 output, see test_gpu_attention.py
+for why the comparison is made before the final bf16 store), for lengths from the host (kernel
+arguments) and from the device."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from_bits
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+
+
+def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partition_tokens=0, d=128):
+    """seq_lens count the new token."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(seed)
+    b = len(seq_lens)
+    num_slots = b + 2
+    slots = rng.permutation(num_slots)[:b]
+    row = hkv * d * 2
+    gpu = GpuSeqs(vmm, num_slots, hkv, d, 2, max(seq_lens) + 1)
+    k_host, v_host = {}, {}
+    for i, t in enumerate(seq_lens):
+        s = int(slots[i])
+        k_host[s], v_host[s] = bf16_randn(rng, (t - 1, hkv, d)), bf16_randn(rng, (t - 1, hkv, d))
+        gpu.upload(s, k_host[s], v_host[s])
+    # the step's bookkeeping maps the chunk a new row needs, as in the engine
+    used = vmm.extend_kv_cache_batch(None, None, [int(s) for s in slots], [row] * b, [gpu.segs[int(s)] for s in slots],
+                                     [0] * b, row, True)
+    assert used == [(t - 1) * row for t in seq_lens]
+    q = bf16_randn(rng, (b, hq, d))
+    nk, nv = bf16_randn(rng, (b, hkv, d)), bf16_randn(rng, (b, hkv, d))
+    slopes = rng.standard_normal(hq).astype(np.float32) if alibi else None
+    scale = float(d) ** -0.5
+
+    kt, vt = gpu.table_tensors()
+    out32 = torch.empty(b, hq, d, dtype=torch.float32, device="cuda")
+    out16 = torch.empty(b, hq, d, dtype=torch.bfloat16, device="cuda")
+    q_t, nk_t, nv_t = (torch_bf16_from_bits(x) for x in (q, nk, nv))
+    lens_arg = list(seq_lens) if lens_from == "host" else torch.tensor(seq_lens, dtype=torch.int32, device="cuda")
+    slot_t = torch.tensor(slots, dtype=torch.int64, device="cuda")
+    al_t = None if slopes is None else torch.from_numpy(slopes).cuda()
+    for o in (out32, out16):  # the second call appends the same rows again: idempotent
+        ops.decode_append_attention(o, q_t, nk_t, nv_t, kt, vt, hkv, scale, lens_arg, max(seq_lens), al_t, slot_t,
+                                    partition_tokens=partition_tokens)
+    torch.cuda.synchronize()
+
+    # cache: old rows untouched, new row in place
+    full_k = [np.zeros((1, hkv, d), np.uint16)] * num_slots
+    full_v = [np.zeros((1, hkv, d), np.uint16)] * num_slots
+    for i, t in enumerate(seq_lens):
+        s = int(slots[i])
+        full_k[s] = np.concatenate([k_host[s], nk[i:i + 1]])
+        full_v[s] = np.concatenate([v_host[s], nv[i:i + 1]])
+        assert np.array_equal(gpu.download(s, t * row, which="k", dtype=np.uint16), full_k[s].reshape(-1)), f"K of seq {i}"
+        assert np.array_equal(gpu.download(s, t * row, which="v", dtype=np.uint16), full_v[s].reshape(-1)), f"V of seq {i}"
+    cache = O.VTensorCache(full_k, full_v, slots, hkv, d)
+    expect32 = O.paged_attention_v1(O.bf16_to_f32(q), cache, scale, seq_lens, slopes)
+    got = out32.cpu().numpy()
+    gpu.close()
+    assert np.array_equal(bits_from_torch_bf16(out16), O.f32_to_bf16(got)), "bf16 output is not RNE(fp32 output)"
+    err = np.abs(got - expect32)
+    bound = TOL + TOL * np.abs(expect32)
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert np.all(err <= bound), (f"max err {err.max():.3e} at (seq, head, d)={worst}: got {got[worst]!r} "
+                                  f"want {expect32[worst]!r}, len {seq_lens[worst[0]]}")
+    return got
+
+
+EDGE = [1, 2, 3, 16, 17, 18, 33, 64, 65, 66, 256, 257, 258, 1025, 1026]
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (8, 8), (16, 1)])
+@pytest.mark.parametrize("lens_from", ["host", "device"])
+def test_edge_lengths(gpu_pool, hq, hkv, lens_from):
+    run_case(gpu_pool, 11, EDGE, hq, hkv, lens_from=lens_from)
+
+
+def test_config2_shape(gpu_pool):
+    rng = np.random.default_rng(1001)
+    run_case(gpu_pool, 1001, rng.integers(512, 4097, 64).tolist(), 32, 8)
+
+
+def test_alibi(gpu_pool):
+    run_case(gpu_pool, 5, [1, 34, 401, 1000], 32, 8, alibi=True)
+
+
+@pytest.mark.parametrize("pt", [64, 512])
+def test_fixed_partitions_agree(gpu_pool, pt):
+    lens = [700, 65, 1, 1500, 2049, 17]
+    got = run_case(gpu_pool, 7, lens, 32, 8, partition_tokens=pt)
+    base = run_case(gpu_pool, 7, lens, 32, 8)
+    assert np.abs(got - base).max() <= 2e-3
+
+
+def test_long_sequence_many_workgroups_per_segment(gpu_pool):
+    # one sequence spread over many workgroups plus short ones: the new row's tile is a segment of its own for some
+    run_case(gpu_pool, 9, [40000, 1, 2, 5000], 32, 8, lens_from="device")
+
+
+def test_rejects_fp8_cache_and_too_many_host_lengths(gpu_pool):
+    import ctypes as C
+
+    import torch
+
+    from glake_amd import _C
+
+    lib = _C.lib()
+    t = torch.zeros(1024, dtype=torch.uint8, device="cuda")
+    p = C.c_void_p(t.data_ptr())
+    host = (C.c_int32 * 600)(*([1] * 600))
+    ws = torch.empty(lib.vtkv_decode_attention_workspace_bytes(600, 8, 128, 16, 0), dtype=torch.uint8, device="cuda")
+    rc = lib.vtkv_decode_append_attention(p, p, p, p, 128, 128, p, p, p, None, host, 600, 8, 1, 128, 1024, 1.0, 16, None,
+                                          _C.BF16, _C.BF16, _C.BF16, C.c_void_p(ws.data_ptr()), ws.numel(), 0, None)
+    assert rc == _C.EINVAL and "512" in _C.last_error()
+    rc = lib.vtkv_decode_append_attention(p, p, p, p, 128, 128, p, p, p, p, None, 1, 8, 1, 128, 1024, 1.0, 16, None,
+                                          _C.BF16, _C.BF16, _C.FP8_E4M3, C.c_void_p(ws.data_ptr()), ws.numel(), 0, None)
+    assert rc == _C.EINVAL and "bf16" in _C.last_error()

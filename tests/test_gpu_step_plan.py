@@ -1,6 +1,6 @@
 """DecodeStepPlan (one call per decode step) against the separate ops and the oracle: the cache bytes
-it appends are exact, its attention output equals the separate ops' bit for bit (same kernels, same
-arguments), and both are within tolerance of the oracle.  The ring of staging rows is lapped several
+it appends are exact, its attention output equals the separate ops' bit for bit when it uses the same
+kernels with the same arguments (unfused), and all outputs are within tolerance of the oracle.  The ring of staging rows is lapped several
 times and one sequence crosses a 2 MiB chunk boundary during the run."""
 import numpy as np
 import pytest
@@ -12,8 +12,8 @@ from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("kv", ["bf16", "fp8"])
-def test_plan_matches_ops_and_oracle(gpu_pool, kv):
+@pytest.mark.parametrize("kv,fused", [("bf16", True), ("bf16", False), ("fp8", False)])
+def test_plan_matches_ops_and_oracle(gpu_pool, kv, fused):
     import torch
 
     from glake_amd import _custom_ops as ops, vmm_allocator as vmm
@@ -48,7 +48,8 @@ def test_plan_matches_ops_and_oracle(gpu_pool, kv):
     slot_ids = list(range(B))
     slot_t = torch.arange(B, dtype=torch.int64, device="cuda")
     plan = DecodeStepPlan(sets[0].segs, slot_ids, tables[0][0], tables[0][1], hq, hkv, d, scale,
-                          kv_cache_dtype=kv_dtype, k_scale=k_scale, v_scale=v_scale, ring=4)
+                          kv_cache_dtype=kv_dtype, k_scale=k_scale, v_scale=v_scale, ring=4, fused=fused)
+    assert plan.fused == fused
     lens = list(ctx)
     for step in range(steps):
         q_bits = bf16_randn(rng, (B, hq, d))
@@ -68,7 +69,10 @@ def test_plan_matches_ops_and_oracle(gpu_pool, kv):
                                torch.tensor(lens, dtype=torch.int32, device="cuda"), 1, max(lens), None, kv_dtype,
                                k_scale, slot_t, v_scale=v_scale)
         torch.cuda.synchronize()
-        assert torch.equal(out_plan, out_ops), f"step {step}: plan and ops outputs differ"
+        if fused:  # other tiling of the rows, so another fp32 summation order
+            assert (out_plan - out_ops).abs().max().item() <= 2e-3
+        else:
+            assert torch.equal(out_plan, out_ops), f"step {step}: plan and ops outputs differ"
         for b in range(B):
             if fp8:
                 nkc = O.fp8_encode(O.bf16_to_f32(nk_bits[b:b + 1]), k_scale)
