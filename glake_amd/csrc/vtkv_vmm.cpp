@@ -11,6 +11,15 @@
 // 222-228); growth in the decode step is done in the calling thread instead of a detached busy-
 // spinning thread signalling through POSIX shared memory (vmm_allocator.cpp:40-72,113-151);
 // failed growth leaves the segment unchanged instead of half-mapped; ranges are freed on destroy.
+//
+// Unmapping is lazy.  hipMemUnmap costs about 260 us per 2 MiB chunk on this hardware (mapping one
+// costs about 55 us), so a segment that shrinks (preempt, release, swap-out) only gives its chunks
+// up logically: they stay mapped at the top of its ranges as "retired" chunks, count as free, and
+// are physically unmapped when another segment needs them (or when the caller asks with
+// vtkv_pool_trim, e.g. while the GPU is busy).  If the same segment grows again first, as a sequence
+// that is swapped back in or a slot that is reused does, its retired chunks are simply taken back
+// without any call into the driver.
+#include <algorithm>
 #include <mutex>
 #include <unordered_set>
 #include <vector>
@@ -38,6 +47,7 @@ struct Pool {
   int device = -1;
   std::vector<hipMemGenericAllocationHandle_t> free_chunks;
   int64_t total = 0;
+  int64_t retired = 0;  // chunks still mapped at the top of shrunken segments; they count as free
   std::unordered_set<vtkv_segment *> segments;
 };
 Pool g_pool;
@@ -49,7 +59,8 @@ struct vtkv_segment {
   int layer_num = 0;
   int64_t context_max = 0;  // reserved bytes per range
   int64_t expand_bytes = 0; // what release keeps mapped
-  int64_t mapped = 0;       // actual_size: bytes mapped per range
+  int64_t mapped = 0;       // actual_size: bytes mapped per range that belong to the sequence
+  int64_t held = 0;         // bytes physically mapped per range, >= mapped; [mapped, held) is retired
   int64_t used = 0;         // used_size: bytes written per range
   std::vector<char *> k_base, v_base;
   // chunks mapped into layer l's K (resp. V) range, in address order
@@ -61,8 +72,9 @@ using vtkv::kChunk;
 
 namespace {
 
-// Map `n` chunks at offset `at` of every range.  Caller holds the pool mutex and has checked the
-// pool holds 2*layers*n chunks.  On a HIP failure everything mapped by this call is rolled back.
+// Map `n` chunks at offset `held` (== `mapped`: the caller has taken back all retired chunks) of
+// every range.  Caller holds the pool mutex and has checked the free list holds 2*layers*n chunks.
+// On a HIP failure everything mapped by this call is rolled back.
 int map_chunks_locked(vtkv_segment *s, int n) {
   hipMemAccessDesc ad = {};
   ad.location.type = hipMemLocationTypeDevice;
@@ -74,7 +86,7 @@ int map_chunks_locked(vtkv_segment *s, int n) {
   for (int l = 0; l < s->layer_num && err == hipSuccess; ++l) {
     for (int j = 0; j < n && err == hipSuccess; ++j) {
       for (int which = 0; which < 2 && err == hipSuccess; ++which) {
-        char *va = (which ? s->v_base[l] : s->k_base[l]) + s->mapped + (int64_t)j * kChunk;
+        char *va = (which ? s->v_base[l] : s->k_base[l]) + s->held + (int64_t)j * kChunk;
         hipMemGenericAllocationHandle_t h = g_pool.free_chunks.back();
         err = hipMemMap(va, kChunk, 0, h, 0);
         if (err != hipSuccess) break;
@@ -82,6 +94,7 @@ int map_chunks_locked(vtkv_segment *s, int n) {
         auto *list = which ? &s->v_chunks[l] : &s->k_chunks[l];
         list->push_back(h);
         done.push_back({va, h, list});
+        // (one call over several chunks costs the same per chunk: measured 28 us each either way)
         err = hipMemSetAccess(va, kChunk, &ad, 1);
       }
     }
@@ -94,8 +107,47 @@ int map_chunks_locked(vtkv_segment *s, int n) {
     }
     return vtkv::fail(VTKV_EHIP, "mapping a chunk failed: %s", hipGetErrorString(err));
   }
-  s->mapped += (int64_t)n * kChunk;
+  s->held += (int64_t)n * kChunk;
+  s->mapped = s->held;
   return VTKV_OK;
+}
+
+// Physically unmap the retired chunks of `s` at offsets >= max(keep_held, mapped), top down, at most
+// `max_rows` chunk rows (one row = one chunk of every range; < 0: all).  Returns rows unmapped or < 0.
+int64_t trim_segment_locked(vtkv_segment *s, int64_t keep_held, int64_t max_rows) {
+  const int64_t floor_n = std::max(keep_held, s->mapped) / kChunk;
+  int64_t rows = 0;
+  while (s->held / kChunk > floor_n && (max_rows < 0 || rows < max_rows)) {
+    const int64_t top = s->held / kChunk - 1;
+    for (int l = 0; l < s->layer_num; ++l) {
+      for (int which = 0; which < 2; ++which) {
+        auto &list = which ? s->v_chunks[l] : s->k_chunks[l];
+        char *base = which ? s->v_base[l] : s->k_base[l];
+        // one call per mapping: each chunk was mapped on its own
+        VTKV_HIP(hipMemUnmap(base + top * kChunk, kChunk));
+        g_pool.free_chunks.push_back(list.back());
+        list.pop_back();
+      }
+    }
+    s->held -= kChunk;
+    g_pool.retired -= 2ll * s->layer_num;
+    ++rows;
+  }
+  return rows;
+}
+
+// Make the free list hold at least `need` chunks by unmapping retired chunks of other segments.
+int reclaim_locked(int64_t need) {
+  if ((int64_t)g_pool.free_chunks.size() >= need) return VTKV_OK;
+  for (vtkv_segment *o : g_pool.segments) {
+    while (o->held > o->mapped && (int64_t)g_pool.free_chunks.size() < need) {
+      int64_t rc = trim_segment_locked(o, 0, 1);
+      if (rc < 0) return (int)rc;
+    }
+    if ((int64_t)g_pool.free_chunks.size() >= need) return VTKV_OK;
+  }
+  return vtkv::fail(VTKV_ENOMEM, "chunk pool exhausted: need %lld, free %lld", (long long)need,
+                    (long long)g_pool.free_chunks.size());
 }
 
 int expand_locked(vtkv_segment *s, int n) {
@@ -103,29 +155,32 @@ int expand_locked(vtkv_segment *s, int n) {
   if (s->mapped + (int64_t)n * kChunk > s->context_max)
     return vtkv::fail(VTKV_EINVAL, "segment would grow to %lld bytes, beyond its reserved %lld",
                       (long long)(s->mapped + (int64_t)n * kChunk), (long long)s->context_max);
-  const int64_t need = 2ll * s->layer_num * n;
-  if ((int64_t)g_pool.free_chunks.size() < need)
+  // the segment's own retired chunks are still mapped right where it grows: take them back first
+  const int revive = (int)std::min<int64_t>(n, (s->held - s->mapped) / kChunk);
+  const int fresh = n - revive;
+  const int64_t need = 2ll * s->layer_num * fresh;
+  // (its retired chunks beyond `revive` are none when fresh > 0, so reclaiming never touches `s`)
+  if (fresh > 0 && (int64_t)g_pool.free_chunks.size() + g_pool.retired - 2ll * s->layer_num * revive < need)
     return vtkv::fail(VTKV_ENOMEM, "chunk pool exhausted: need %lld, free %lld", (long long)need,
-                      (long long)g_pool.free_chunks.size());
-  return map_chunks_locked(s, n);
+                      (long long)((int64_t)g_pool.free_chunks.size() + g_pool.retired - 2ll * s->layer_num * revive));
+  s->mapped += (int64_t)revive * kChunk;
+  g_pool.retired -= 2ll * s->layer_num * revive;
+  if (fresh == 0) return VTKV_OK;
+  int rc = reclaim_locked(need);
+  if (rc >= 0) rc = map_chunks_locked(s, fresh);
+  if (rc < 0) {  // leave the segment as it was
+    s->mapped -= (int64_t)revive * kChunk;
+    g_pool.retired += 2ll * s->layer_num * revive;
+  }
+  return rc;
 }
 
-// Unmap every chunk at offset >= keep_bytes of every range and return them to the pool.
+// Give up every chunk at offset >= keep_bytes of every range.  The chunks stay mapped (retired)
+// until the pool needs them; see the note at the top of the file.
 int shrink_locked(vtkv_segment *s, int64_t keep_bytes) {
   if (keep_bytes >= s->mapped) return VTKV_OK;
   const int64_t keep_n = keep_bytes / kChunk;
-  for (int l = 0; l < s->layer_num; ++l) {
-    for (int which = 0; which < 2; ++which) {
-      auto &list = which ? s->v_chunks[l] : s->k_chunks[l];
-      char *base = which ? s->v_base[l] : s->k_base[l];
-      // one call per mapping: each chunk was mapped on its own
-      while ((int64_t)list.size() > keep_n) {
-        VTKV_HIP(hipMemUnmap(base + ((int64_t)list.size() - 1) * kChunk, kChunk));
-        g_pool.free_chunks.push_back(list.back());
-        list.pop_back();
-      }
-    }
-  }
+  g_pool.retired += 2ll * s->layer_num * (s->mapped / kChunk - keep_n);
   s->mapped = keep_n * kChunk;
   return VTKV_OK;
 }
@@ -197,7 +252,25 @@ int vtkv_pool_init(int device, int64_t num_chunks) {
 
 int64_t vtkv_pool_free_chunks(void) {
   std::lock_guard<std::mutex> lk(g_pool.mu);
-  return (int64_t)g_pool.free_chunks.size();
+  return (int64_t)g_pool.free_chunks.size() + g_pool.retired;
+}
+
+int64_t vtkv_pool_retired_chunks(void) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  return g_pool.retired;
+}
+
+int64_t vtkv_pool_trim(int64_t max_chunks) {
+  std::lock_guard<std::mutex> lk(g_pool.mu);
+  int64_t chunks = 0;
+  for (vtkv_segment *s : g_pool.segments) {
+    while (s->held > s->mapped && (max_chunks < 0 || chunks < max_chunks)) {
+      int64_t rc = trim_segment_locked(s, 0, 1);
+      if (rc < 0) return rc;
+      chunks += 2ll * s->layer_num * rc;
+    }
+  }
+  return chunks;
 }
 
 int64_t vtkv_pool_total_chunks(void) {
@@ -271,6 +344,7 @@ int vtkv_seg_destroy(vtkv_segment *s) {
   SEG_CHECK(s);
   int rc = shrink_locked(s, 0);
   if (rc < 0) return rc;
+  if (trim_segment_locked(s, 0, -1) < 0) return VTKV_EHIP;
   for (char *p : s->k_base) VTKV_HIP(hipMemAddressFree(p, s->context_max));
   for (char *p : s->v_base) VTKV_HIP(hipMemAddressFree(p, s->context_max));
   g_pool.segments.erase(s);

@@ -36,6 +36,16 @@ def totalBlocks() -> int:
     return int(_C.check(_C.lib().vtkv_pool_total_chunks()))
 
 
+def retiredBlocks() -> int:
+    """Free chunks that are still mapped at the top of a shrunken segment (unmapping is lazy)."""
+    return int(_C.check(_C.lib().vtkv_pool_retired_chunks()))
+
+
+def trim(max_chunks: int = -1) -> int:
+    """Unmap up to ``max_chunks`` retired chunks now (all by default); returns how many."""
+    return int(_C.check(_C.lib().vtkv_pool_trim(int(max_chunks))))
+
+
 def destroy_pool() -> None:
     _C.check(_C.lib().vtkv_pool_destroy())
 

@@ -55,8 +55,18 @@ int64_t vtkv_chunk_bytes(void);
  * Replaces init_physical_handle(num_blocks, device_id) (vmm_allocator.cpp:113-151).
  * May be called again to add chunks. */
 int vtkv_pool_init(int device, int64_t num_chunks);
-/* Free chunks in the pool; replaces showFreeBlocks() (vmm_allocator.cpp:472-474). <0 on error. */
+/* Chunks no sequence owns; replaces showFreeBlocks() (vmm_allocator.cpp:472-474). <0 on error.
+ * Unmapping is lazy: a segment that shrinks (preempt, release, swap-out) keeps its chunks mapped at the
+ * top of its ranges as "retired" chunks, which count as free here; they are unmapped when another
+ * segment needs them, and taken back without a driver call if the same segment grows again first. */
 int64_t vtkv_pool_free_chunks(void);
+/* How many of the free chunks are retired, i.e. still mapped.  No counterpart in the reference. */
+int64_t vtkv_pool_retired_chunks(void);
+/* Unmap retired chunks now, until at least `max_chunks` are unmapped or none is left (< 0: all; whole
+ * rows, i.e. one chunk of every range of a segment, at a time), so that later growth finds them on the
+ * free list; meant for idle moments of the host thread.  Returns the number unmapped, < 0 on error.
+ * No counterpart in the reference (its release path unmaps at once, vmm_allocator.cpp:393-420). */
+int64_t vtkv_pool_trim(int64_t max_chunks);
 /* Chunks ever created and still owned (free + mapped). */
 int64_t vtkv_pool_total_chunks(void);
 /* Release every chunk and every segment's address range.  All segments must have been destroyed. */

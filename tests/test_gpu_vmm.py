@@ -139,3 +139,48 @@ def test_pointer_tables(gpu_pool):
         s.destroy()
     for t in kt + vt:
         t.destroy()
+
+
+def test_lazy_unmap_retire_revive_trim_reclaim(gpu_pool):
+    """A shrinking segment keeps its chunks mapped ("retired", counted as free); the same segment takes
+    them back with their contents, vtkv_pool_trim unmaps them, and another segment's growth reclaims
+    them when the free list runs dry."""
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    vmm.trim()
+    assert vmm.retiredBlocks() == 0
+    free0 = vmm.showFreeBlocks()
+    layers = 2
+    a = vmm.KVcacheSegment(layers, 8 * CHUNK, 0, False)
+    a.expandMultiSegment(3)
+    blob = np.random.default_rng(3).integers(0, 256, 3 * CHUNK, dtype=np.uint8)
+    _C.check(_C.lib().vtkv_memcpy_h2d(a.getValueDevicePtr(1), blob.ctypes.data_as(C.c_void_p), blob.nbytes))
+    a.preempt_seq(0)
+    assert a.actual_size == 0 and vmm.showFreeBlocks() == free0 and vmm.retiredBlocks() == 3 * 2 * layers
+    # revival: same chunks, same place, no driver call; the bytes are still there
+    a.expandMultiSegment(2)
+    assert a.actual_size == 2 * CHUNK and vmm.retiredBlocks() == 1 * 2 * layers
+    back = np.empty(2 * CHUNK, np.uint8)
+    _C.check(_C.lib().vtkv_memcpy_d2h(back.ctypes.data_as(C.c_void_p), a.getValueDevicePtr(1), back.nbytes))
+    assert np.array_equal(back, blob[:2 * CHUNK])
+    # growing past the retired part mixes revived and fresh chunks
+    a.expandMultiSegment(3)
+    assert a.actual_size == 5 * CHUNK and vmm.retiredBlocks() == 0 and vmm.showFreeBlocks() == free0 - 5 * 2 * layers
+    a.preempt_seq(0)
+    assert vmm.retiredBlocks() == 5 * 2 * layers
+    # trim unmaps whole rows (one chunk of every range of a segment)
+    assert vmm.trim(1) == 2 * layers and vmm.retiredBlocks() == 4 * 2 * layers and vmm.showFreeBlocks() == free0
+    # reclaim: b needs more chunks than the free list holds, so a's retired chunks are unmapped for it
+    on_list = vmm.showFreeBlocks() - vmm.retiredBlocks()
+    n = on_list // 2 + 2                                           # 2 chunks per row of a 1-layer segment
+    b = vmm.KVcacheSegment(1, (n + 1) * CHUNK, 0, False)
+    b.expandMultiSegment(n)
+    assert b.actual_size == n * CHUNK and vmm.retiredBlocks() < 4 * 2 * layers
+    assert vmm.showFreeBlocks() == free0 - 2 * n
+    # a can still grow: whatever is left of its retired chunks is revived, the rest is fresh
+    a.expandMultiSegment(1)
+    assert a.actual_size == CHUNK
+    b.destroy()
+    a.destroy()
+    assert vmm.showFreeBlocks() == free0 and vmm.retiredBlocks() == 0
