@@ -61,6 +61,8 @@ def main() -> int:
                     help="plan: DecodeStepPlan (arguments prepared once); ops: the separate reference-style op calls")
     ap.add_argument("--unfused", action="store_true",
                     help="plan path: separate reshape_and_cache and attention launches instead of the fused one")
+    ap.add_argument("--merge", default="auto", choices=["auto", "fused", "separate"],
+                    help="where the attention's partial results are merged (auto: the library decides per call)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -75,6 +77,7 @@ def main() -> int:
     from glake_amd.worker.cache_engine import CacheEngine
 
     cfg = CONFIGS[args.config]
+    _C.check(_C.lib().vtkv_set_fused_merge({"auto": -1, "fused": 1, "separate": 0}[args.merge]))
     B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
     K, W = args.steps, args.warmup
     torch.cuda.set_device(0)

@@ -56,14 +56,15 @@ def _require_cuda(*tensors) -> None:
             raise _C.VtkvError(_C.EINVAL, "tensor must live on the GPU")
 
 
-# scratch for split-K partials, grown on demand, one per device
+# scratch for the attention's partial results, grown on demand, one per device.  The library wants it
+# zero-filled before its first use (it keeps arrival counters there that it resets itself).
 _workspaces = {}
 
 
 def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
     ws = _workspaces.get(device)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[device] = ws
     return ws
 

@@ -77,6 +77,7 @@ constexpr int kRowBytes = kD * 2;  // bf16 row of one head
 constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
 constexpr int kMinSpan = 4;        // a workgroup takes at least one tile per wave
 constexpr int kDefaultMaxGrid = 4096;  // upper bound of the resident-workgroup grid, sizes the scratch
+constexpr int kMaxKvHeads = 64;        // kv heads per call (sizes the arrival counters)
 constexpr int kInlineLens = 512;       // sequence lengths that fit the kernel argument block
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -90,6 +91,10 @@ struct AttnParams {
   float *part_max;  // [slots][G]   (log2 units)
   float *part_sum;  // [slots][G]
   int32_t *cum_tiles;  // [num_seqs + 1]
+  // [num_seqs * num_kv_heads] arrivals per (sequence, kv head) when the merge is done in the streaming
+  // kernel (fused_merge); zero between launches: the workgroup that arrives last resets its counter
+  uint32_t *seg_count;
+  int fused_merge;
   void *out;           // [B,Hq,D] bf16, or fp32 when out_f32
   int out_f32;
   int64_t q_stride;
@@ -179,6 +184,16 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(unsigned lo, unsigned hi) {
   return r;
 }
 
+// Loads and stores that are coherent across the whole device (they go past the per-XCD L2), for the
+// few values that workgroups hand to each other inside one launch.  A device-scope fence would also
+// do, but it writes back and invalidates a whole L2 each time, which costs far more than these.
+__device__ __forceinline__ void store_device_coherent(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_device_coherent(const float *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
 // Tiles per workgroup span, the same rule in both kernels.
@@ -205,6 +220,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
   __shared__ __attribute__((aligned(16))) char smem[2 * kWaves * kTile * kRowBytes + 1024];
   __shared__ int s_cum[kMaxSeqs + 1];  // s_cum[b] = tiles (of one kv head) of sequences before b
   __shared__ int s_wave_tot[kWaves];
+  __shared__ int s_last;  // this workgroup delivered the last piece of the current (sequence, kv head)
 
   const int lane = threadIdx.x & 63;
   // everything that decides control flow and base addresses is kept wave-uniform (scalar registers)
@@ -545,6 +561,18 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
     const float f = __builtin_amdgcn_exp2f(m_run - m_wg);  // 0 for a wave that saw no row
     // slot of this (workgroup, segment): both indices only grow along the tile order, so the sum is unique
     const int64_t slot_idx = (int64_t)blockIdx.x + (int64_t)b * Hkv + kvh;
+    // workgroups w0..w1 hold the pieces of this (sequence, kv head): its tiles are [first, first + nt_b)
+    // of the global order
+    const int first_tile = uniform(s_cum[b]) * Hkv + kvh * nt_b;
+    const int w0 = first_tile / span, w1 = (first_tile + nt_b - 1) / span;
+    const bool whole = p.fused_merge && w0 == w1;  // no other workgroup: the result is final
+    auto store_out = [&](int head, int d, float r) {
+      const int64_t oi = ((int64_t)b * p.num_heads + kvh * G + head) * kD + d;
+      if (p.out_f32)
+        reinterpret_cast<float *>(p.out)[oi] = r;
+      else
+        reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
+    };
     // G <= 8 fits the 16 KiB; for larger groups the merge runs in two halves of 8 heads
     for (int h0 = 0; h0 < G; h0 += 8) {
       if (h0 > 0) __syncthreads();
@@ -567,11 +595,71 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
           lsum += sm_l[w * 16 + head] * __builtin_amdgcn_exp2f(sm_m[w * 16 + head] - mw);
           o += sm_o[(w * 8 + hh) * kD + d];
         }
+        if (whole) {
+          store_out(head, d, o / lsum * p.v_scale);
+          continue;
+        }
         const int64_t pidx = slot_idx * G + head;
-        p.part_out[pidx * kD + d] = o / lsum;
-        if (d == 0) {
-          p.part_max[pidx] = mw;  // log2 units
-          p.part_sum[pidx] = lsum;
+        if (p.fused_merge) {
+          store_device_coherent(&p.part_out[pidx * kD + d], o / lsum);
+          if (d == 0) {
+            store_device_coherent(&p.part_max[pidx], mw);
+            store_device_coherent(&p.part_sum[pidx], lsum);
+          }
+        } else {
+          p.part_out[pidx * kD + d] = o / lsum;
+          if (d == 0) {
+            p.part_max[pidx] = mw;  // log2 units
+            p.part_sum[pidx] = lsum;
+          }
+        }
+      }
+    }
+    if (p.fused_merge && !whole) {
+      // Count the arrival and let the workgroup that arrives last merge all pieces (the rule of
+      // decode_attn_reduce_kernel below).  Pieces come from other CUs and other L2s: they were written
+      // with device-coherent stores, every wave waits until its stores have completed before the
+      // arrival is counted, and the merging workgroup reads them with device-coherent loads.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      const int64_t seg = (int64_t)b * Hkv + kvh;
+      if (threadIdx.x == 0) {
+        const unsigned old = __hip_atomic_fetch_add(&p.seg_count[seg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last_piece = old + 1 == (unsigned)(w1 - w0 + 1);
+        if (last_piece) __hip_atomic_store(&p.seg_count[seg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = last_piece;
+      }
+      __syncthreads();
+      if (s_last) {
+        for (int idx = threadIdx.x; idx < G * kD; idx += kThreads) {
+          const int head = idx / kD, d = idx % kD;
+          // four pieces at a time, all their loads in flight together; running (max, sum, out) across batches
+          float m = -INFINITY, wsum = 0.f, o = 0.f;
+          for (int wb = w0; wb <= w1; wb += 4) {
+            float pm[4], ps[4], po[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int64_t pidx = (min(wb + j, w1) + seg) * G + head;
+              pm[j] = load_device_coherent(&p.part_max[pidx]);
+              ps[j] = load_device_coherent(&p.part_sum[pidx]);
+              po[j] = load_device_coherent(&p.part_out[pidx * kD + d]);
+            }
+            float bm = pm[0];
+#pragma unroll
+            for (int j = 1; j < 4; ++j) bm = fmaxf(bm, pm[j]);
+            const float m_new = fmaxf(m, bm);
+            const float keep = __builtin_amdgcn_exp2f(m - m_new);  // 0 for the first batch
+            wsum *= keep;
+            o *= keep;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float wt = wb + j <= w1 ? ps[j] * __builtin_amdgcn_exp2f(pm[j] - m_new) : 0.f;
+              wsum += wt;
+              o += po[j] * wt;
+            }
+            m = m_new;
+          }
+          store_out(head, d, o / wsum * p.v_scale);
         }
       }
     }
@@ -670,6 +758,12 @@ int64_t scratch_floats(int64_t grid, int num_seqs, int num_heads, int head_size)
   return (grid * 16 + (int64_t)num_seqs * num_heads) * (head_size + 2);
 }
 
+// Arrival counters, one per (sequence, kv head); sized for the largest batch so that their place in
+// the workspace is fixed (num_kv_heads <= num_heads).
+int64_t counter_bytes(int /*num_seqs*/, int /*num_heads*/) { return (int64_t)kMaxSeqs * kMaxKvHeads * 4; }
+
+int g_fused_merge = -1;  // -1: decide per call, 0: never, 1: always
+
 int64_t fixed_span_grid(int num_seqs, int num_kv_heads_bound, int max_seq_len, int partition_tokens) {
   const int64_t tiles = (int64_t)num_seqs * num_kv_heads_bound * ((max_seq_len + kTile - 1) / kTile);
   const int64_t span = partition_tokens / kTile;
@@ -698,6 +792,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   if (kv_dtype == VTKV_FP8_E4M3) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
   const int group = num_heads / num_kv_heads;
   VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
+  VTKV_REQUIRE(num_kv_heads <= kMaxKvHeads, "num_kv_heads %d exceeds %d", num_kv_heads, kMaxKvHeads);
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0,
                "q rows must be 16-byte aligned and at least num_heads*head_size apart");
   VTKV_REQUIRE(max_seq_len > 0, "max_seq_len must be > 0");
@@ -740,8 +835,9 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
     grid = g;
   }
   const int64_t n_float = scratch_floats(grid, num_seqs, num_heads, head_size);
+  const int64_t count_bytes = counter_bytes(num_seqs, num_heads);
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
-  const int64_t need = n_float * (int64_t)sizeof(float) + cum_bytes;
+  const int64_t need = n_float * (int64_t)sizeof(float) + cum_bytes + count_bytes;
   if (!workspace || workspace_bytes < need)
     return vtkv::fail(VTKV_ENOMEM, "workspace of %lld bytes is smaller than the %lld needed",
                       (long long)workspace_bytes, (long long)need);
@@ -755,8 +851,16 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.seq_lens = seq_lens;
   p.alibi_slopes = alibi_slopes;
   const int64_t n_stat = grid * 16 + (int64_t)num_seqs * num_heads;  // (slot, head) pairs
-  p.cum_tiles = (int32_t *)workspace;
-  p.part_out = (float *)((char *)workspace + cum_bytes);
+  // the counters come first, at a place that does not depend on the sizes of a call
+  p.seg_count = (uint32_t *)workspace;
+  // Merging inside the streaming kernel saves the second launch, but the workgroup that arrives last
+  // does it at the very end of the kernel with device-coherent round trips (about 6 us).  That pays when
+  // most (sequence, kv head) segments lie inside one workgroup and need no merge at all (measured: +4.5 %
+  // per step at 2048 segments on 512 workgroups, +1.5 % at 1024, -1.6 % at 512), so it is the default
+  // from two segments per workgroup on.
+  p.fused_merge = g_fused_merge == 1 || (g_fused_merge < 0 && (int64_t)num_seqs * num_kv_heads >= 2 * grid);
+  p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
+  p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);
   p.part_max = p.part_out + n_stat * kD;
   p.part_sum = p.part_max + n_stat;
   p.out = out;
@@ -793,7 +897,8 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, p, il);
   if (timed) VTKV_HIP(hipEventRecord(ev[1], st));
-  hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
+  if (!p.fused_merge)
+    hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
   if (timed) {
     VTKV_HIP(hipEventRecord(ev[2], st));
     ++g_timer.calls;
@@ -813,7 +918,8 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
                            ? fixed_span_grid(num_seqs, num_heads, max_seq_len + kTile, partition_tokens)
                            : kDefaultMaxGrid;
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
-  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes;
+  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes +
+         counter_bytes(num_seqs, num_heads);
 }
 
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
@@ -839,6 +945,11 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
   return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, host_seq_lens, num_seqs, num_heads, num_kv_heads,
                         head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, 1.f, 1.f,
                         workspace, workspace_bytes, partition_tokens, stream, key, value, key_stride, value_stride);
+}
+
+int vtkv_set_fused_merge(int on) {
+  g_fused_merge = on < 0 ? -1 : (on != 0);
+  return VTKV_OK;
 }
 
 int vtkv_set_kernel_timing(int on) {

@@ -214,8 +214,10 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  *   max_seq_len  host upper bound of seq_lens (sizes the grid, as in the reference launcher)
  *   alibi_slopes device float[num_heads] or NULL
  *   kv_dtype     q_dtype, or VTKV_FP8_E4M3 with k_scale / v_scale (x = code * scale)
- *   workspace    device scratch of at least vtkv_decode_attention_workspace_bytes(...) bytes; calls that
- *                share a workspace must be ordered on one stream
+ *   workspace    device scratch of at least vtkv_decode_attention_workspace_bytes(...) bytes, zero-filled by
+ *                the caller before its first use and written by nobody else afterwards (the library keeps
+ *                arrival counters in it and leaves them at zero after every call); calls that share a
+ *                workspace must be ordered on one stream
  *   partition_tokens  0: the rows of the whole batch are cut into equal contiguous spans, one per
  *                workgroup of a grid that fills the device once, whatever the sequence lengths are;
  *                > 0 (a multiple of 16, at least 64): every workgroup takes that many rows, the
@@ -246,6 +248,12 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
                                  float scale, int max_seq_len, const float *alibi_slopes, int q_dtype, int out_dtype,
                                  int kv_dtype, void *workspace, int64_t workspace_bytes, int partition_tokens,
                                  void *stream);
+
+/* Where the partial results of the workgroups that share a (sequence, kv head) are merged: 1 = inside the
+ * attention kernel, by whichever of them finishes last; 0 = by a second kernel; -1 (the default) = inside
+ * when the batch has at least two (sequence, kv head) pairs per workgroup, so that most need no merge.
+ * For A/B measurements; results agree up to fp32 summation order.  No counterpart in the reference. */
+int vtkv_set_fused_merge(int on);
 
 /* Benchmark aid without a counterpart in the reference (its kernel benchmark times from the host,
  * benchmarks/kernels/benchmark_paged_attention.py:147-157): while switched on, each vtkv_decode_attention

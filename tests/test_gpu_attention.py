@@ -123,3 +123,23 @@ def test_config3_long_context_split_k(gpu_pool):
     rng = np.random.default_rng(1002)
     lens = [int(rng.integers(32768, 131073)), 131072, 40000]
     run_case(gpu_pool, 1002, lens, 32, 8)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_merge_inside_and_outside_the_kernel(gpu_pool, mode):
+    """The partial results of workgroups that share a (sequence, kv head) are merged either by the
+    workgroup that finishes last or by a second kernel; the library picks per call.  Both forced here,
+    on short sequences (many per workgroup), long ones (many workgroups per sequence) and fixed
+    partitions."""
+    from glake_amd import _C
+
+    lib = _C.lib()
+    _C.check(lib.vtkv_set_fused_merge(mode))
+    try:
+        run_case(gpu_pool, 21, [1, 15, 16, 17, 64, 65, 257, 1025], 32, 8)
+        run_case(gpu_pool, 22, [30000, 3, 9000, 700], 32, 8)
+        run_case(gpu_pool, 23, [700, 64, 1500, 2049], 64, 8, partition_tokens=128)
+        rng = np.random.default_rng(1001)
+        run_case(gpu_pool, 1001, rng.integers(512, 4097, 64).tolist(), 32, 8)
+    finally:
+        _C.check(lib.vtkv_set_fused_merge(-1))
