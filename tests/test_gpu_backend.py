@@ -13,7 +13,8 @@ from kvharness import bits_from_torch_bf16, torch_bf16_from_bits
 pytestmark = pytest.mark.gpu
 
 
-def test_backend_decode_steps_match_oracle(gpu_pool):
+@pytest.mark.parametrize("fuse", [True, False])
+def test_backend_decode_steps_match_oracle(gpu_pool, fuse):
     import torch
 
     from glake_amd import _C
@@ -27,6 +28,7 @@ def test_backend_decode_steps_match_oracle(gpu_pool):
     rng = np.random.default_rng(0)
     eng = CacheEngine(layers, hkv, d, torch.bfloat16, max_seqs, 4096)
     impl = VTensorBackend.get_impl_cls()(hq, d, d ** -0.5, hkv, None, None, "auto")
+    impl.fuse_decode_append = fuse                      # one launch per layer, or cache write + attention
     slots = [4, 1, 5]                                   # three running sequences in slots 4, 1, 5
     lens = [1023, 37, 600]                              # the first crosses a 2 MiB boundary at step 2
     hist_k = {(l, s): [] for l in range(layers) for s in slots}
