@@ -168,6 +168,72 @@ def decode_append_attention(
         ws.numel(), int(partition_tokens), _stream()))
 
 
+_MAX_UNITS = 1024  # units one vtkv_prefill_attention call takes
+
+
+def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], group: int) -> List[List[int]]:
+    """Cut each sequence's query tokens into runs of up to 16/group consecutive tokens: rows
+    [sequence index, first query row, tokens, position of the first token]."""
+    per = max(1, 16 // group)
+    units, row = [], 0
+    for b, (ql, sl) in enumerate(zip(query_lens, seq_lens)):
+        if ql < 0 or sl < ql:
+            raise _C.VtkvError(_C.EINVAL, f"sequence {b}: {ql} query tokens but {sl} rows")
+        ctx = sl - ql
+        for j in range(0, ql, per):
+            units.append([b, row + j, min(per, ql - j), ctx + j])
+        row += ql
+    return units
+
+
+def prefill_attention(
+    out: torch.Tensor,
+    query: torch.Tensor,
+    key_cache: Union[int, torch.Tensor],
+    value_cache: Union[int, torch.Tensor],
+    num_kv_heads: int,
+    scale: float,
+    query_lens: Sequence[int],
+    seq_lens: Sequence[int],
+    slot_mapping: torch.Tensor,
+    alibi_slopes: Optional[torch.Tensor] = None,
+    kv_cache_dtype: str = "auto",
+    kv_scale: float = 1.0,
+    v_scale: Optional[float] = None,
+) -> None:
+    """Causal attention of the prompt tokens of a batch over the contiguous ranges, which already
+    hold the prompt's rows (``reshape_and_cache`` runs first, vllm/attention/backends/xformers.py:
+    301-312).  Stands in for both prompt-run branches of the reference backend (:331-386): a plain
+    prompt (``seq_lens[b] == query_lens[b]``) and a prompt chunk behind a cached prefix
+    (``seq_lens[b] > query_lens[b]``: the last ``query_lens[b]`` positions are the queries).
+    ``query`` / ``out`` are [num_query_tokens, num_heads, head_size], sequences packed in order;
+    ``query_lens`` / ``seq_lens`` are host lists; ``slot_mapping`` holds each sequence's slot."""
+    _require_cuda(out, query, slot_mapping)
+    num_tokens, num_heads, head_size = query.shape
+    if not out.is_contiguous() or out.shape != query.shape:
+        raise _C.VtkvError(_C.EINVAL, "out must be contiguous and shaped like query")
+    if slot_mapping.dtype != torch.int64 or len(query_lens) != len(seq_lens) or sum(query_lens) != num_tokens:
+        raise _C.VtkvError(_C.EINVAL, "slot_mapping must be int64 and query_lens must add up to the query rows")
+    units = prefill_units(query_lens, seq_lens, num_heads // num_kv_heads)
+    if not units:
+        return
+    qd = _dt(query)
+    lib = _C.lib()
+    need = lib.vtkv_prefill_attention_workspace_bytes(min(len(units), _MAX_UNITS), num_kv_heads, head_size)
+    ws = _workspace(need, query.device)
+    if alibi_slopes is not None:
+        alibi_slopes = alibi_slopes.to(device=query.device, dtype=torch.float32)
+    units_t = torch.tensor(units, dtype=torch.int32, device=query.device)
+    max_len = max(seq_lens)
+    for lo in range(0, len(units), _MAX_UNITS):
+        n = min(_MAX_UNITS, len(units) - lo)
+        _C.check(lib.vtkv_prefill_attention(
+            _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping),
+            C.c_void_p(units_t.data_ptr() + 16 * lo), n, num_heads, num_kv_heads, head_size, query.stride(0),
+            float(scale), int(max_len), _ptr(alibi_slopes), qd, _dt(out), _kv_dtype(kv_cache_dtype, qd),
+            float(kv_scale), float(kv_scale if v_scale is None else v_scale), _ptr(ws), ws.numel(), _stream()))
+
+
 def paged_attention_v2(
     out: torch.Tensor,
     exp_sum: Optional[torch.Tensor],

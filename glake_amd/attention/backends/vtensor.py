@@ -3,8 +3,8 @@ one working backend (``vllm/attention/backends/xformers.py``: ``XFormersBackend`
 ``XFormersMetadata`` :65-211, ``XFormersImpl`` :214-433), with the cache write and the decode
 attention served by the HIP kernels of ``libvtkv.so``.
 
-Decode is complete.  Prefill writes its rows into the cache; prefill attention itself belongs
-to a different kernel family and raises ``NotImplementedError``.
+Decode and prompt runs are served (a batch holds one kind, as the fork schedules them); a prompt
+run writes its rows into the cache and then attends over the ranges causally.
 """
 from __future__ import annotations
 
@@ -69,6 +69,9 @@ class VTensorMetadata(AttentionMetadata, PagedAttentionMetadata):
     v_cache_segment_ptr_list: Optional[List[torch.Tensor]] = None
     kvcache_segment: Optional[list] = None
     decode_seq_len: Optional[torch.Tensor] = None
+    # query tokens per prompt when a prompt continues behind rows that are already cached (a reused
+    # prefix, a later chunk of a long prompt); None: every prompt is attended in full (query = all rows)
+    query_lens: Optional[List[int]] = None
     _cached_prefill_metadata: Optional["VTensorMetadata"] = None
     _cached_decode_metadata: Optional["VTensorMetadata"] = None
 
@@ -177,10 +180,28 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
         num_prefill_tokens = attn_metadata.num_prefill_tokens
         num_decode_tokens = attn_metadata.num_decode_tokens
         assert key.shape[0] == num_prefill_tokens + num_decode_tokens
-        if attn_metadata.prefill_metadata is not None:
-            raise NotImplementedError("prefill attention is outside the decode hot path of this backend")
-
         output = None
+        if attn_metadata.prefill_metadata is not None:
+            # xformers.py:331-386: the prompt run.  The reference attends over the key/value tensors
+            # (plain prompt) or over the cache through an external kernel (cached prefix); the rows were
+            # written to the cache above, so both are one causal attention over the ranges here.
+            if key_cache is None:
+                raise NotImplementedError("prompt attention without a KV cache (the reference's profiling run)")
+            from ... import _custom_ops as ops
+            n = attn_metadata.num_prefills
+            seq_lens = list(attn_metadata.seq_lens[:n])
+            query_lens = list(attn_metadata.query_lens[:n]) if attn_metadata.query_lens is not None else seq_lens
+            output = torch.empty_like(query)
+            ops.prefill_attention(
+                output[:num_prefill_tokens], query[:num_prefill_tokens],
+                attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
+                attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], self.num_kv_heads, self.scale,
+                query_lens, seq_lens, attn_metadata.slot_mapping[:n], self.alibi_slopes, self.kv_cache_dtype,
+                kv_scale, vs)
+            if attn_metadata.decode_metadata is None:
+                return output.view(-1, self.num_heads * self.head_size)
+            raise NotImplementedError("a batch that mixes prompt and decode tokens (the fork schedules them apart)")
+
         if attn_metadata.decode_metadata is not None:
             assert key_cache is not None, "decode needs a KV cache"
             output = PagedAttention.forward_decode(

@@ -285,3 +285,42 @@ def textbook_attention(q_f, k_rows, v_rows, scale, alibi_slope=None):
     p = np.exp(s)
     p /= p.sum()
     return p @ v_rows.astype(np.float64)
+
+
+def prefill_attention(q: np.ndarray, cache: "VTensorCache", scale: float, query_lens, seq_lens, alibi_slopes=None,
+                      bf16_round: bool = True):
+    """Causal attention of packed prompt tokens over the contiguous cache, which already holds their
+    rows: the token at position t of its sequence attends to rows 0..t.  This is what both prompt-run
+    branches of the reference backend compute (vllm/attention/backends/xformers.py:331-386; mask
+    convention of tests/kernels/test_prefix_prefill.py:182-192, BlockDiagonalCausalFromBottomRightMask: the
+    queries are the last query_len
+    positions of the sequence).  Restated through the pinned decode oracle: one query token at position
+    t is a decode step over a context of t + 1 rows.
+    q [sum(query_lens), Hq, D]; returns the same shape."""
+    slots, lens = [], []
+    for b, (ql, sl) in enumerate(zip(query_lens, seq_lens)):
+        for i in range(ql):
+            slots.append(cache.slots[b])
+            lens.append(sl - ql + i + 1)
+    per_token = VTensorCache(cache.k_bufs, cache.v_bufs, np.array(slots, np.int64), cache.c.num_kv_heads,
+                             cache.c.head_size)
+    return paged_attention_v1(q, per_token, scale, np.array(lens, np.int32), alibi_slopes, bf16_round)
+
+
+def textbook_causal_attention(q_f, k_rows, v_rows, scale, context_len: int, alibi_slope=None):
+    """Whole-matrix form in float64 for one head of one sequence: q_f [Q, D] are the queries at
+    positions context_len .. context_len+Q-1, k_rows / v_rows [context_len+Q, D]; lower-right aligned
+    causal mask, optional ALiBi bias slope * (key position - query position)."""
+    q64, k64, v64 = (x.astype(np.float64) for x in (q_f, k_rows, v_rows))
+    nq, nk = q64.shape[0], k64.shape[0]
+    assert nk == context_len + nq
+    s = scale * (q64 @ k64.T)
+    qpos = context_len + np.arange(nq)[:, None]
+    kpos = np.arange(nk)[None, :]
+    if alibi_slope is not None:
+        s = s + alibi_slope * (kpos - qpos)
+    s = np.where(kpos <= qpos, s, -np.inf)
+    s -= s.max(axis=1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(axis=1, keepdims=True)
+    return p @ v64

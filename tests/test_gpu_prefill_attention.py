@@ -1,0 +1,120 @@
+"""GPU parity of prompt (prefill) attention over the contiguous ranges, through the C ABI, against
+the prefill oracle on the same seeded inputs: plain prompts, prompt chunks behind a cached prefix,
+GQA groups 1..8, ALiBi, an fp8 cache, and more units than one call takes.  Tolerance as for decode:
+2e-3 abs + 2e-3 rel on the fp32 output (3e-2 for the fp8 cache against the reference's test protocol of
+dequantising to bf16 first); the bf16 output must be the round-to-nearest of the fp32 one."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def run_case(vmm, seed, query_lens, seq_lens, hq, hkv, d=128, alibi=False, fp8=False, tol=2e-3):
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(seed)
+    b = len(seq_lens)
+    slots = rng.permutation(b + 2)[:b]
+    gpu = GpuSeqs(vmm, b + 2, hkv, d, 1 if fp8 else 2, max(seq_lens))
+    empty = np.zeros((1, hkv, d), np.uint8 if fp8 else np.uint16)
+    k_host, v_host = [empty] * (b + 2), [empty] * (b + 2)
+    k_scale = v_scale = 1.0
+    if fp8:
+        k_f = [rng.standard_normal((t, hkv, d)).astype(np.float32) for t in seq_lens]
+        v_f = [rng.standard_normal((t, hkv, d)).astype(np.float32) for t in seq_lens]
+        k_scale = float(max(np.abs(x).max() for x in k_f) / 448.0)
+        v_scale = float(max(np.abs(x).max() for x in v_f) / 448.0)
+    for i, t in enumerate(seq_lens):
+        s = int(slots[i])
+        if fp8:
+            k_host[s], v_host[s] = O.fp8_encode(k_f[i], k_scale), O.fp8_encode(v_f[i], v_scale)
+        else:
+            k_host[s], v_host[s] = bf16_randn(rng, (t, hkv, d)), bf16_randn(rng, (t, hkv, d))
+        gpu.upload(s, k_host[s], v_host[s])
+    n_tok = sum(query_lens)
+    q = bf16_randn(rng, (n_tok, hq, d))
+    scale = float(d) ** -0.5
+    slopes = (rng.standard_normal(hq) * 0.1).astype(np.float32) if alibi else None
+    if fp8:  # exact dequantisation in fp32, which is what the kernel computes with
+        kk = [O.fp8_decode(c, k_scale) for c in k_host]
+        vv = [O.fp8_decode(c, v_scale) for c in v_host]
+    else:
+        kk, vv = k_host, v_host
+    expect = O.prefill_attention(O.bf16_to_f32(q), O.VTensorCache(kk, vv, slots, hkv, d), scale, query_lens, seq_lens,
+                                 slopes)
+    kt, vt = gpu.table_tensors()
+    out32 = torch.empty(n_tok, hq, d, dtype=torch.float32, device="cuda")
+    out16 = torch.empty(n_tok, hq, d, dtype=torch.bfloat16, device="cuda")
+    for o in (out32, out16):
+        ops.prefill_attention(o, torch_bf16_from_bits(q), kt, vt, hkv, scale, query_lens, seq_lens,
+                              torch.tensor(slots, dtype=torch.int64, device="cuda"),
+                              None if slopes is None else torch.from_numpy(slopes).cuda(),
+                              "fp8" if fp8 else "auto", k_scale, v_scale)
+    torch.cuda.synchronize()
+    gpu.close()
+    got = out32.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert np.array_equal(bits_from_torch_bf16(out16), O.f32_to_bf16(got)), "bf16 output is not RNE(fp32 output)"
+    err = np.abs(got - expect)
+    bound = tol + tol * np.abs(expect)
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert np.all(err <= bound), (f"max err {err.max():.3e} at (token, head, d)={worst}: got {got[worst]!r} "
+                                  f"want {expect[worst]!r}")
+    return got
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (8, 8), (16, 1), (12, 4)])
+def test_plain_prompts(gpu_pool, hq, hkv):
+    lens = [1, 2, 3, 15, 16, 17, 33, 100, 257, 700]
+    run_case(gpu_pool, 1, lens, lens, hq, hkv)
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (16, 1)])
+def test_prompt_chunks_behind_a_cached_prefix(gpu_pool, hq, hkv):
+    # (query tokens, rows): chunked prefill and prefix reuse; one decode-like entry with a single query token
+    query_lens = [5, 64, 1, 130, 17, 300]
+    seq_lens = [21, 64 + 1000, 400, 130 + 16, 17 + 2047, 300 + 300]
+    run_case(gpu_pool, 2, query_lens, seq_lens, hq, hkv)
+
+
+def test_alibi(gpu_pool):
+    run_case(gpu_pool, 3, [40, 7, 260], [40, 100, 500], 32, 8, alibi=True)
+
+
+def test_fp8_cache(gpu_pool):
+    run_case(gpu_pool, 4, [33, 200, 64], [33, 200, 64 + 500], 32, 8, fp8=True)
+
+
+def test_long_prompt_needs_several_calls(gpu_pool):
+    # 5000 query tokens at 4 tokens per unit: 1250 units, more than the 1024 one call takes
+    run_case(gpu_pool, 5, [4200, 800], [4200, 800 + 100], 32, 8)
+
+
+def test_prefill_row_equals_decode_of_the_same_position(gpu_pool):
+    """Cross-check without the oracle: every prompt token's output equals (up to fp32 summation order)
+    what decode attention gives for a context cut at that token."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(6)
+    hq, hkv, d, t = 32, 8, 128, 150
+    gpu = GpuSeqs(gpu_pool, 1, hkv, d, 2, t)
+    gpu.upload(0, bf16_randn(rng, (t, hkv, d)), bf16_randn(rng, (t, hkv, d)))
+    q = torch_bf16_from_bits(bf16_randn(rng, (t, hq, d)))
+    kt, vt = gpu.table_tensors()
+    slot = torch.zeros(1, dtype=torch.int64, device="cuda")
+    pre = torch.empty(t, hq, d, dtype=torch.float32, device="cuda")
+    ops.prefill_attention(pre, q, kt, vt, hkv, d ** -0.5, [t], [t], slot)
+    dec = torch.empty(t, hq, d, dtype=torch.float32, device="cuda")
+    ops.paged_attention_v1(dec, q, kt, vt, hkv, d ** -0.5, torch.arange(1, t + 1, dtype=torch.int32, device="cuda"), 1,
+                           t, None, "auto", 1.0, torch.zeros(t, dtype=torch.int64, device="cuda"))
+    torch.cuda.synchronize()
+    gpu.close()
+    assert (pre - dec).abs().max().item() <= 2e-5 + 2e-5 * dec.abs().max().item()

@@ -194,3 +194,27 @@ def test_vtensor_scatter_brute_force():
                                 np.array([1, 0], np.int64), [3, 5], [0, 3], 5, hkv, d)
     assert np.array_equal(bufs_k[1][row:4 * row], key[0:3].reshape(-1)) and not bufs_k[1][4 * row:].any()
     assert np.array_equal(bufs_v[0][2 * row:7 * row], value[3:8].reshape(-1))
+
+
+def test_prefill_oracle_equals_whole_matrix_causal_attention():
+    """The prefill oracle (decode oracle applied per query position) against the float64 whole-matrix
+    form with a lower-right aligned causal mask, with and without a cached prefix and ALiBi."""
+    rng = np.random.default_rng(41)
+    hq, hkv, d = 8, 2, 128
+    g = hq // hkv
+    query_lens, seq_lens = [5, 1, 19, 33], [5, 7, 40, 33]
+    slots = [2, 0, 3, 1]
+    k = [rng.standard_normal((40, hkv, d)).astype(np.float32) for _ in range(4)]
+    v = [rng.standard_normal((40, hkv, d)).astype(np.float32) for _ in range(4)]
+    q = rng.standard_normal((sum(query_lens), hq, d)).astype(np.float32)
+    scale = d ** -0.5
+    for slopes in (None, rng.standard_normal(hq).astype(np.float32)):
+        cache = O.VTensorCache(k, v, slots, hkv, d)
+        got = O.prefill_attention(q, cache, scale, query_lens, seq_lens, slopes)
+        row = 0
+        for b, (ql, sl) in enumerate(zip(query_lens, seq_lens)):
+            for h in range(hq):
+                want = O.textbook_causal_attention(q[row:row + ql, h], k[slots[b]][:sl, h // g], v[slots[b]][:sl, h // g],
+                                                   scale, sl - ql, None if slopes is None else float(slopes[h]))
+                np.testing.assert_allclose(got[row:row + ql, h], want, rtol=2e-5, atol=2e-6)
+            row += ql
