@@ -47,7 +47,90 @@ CONFIGS = {
     # configs[4] without its swap events: 256 sequences
     "c5": dict(name="growth-bf16 B=256 Hq=32 Hkv=8 D=128 ctx~U[256,2048]", batch=256, hq=32, hkv=8, d=128, lo=256,
                hi=2048, seed=1004, kv="bf16"),
+    # outside BASELINE.json: a prompt run (cache write + causal attention over the ranges), 8 prompts of 2048
+    "p2k": dict(name="llama3-8b-prompt-run-bf16 B=8 Hq=32 Hkv=8 D=128 prompt=2048", batch=8, hq=32, hkv=8, d=128,
+                lo=2048, hi=2048, seed=1006, kv="bf16", prefill=True),
 }
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 rate
+
+
+def prompt_run(args, cfg) -> int:
+    """One step = one prompt run of one layer: reshape_and_cache of every prompt row, then causal
+    attention of all prompt tokens over the ranges.  Reported in TFLOP/s (4*Hq*D flop per visible
+    (query, key) pair) against the dense bf16 MFMA peak; this kernel is a first version."""
+    import torch
+
+    from glake_amd import _custom_ops as ops, vmm_allocator as vmm
+    from glake_amd.worker.cache_engine import CacheEngine
+
+    B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
+    K, W = args.steps, args.warmup
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda", 0)
+    gen = torch.Generator().manual_seed(cfg["seed"])
+    lens = torch.randint(cfg["lo"], cfg["hi"] + 1, (B,), generator=gen).tolist()
+    row = Hkv * D * 2
+    chunks = (max(lens) * row + (2 << 20) - 1) // (2 << 20) + 1
+    vmm.init_physical_handle(2 * B * chunks + 16, 0)
+    engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.bfloat16, max_num_seqs=B,
+                         max_num_batched_tokens=max(lens) + 128, swap_space_bytes=0)
+    segs = engine.vmm_kvcache_segment
+    n_tok = sum(lens)
+    ggen = torch.Generator(device=dev).manual_seed(cfg["seed"])
+    q = torch.randn(n_tok, Hq, D, generator=ggen, device=dev).to(torch.bfloat16)
+    k = torch.randn(n_tok, Hkv, D, generator=ggen, device=dev).to(torch.bfloat16)
+    v = torch.randn(n_tok, Hkv, D, generator=ggen, device=dev).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    slot_ids = list(range(B))
+    slot_t = torch.arange(B, dtype=torch.int64, device=dev)
+    lens_t = torch.tensor(lens, dtype=torch.int32, device=dev)
+    starts = torch.tensor([sum(lens[:i]) for i in range(B)], dtype=torch.int32, device=dev)
+    zeros_t = torch.zeros(B, dtype=torch.int64, device=dev)
+    # rows are reserved once (the prompt's chunks are mapped by the step prologue before the first layer)
+    vmm.extend_kv_cache_batch(None, None, slot_ids, [n * row for n in lens], segs, [0] * B, row, False)
+    scale = float(D) ** -0.5
+    torch.cuda.synchronize()
+    torch.cuda.set_stream(torch.cuda.Stream(device=dev))
+
+    def step():
+        ops.reshape_and_cache(k, v, engine.k_cache_ptr[0], engine.v_cache_ptr[0], zeros_t, slot_t, lens_t, starts,
+                              max(lens), Hkv, D)
+        ops.prefill_attention(out, q, engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hkv, scale, lens, lens, slot_t)
+
+    for _ in range(W):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / K
+    # attention alone, with HIP events on the stream it runs on
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev[0].record()
+    for _ in range(K):
+        ops.prefill_attention(out, q, engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hkv, scale, lens, lens, slot_t)
+    ev[1].record()
+    torch.cuda.synchronize()
+    attn_ms = ev[0].elapsed_time(ev[1]) / K
+    pairs = sum(n * (n + 1) // 2 for n in lens)
+    flops = 4 * Hq * D * pairs
+    achieved = flops / (attn_ms * 1e-3) / 1e12
+    result = {
+        "metric": "prompt-run attention TFLOP/s (causal, over contiguous ranges)", "value": round(flops / dt / 1e12, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(dt * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": cfg["name"], "layers": 1, "prompt_tokens": n_tok},
+        "tokens_per_s": round(n_tok / dt, 1),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "decode_attn_stream_kernel (prefill units)", "avg_call_ms": round(attn_ms, 4),
+                     "algorithmic_flops_per_call": flops},
+    }
+    print(json.dumps(result))
+    engine.close()
+    return 0
 
 
 def main() -> int:
@@ -77,6 +160,10 @@ def main() -> int:
     from glake_amd.worker.cache_engine import CacheEngine
 
     cfg = CONFIGS[args.config]
+    if cfg.get("prefill"):
+        if args.steps == 200 and args.warmup == 20:
+            args.steps, args.warmup = 20, 3
+        return prompt_run(args, cfg)
     _C.check(_C.lib().vtkv_set_fused_merge({"auto": -1, "fused": 1, "separate": 0}[args.merge]))
     B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
     K, W = args.steps, args.warmup

@@ -171,19 +171,25 @@ def decode_append_attention(
 _MAX_UNITS = 1024  # units one vtkv_prefill_attention call takes
 
 
-def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], group: int) -> List[List[int]]:
-    """Cut each sequence's query tokens into runs of up to 16/group consecutive tokens: rows
+def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], group: int):
+    """Cut each sequence's query tokens into runs of up to 16/group consecutive tokens: int32 rows
     [sequence index, first query row, tokens, position of the first token]."""
+    import numpy as np
+
     per = max(1, 16 // group)
-    units, row = [], 0
+    parts, row = [], 0
     for b, (ql, sl) in enumerate(zip(query_lens, seq_lens)):
         if ql < 0 or sl < ql:
             raise _C.VtkvError(_C.EINVAL, f"sequence {b}: {ql} query tokens but {sl} rows")
-        ctx = sl - ql
-        for j in range(0, ql, per):
-            units.append([b, row + j, min(per, ql - j), ctx + j])
+        j = np.arange(0, ql, per, dtype=np.int32)
+        u = np.empty((j.size, 4), np.int32)
+        u[:, 0] = b
+        u[:, 1] = row + j
+        u[:, 2] = np.minimum(per, ql - j)
+        u[:, 3] = sl - ql + j
+        parts.append(u)
         row += ql
-    return units
+    return np.concatenate(parts) if parts else np.empty((0, 4), np.int32)
 
 
 def prefill_attention(
@@ -215,7 +221,7 @@ def prefill_attention(
     if slot_mapping.dtype != torch.int64 or len(query_lens) != len(seq_lens) or sum(query_lens) != num_tokens:
         raise _C.VtkvError(_C.EINVAL, "slot_mapping must be int64 and query_lens must add up to the query rows")
     units = prefill_units(query_lens, seq_lens, num_heads // num_kv_heads)
-    if not units:
+    if len(units) == 0:
         return
     qd = _dt(query)
     lib = _C.lib()
@@ -223,7 +229,7 @@ def prefill_attention(
     ws = _workspace(need, query.device)
     if alibi_slopes is not None:
         alibi_slopes = alibi_slopes.to(device=query.device, dtype=torch.float32)
-    units_t = torch.tensor(units, dtype=torch.int32, device=query.device)
+    units_t = torch.from_numpy(units).to(query.device)
     max_len = max(seq_lens)
     for lo in range(0, len(units), _MAX_UNITS):
         n = min(_MAX_UNITS, len(units) - lo)

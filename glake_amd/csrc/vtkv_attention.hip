@@ -288,7 +288,12 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
 
   // ---- this workgroup's span [g_cur, g_end) of the global tile order
   const int span = span_of(p, total_tiles);
-  int g_cur = blockIdx.x * span;
+  // Which span this workgroup takes.  Workgroups are dealt to the 8 XCDs round-robin by their index;
+  // in prefill consecutive spans belong to consecutive units of one sequence, which read the same rows,
+  // so there the workgroups of one XCD take consecutive spans and meet in that XCD's L2 (the grid is a
+  // multiple of 8 then).  Decode reads nothing twice and keeps the plain order.
+  const int wg = PREFILL ? (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : (int)blockIdx.x;
+  int g_cur = wg * span;
   if (g_cur >= total_tiles) return;
   const int g_end = min(total_tiles, g_cur + span);
 
@@ -410,7 +415,9 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
       for (int j = 0; j < kLoads; ++j) {
         uint32_t off = (last ? t_off_last[j] : t_off[j]) & mask;
         if (APPEND) off |= t_off_new & mask_new;
-        regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off));
+        // decode reads every byte once: streaming loads; prefill units of one sequence read the same rows
+        // at about the same time: ordinary loads, so that they meet in L2
+        regs[j] = PREFILL ? *(gvec)(src + row0 + off) : __builtin_nontemporal_load((gvec)(src + row0 + off));
       }
     };
     auto load_k = [&](int i, u32x4 *kr) { load_tile(k_base, nk_base, i, kr); };
@@ -597,7 +604,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
     if (PREFILL && m_wg == -INFINITY) m_wg = 0.f;           // a column none of whose rows lie in this piece
     const float f = __builtin_amdgcn_exp2f(m_run - m_wg);  // 0 for a wave that saw no row
     // slot of this (workgroup, segment): both indices only grow along the tile order, so the sum is unique
-    const int64_t slot_idx = (int64_t)blockIdx.x + (int64_t)b * Hkv + kvh;
+    const int64_t slot_idx = (int64_t)wg + (int64_t)b * Hkv + kvh;
     // workgroups w0..w1 hold the pieces of this (sequence, kv head): its tiles are [first, first + nt_b)
     // of the global order
     const int first_tile = uniform(s_cum[b]) * Hkv + kvh * nt_b;
@@ -886,7 +893,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   } else {
     const int g = resident_grid(kernel, variant);
     if (g <= 0) return vtkv::fail(VTKV_EHIP, "cannot query the kernel's occupancy");
-    grid = g;
+    grid = prefill ? std::max(8, g / 8 * 8) : g;  // prefill deals spans to XCDs in eighths of the grid
   }
   // (prefill keeps 16 columns per slot and kv head instead of the group's heads)
   const int64_t n_float = scratch_floats(grid, num_seqs, prefill ? 16 * num_kv_heads : num_heads, head_size);
