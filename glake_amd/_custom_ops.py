@@ -171,25 +171,28 @@ def decode_append_attention(
 _MAX_UNITS = 1024  # units one vtkv_prefill_attention call takes
 
 
-def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], group: int):
-    """Cut each sequence's query tokens into runs of up to 16/group consecutive tokens: int32 rows
-    [sequence index, first query row, tokens, position of the first token]."""
+def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], per_unit: int):
+    """Cut each sequence's query tokens into runs of up to ``per_unit`` consecutive tokens: int32 rows
+    [sequence index, first query row, tokens, position of the first token], longest context first."""
     import numpy as np
 
-    per = max(1, 16 // group)
     parts, row = [], 0
     for b, (ql, sl) in enumerate(zip(query_lens, seq_lens)):
         if ql < 0 or sl < ql:
             raise _C.VtkvError(_C.EINVAL, f"sequence {b}: {ql} query tokens but {sl} rows")
-        j = np.arange(0, ql, per, dtype=np.int32)
+        j = np.arange(0, ql, per_unit, dtype=np.int32)
         u = np.empty((j.size, 4), np.int32)
         u[:, 0] = b
         u[:, 1] = row + j
-        u[:, 2] = np.minimum(per, ql - j)
+        u[:, 2] = np.minimum(per_unit, ql - j)
         u[:, 3] = sl - ql + j
         parts.append(u)
         row += ql
-    return np.concatenate(parts) if parts else np.empty((0, 4), np.int32)
+    if not parts:
+        return np.empty((0, 4), np.int32)
+    units = np.concatenate(parts)
+    order = np.argsort(-(units[:, 2] + units[:, 3]), kind="stable")  # most rows first: the tail stays short
+    return np.ascontiguousarray(units[order])
 
 
 def prefill_attention(
@@ -220,23 +223,28 @@ def prefill_attention(
         raise _C.VtkvError(_C.EINVAL, "out must be contiguous and shaped like query")
     if slot_mapping.dtype != torch.int64 or len(query_lens) != len(seq_lens) or sum(query_lens) != num_tokens:
         raise _C.VtkvError(_C.EINVAL, "slot_mapping must be int64 and query_lens must add up to the query rows")
-    units = prefill_units(query_lens, seq_lens, num_heads // num_kv_heads)
+    qd = _dt(query)
+    kvd = _kv_dtype(kv_cache_dtype, qd)
+    lib = _C.lib()
+    per_unit = lib.vtkv_prefill_unit_tokens(num_heads, num_kv_heads, kvd)
+    if per_unit <= 0:
+        raise _C.VtkvError(_C.EINVAL, f"unsupported head counts {num_heads}/{num_kv_heads}")
+    units = prefill_units(query_lens, seq_lens, per_unit)
     if len(units) == 0:
         return
-    qd = _dt(query)
-    lib = _C.lib()
     need = lib.vtkv_prefill_attention_workspace_bytes(min(len(units), _MAX_UNITS), num_kv_heads, head_size)
     ws = _workspace(need, query.device)
     if alibi_slopes is not None:
         alibi_slopes = alibi_slopes.to(device=query.device, dtype=torch.float32)
     units_t = torch.from_numpy(units).to(query.device)
     max_len = max(seq_lens)
-    for lo in range(0, len(units), _MAX_UNITS):
-        n = min(_MAX_UNITS, len(units) - lo)
+    per_call = _MAX_UNITS if kvd == _C.FP8_E4M3 else len(units)
+    for lo in range(0, len(units), per_call):
+        n = min(per_call, len(units) - lo)
         _C.check(lib.vtkv_prefill_attention(
             _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping),
             C.c_void_p(units_t.data_ptr() + 16 * lo), n, num_heads, num_kv_heads, head_size, query.stride(0),
-            float(scale), int(max_len), _ptr(alibi_slopes), qd, _dt(out), _kv_dtype(kv_cache_dtype, qd),
+            float(scale), int(max_len), _ptr(alibi_slopes), qd, _dt(out), kvd,
             float(kv_scale), float(kv_scale if v_scale is None else v_scale), _ptr(ws), ws.numel(), _stream()))
 
 

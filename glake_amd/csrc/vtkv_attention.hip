@@ -58,28 +58,29 @@
 #define VTKV_ATTN_OCCUPANCY
 #endif
 static_assert(VTKV_ATTN_STAGES >= 1 && VTKV_ATTN_STAGES <= 4, "1 to 4 register tiles per wave");
+#include "vtkv_attn_common.h"
 #include "vtkv_fp8.h"
+
+namespace vtkv {
+int prefill_attention_bf16(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                           const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
+                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                           const float *alibi_slopes, int q_dtype, int out_dtype, void *stream);
+}
 
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+using namespace vtkv_attn;
 
-constexpr int kD = 128;            // head size
-constexpr int kTile = 16;          // rows per MFMA tile
+
 constexpr int kWaves = 4;          // waves per workgroup
 constexpr int kThreads = kWaves * 64;
 constexpr int kStages = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
-constexpr int kRowBytes = kD * 2;  // bf16 row of one head
 constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
 constexpr int kMinSpan = 4;        // a workgroup takes at least one tile per wave
 constexpr int kDefaultMaxGrid = 4096;  // upper bound of the resident-workgroup grid, sizes the scratch
 constexpr int kMaxKvHeads = 64;        // kv heads per call (sizes the arrival counters)
 constexpr int kInlineLens = 512;       // sequence lengths that fit the kernel argument block
-constexpr float kLog2e = 1.4426950408889634f;
 
 struct AttnParams {
   const uint16_t *q;
@@ -117,87 +118,6 @@ struct InlineLens {
   int32_t v[kInlineLens];
 };
 
-__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
-  // round to nearest even, as the reference's from_float(bf16) does
-  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-  bf16x2 v = {(__bf16)a, (__bf16)b};
-  return __builtin_bit_cast(unsigned, v);
-}
-
-// LDS tile of 16 V rows x 256 bytes.  The 16-byte piece p of row r lives at piece slot
-// p ^ (2*(r & 7)): a transposing read then touches all 64 banks evenly (rows of one read differ
-// in r, pieces in one read are the pair {2*dblk, 2*dblk+1}).
-__device__ __forceinline__ int v_lds_offset(int row, int piece16) {
-  return row * kRowBytes + ((piece16 ^ ((row & 7) << 1)) << 4);
-}
-
-// LDS tile of 16 K rows as loaded (256 bytes of bf16, or 128 bytes of fp8 codes).  It is written a
-// row quarter per 16 lanes and read back one piece per row by 16 lanes; the swizzles keep both
-// conflict-free.
-__device__ __forceinline__ int k_lds_offset(int row, int piece16) {
-  return row * kRowBytes + ((piece16 ^ (row & 15)) << 4);
-}
-__device__ __forceinline__ int k8_lds_offset(int row, int piece16) {
-  return row * kD + ((piece16 ^ ((row >> 1) & 7)) << 4);
-}
-
-// max / sum over the four row groups (lanes l, l^16, l^32, l^48) with the gfx950 lane-swap
-// instructions: v_permlane16_swap exchanges odd 16-lane rows of its first operand with even rows of its
-// second, v_permlane32_swap does the same for 32-lane halves, so swapping a value with itself and
-// combining the two results folds rows pairwise.
-// (the two results are copied to scalars before the bit cast: a bit cast applied directly to an
-// element of the returned vector reads element 0 both times with this compiler)
-__device__ __forceinline__ void swap_rows16(float x, float &a, float &b) {
-  const unsigned u = __builtin_bit_cast(unsigned, x);
-  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  const unsigned r0 = r[0], r1 = r[1];
-  a = __builtin_bit_cast(float, r0);
-  b = __builtin_bit_cast(float, r1);
-}
-__device__ __forceinline__ void swap_rows32(float x, float &a, float &b) {
-  const unsigned u = __builtin_bit_cast(unsigned, x);
-  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  const unsigned r0 = r[0], r1 = r[1];
-  a = __builtin_bit_cast(float, r0);
-  b = __builtin_bit_cast(float, r1);
-}
-
-__device__ __forceinline__ float max_over_row_groups(float x) {
-  float a, b;
-  swap_rows16(x, a, b);
-  swap_rows32(fmaxf(a, b), a, b);
-  return fmaxf(a, b);
-}
-
-__device__ __forceinline__ float sum_over_row_groups(float x) {
-  float a, b;
-  swap_rows16(x, a, b);
-  swap_rows32(a + b, a, b);
-  return a + b;
-}
-
-// eight e4m3fn codes (two dwords) -> eight bf16 values; exact, every e4m3fn value is a bf16 value
-__device__ __forceinline__ u32x4 fp8x8_to_bf16x8(unsigned lo, unsigned hi) {
-  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-  u32x4 r;
-  r[0] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false));
-  r[1] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true));
-  r[2] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false));
-  r[3] = __builtin_bit_cast(unsigned, (bf16x2)__builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true));
-  return r;
-}
-
-// Loads and stores that are coherent across the whole device (they go past the per-XCD L2), for the
-// few values that workgroups hand to each other inside one launch.  A device-scope fence would also
-// do, but it writes back and invalidates a whole L2 each time, which costs far more than these.
-__device__ __forceinline__ void store_device_coherent(float *p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float load_device_coherent(const float *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
 // Tiles per workgroup span, the same rule in both kernels.
 __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
@@ -1004,6 +924,11 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
                            const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
                            float v_scale, void *workspace, int64_t workspace_bytes, void *stream) {
   VTKV_REQUIRE(units, "null argument");
+  if (kv_dtype == VTKV_BF16)  // the dedicated kernel (vtkv_prefill.hip); it needs no workspace
+    return vtkv::prefill_attention_bf16(out, q, k_ptrs, v_ptrs, slot_ids, units, num_units, num_heads, num_kv_heads,
+                                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype,
+                                        stream);
+  // fp8 cache: units of up to 16/G tokens through the streaming kernel
   return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, nullptr, nullptr, num_units, num_heads, num_kv_heads,
                         head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
                         v_scale, workspace, workspace_bytes, 0, stream, nullptr, nullptr, 0, 0, units);

@@ -238,13 +238,18 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
  * function of the cache contents).  The query token at position t of its sequence attends to rows 0..t.
  *   q, out   [num_query_tokens, num_heads, head_size]: the query tokens of all sequences, packed
  *   units    device int32[num_units][4] = {sequence index into slot_ids, first query row, number of query
- *            tokens (1 .. max(1, 16 / (num_heads/num_kv_heads))), position of the first of them in its
- *            sequence}: consecutive query tokens of one sequence that share one pass over its rows;
- *            every query token belongs to exactly one unit; at most 1024 units per call
+ *            tokens (1 .. vtkv_prefill_unit_tokens(...)), position of the first of them in its sequence}:
+ *            consecutive query tokens of one sequence that share one pass over its rows; every query
+ *            token belongs to exactly one unit; longest units first balances the load best; for an fp8
+ *            cache at most 1024 units per call
  *   max_seq_len  host upper bound of position + 1 over all query tokens
  *   workspace    as for vtkv_decode_attention (zero-filled once), at least
  *            vtkv_prefill_attention_workspace_bytes(num_units, num_kv_heads, head_size) bytes
  * Other arguments as for vtkv_decode_attention. */
+/* Query tokens one unit may hold: 128 / (num_heads/num_kv_heads) for a bf16 cache (one workgroup per unit
+ * and kv head), 16 / (num_heads/num_kv_heads), at least 1, for an fp8 cache.  0 for unsupported shapes. */
+int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
+/* Workspace needed for an fp8 cache (a bf16 cache needs none; NULL / 0 may be passed then). */
 int64_t vtkv_prefill_attention_workspace_bytes(int num_units, int num_kv_heads, int head_size);
 int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                            const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
