@@ -57,6 +57,9 @@ SIGNATURES = {
     "vtkv_seg_ensure": (_i, [_p, _i64]),
     "vtkv_seg_preempt": (_i, [_p]),
     "vtkv_seg_release": (_i, [_p]),
+    "vtkv_seg_eager_extend": (_i, [_p, _i]),
+    "vtkv_seg_pending": (_i, [_p]),
+    "vtkv_map_ahead_wait": (_i, []),
     "vtkv_extend_kv_cache_batch": (_i, [_p, _i, _p, _p, _i64, _i, _p]),
     "vtkv_ptr_table_create": (_u64, [_i]),
     "vtkv_ptr_table_destroy": (_i, [_u64]),

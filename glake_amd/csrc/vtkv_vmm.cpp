@@ -19,8 +19,17 @@
 // vtkv_pool_trim, e.g. while the GPU is busy).  If the same segment grows again first, as a sequence
 // that is swapped back in or a slot that is reused does, its retired chunks are simply taken back
 // without any call into the driver.
+//
+// Growth can also be requested ahead of need (vtkv_seg_eager_extend): a worker thread maps the chunks
+// while the caller goes on, with the driver calls made outside the pool mutex, so the only thing that
+// ever waits is an operation on the very segment that is being grown.  This is the reference's
+// eagerExtend / eagerly_extend pair (vmm_allocator.cpp:40-72,307-320) with a condition variable in
+// place of its busy-waiting thread and shared-memory flags, and with the request queue under the lock.
 #include <algorithm>
+#include <condition_variable>
+#include <deque>
 #include <mutex>
+#include <thread>
 #include <unordered_set>
 #include <vector>
 
@@ -42,12 +51,32 @@ namespace {
 
 constexpr int64_t kChunk = 2ll << 20;  // vmm_allocator.h:45 granularitySize
 
+}  // namespace
+}  // namespace vtkv
+struct vtkv_segment;
+namespace vtkv {
+namespace {
+
 struct Pool {
   std::mutex mu;
   int device = -1;
   std::vector<hipMemGenericAllocationHandle_t> free_chunks;
   int64_t total = 0;
   int64_t retired = 0;  // chunks still mapped at the top of shrunken segments; they count as free
+  // map-ahead worker (started on the first request, joined by vtkv_pool_destroy or at exit)
+  struct Request { vtkv_segment *seg; int chunks; };
+  std::deque<Request> requests;
+  std::condition_variable work_cv, done_cv;
+  std::thread worker;
+  bool stop = false;
+  ~Pool() {
+    {
+      std::unique_lock<std::mutex> lk(mu);
+      stop = true;
+    }
+    work_cv.notify_all();
+    if (worker.joinable()) worker.join();
+  }
   std::unordered_set<vtkv_segment *> segments;
 };
 Pool g_pool;
@@ -61,6 +90,8 @@ struct vtkv_segment {
   int64_t expand_bytes = 0; // what release keeps mapped
   int64_t mapped = 0;       // actual_size: bytes mapped per range that belong to the sequence
   int64_t held = 0;         // bytes physically mapped per range, >= mapped; [mapped, held) is retired
+  int pending = 0;          // map-ahead requests queued or in progress; other changes of the segment wait
+  int async_error = 0;      // a map-ahead request failed (reported by the next operation on the segment)
   int64_t used = 0;         // used_size: bytes written per range
   std::vector<char *> k_base, v_base;
   // chunks mapped into layer l's K (resp. V) range, in address order
@@ -185,6 +216,84 @@ int shrink_locked(vtkv_segment *s, int64_t keep_bytes) {
   return VTKV_OK;
 }
 
+// Wait until no map-ahead request of `s` is queued or running (the lock is released meanwhile).
+void settle(std::unique_lock<std::mutex> &lk, vtkv_segment *s) {
+  g_pool.done_cv.wait(lk, [&] { return s->pending == 0; });
+}
+
+// The map-ahead worker.  A request grows one segment by some chunks: retired chunks are taken back and
+// handles for the rest are taken from the free list under the lock, the driver calls run without it,
+// and the result is committed under the lock again.
+void worker_main() {
+  const bool device_ok = hipSetDevice(g_pool.device) == hipSuccess;
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  for (;;) {
+    g_pool.work_cv.wait(lk, [] { return g_pool.stop || !g_pool.requests.empty(); });
+    if (g_pool.stop) return;  // (vtkv_pool_destroy stops it with an empty queue; at exit requests are dropped)
+    const auto rq = g_pool.requests.front();
+    g_pool.requests.pop_front();
+    vtkv_segment *s = rq.seg;
+    if (!device_ok) {
+      s->async_error = VTKV_EHIP;
+      --s->pending;
+      g_pool.done_cv.notify_all();
+      continue;
+    }
+    int n = (int)std::min<int64_t>(rq.chunks, (s->context_max - s->mapped) / kChunk);
+    const int revive = (int)std::min<int64_t>(n, (s->held - s->mapped) / kChunk);
+    s->mapped += (int64_t)revive * kChunk;
+    g_pool.retired -= 2ll * s->layer_num * revive;
+    n -= revive;
+    const int64_t need = 2ll * s->layer_num * n;
+    std::vector<hipMemGenericAllocationHandle_t> handles;
+    if (n > 0 && reclaim_locked(need) >= 0) {
+      handles.assign(g_pool.free_chunks.end() - need, g_pool.free_chunks.end());
+      g_pool.free_chunks.resize(g_pool.free_chunks.size() - need);
+    }
+    if (n > 0 && handles.empty()) s->async_error = VTKV_ENOMEM;
+    if (!handles.empty()) {
+      const int64_t at = s->held;  // == mapped: nothing else changes the segment while it is pending
+      const int layers = s->layer_num;
+      lk.unlock();
+      hipMemAccessDesc ad = {};
+      ad.location.type = hipMemLocationTypeDevice;
+      ad.location.id = g_pool.device;
+      ad.flags = hipMemAccessFlagsProtReadWrite;
+      hipError_t err = hipSuccess;
+      size_t done = 0;  // handle index i maps range (layer, which) = (i / (2n), (i / n) % 2), chunk i % n
+      auto va_of = [&](size_t i) {
+        const int l = (int)(i / (2 * (size_t)n)), which = (int)((i / n) % 2), j = (int)(i % n);
+        return (which ? s->v_base[l] : s->k_base[l]) + at + (int64_t)j * kChunk;
+      };
+      for (; done < handles.size() && err == hipSuccess; ++done) {
+        err = hipMemMap(va_of(done), kChunk, 0, handles[done], 0);
+        if (err != hipSuccess) break;
+        err = hipMemSetAccess(va_of(done), kChunk, &ad, 1);
+        if (err != hipSuccess) {
+          (void)hipMemUnmap(va_of(done), kChunk);
+          break;
+        }
+      }
+      if (err != hipSuccess)
+        for (size_t i = 0; i < done; ++i) (void)hipMemUnmap(va_of(i), kChunk);
+      lk.lock();
+      if (err == hipSuccess) {
+        for (int l = 0; l < layers; ++l)
+          for (int which = 0; which < 2; ++which)
+            for (int j = 0; j < n; ++j)
+              (which ? s->v_chunks[l] : s->k_chunks[l]).push_back(handles[((size_t)l * 2 + which) * n + j]);
+        s->held += (int64_t)n * kChunk;
+        s->mapped = s->held;
+      } else {
+        for (auto h : handles) g_pool.free_chunks.push_back(h);
+        s->async_error = VTKV_EHIP;
+      }
+    }
+    --s->pending;
+    g_pool.done_cv.notify_all();
+  }
+}
+
 int ensure_locked(vtkv_segment *s, int64_t token_bytes) {
   if (s->used + token_bytes <= s->mapped) return 0;
   const int64_t gap = s->used + token_bytes - s->mapped;
@@ -220,7 +329,7 @@ int vtkv_version(void) { return 100; }
 int64_t vtkv_chunk_bytes(void) { return kChunk; }
 
 int vtkv_pool_init(int device, int64_t num_chunks) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   VTKV_REQUIRE(num_chunks >= 0, "num_chunks must be >= 0");
   if (g_pool.device >= 0 && g_pool.device != device)
     return vtkv::fail(VTKV_ESTATE, "pool already lives on device %d", g_pool.device);
@@ -251,17 +360,17 @@ int vtkv_pool_init(int device, int64_t num_chunks) {
 }
 
 int64_t vtkv_pool_free_chunks(void) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   return (int64_t)g_pool.free_chunks.size() + g_pool.retired;
 }
 
 int64_t vtkv_pool_retired_chunks(void) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   return g_pool.retired;
 }
 
 int64_t vtkv_pool_trim(int64_t max_chunks) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   int64_t chunks = 0;
   for (vtkv_segment *s : g_pool.segments) {
     while (s->held > s->mapped && (max_chunks < 0 || chunks < max_chunks)) {
@@ -274,14 +383,22 @@ int64_t vtkv_pool_trim(int64_t max_chunks) {
 }
 
 int64_t vtkv_pool_total_chunks(void) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   return g_pool.total;
 }
 
 int vtkv_pool_destroy(void) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   if (!g_pool.segments.empty())
     return vtkv::fail(VTKV_ESTATE, "%zu segments still alive", g_pool.segments.size());
+  if (g_pool.worker.joinable()) {  // no segment is alive, so no request is queued
+    g_pool.stop = true;
+    g_pool.work_cv.notify_all();
+    lk.unlock();
+    g_pool.worker.join();
+    lk.lock();
+    g_pool.stop = false;
+  }
   for (auto h : g_pool.free_chunks) VTKV_HIP(hipMemRelease(h));
   g_pool.free_chunks.clear();
   g_pool.total = 0;
@@ -290,7 +407,7 @@ int vtkv_pool_destroy(void) {
 }
 
 vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t expand_bytes, int expand) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   if (g_pool.device < 0) {
     vtkv::fail(VTKV_ESTATE, "vtkv_pool_init has not been called");
     return nullptr;
@@ -339,9 +456,22 @@ vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t 
   if (!(s) || !g_pool.segments.count(const_cast<vtkv_segment *>(s)))                                  \
   return vtkv::fail(VTKV_ESTATE, "not a live segment")
 
+// Before changing a segment: let its map-ahead requests finish, and report one that failed.
+#define SEG_SETTLE(s)                                                                                 \
+  do {                                                                                                \
+    settle(lk, (s));                                                                                  \
+    if ((s)->async_error) {                                                                           \
+      const int e_ = (s)->async_error;                                                                \
+      (s)->async_error = 0;                                                                           \
+      return vtkv::fail(e_, "a map-ahead request of this segment failed (%s)",                        \
+                        e_ == VTKV_ENOMEM ? "chunk pool exhausted" : "driver error");                 \
+    }                                                                                                 \
+  } while (0)
+
 int vtkv_seg_destroy(vtkv_segment *s) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
+  SEG_SETTLE(s);
   int rc = shrink_locked(s, 0);
   if (rc < 0) return rc;
   if (trim_segment_locked(s, 0, -1) < 0) return VTKV_EHIP;
@@ -353,7 +483,7 @@ int vtkv_seg_destroy(vtkv_segment *s) {
 }
 
 uint64_t vtkv_seg_key_ptr(const vtkv_segment *s, int layer) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   if (!s || !g_pool.segments.count(const_cast<vtkv_segment *>(s)) || layer < 0 || layer >= s->layer_num) {
     vtkv::fail(VTKV_EINVAL, "bad segment or layer %d", layer);
     return 0;
@@ -362,7 +492,7 @@ uint64_t vtkv_seg_key_ptr(const vtkv_segment *s, int layer) {
 }
 
 uint64_t vtkv_seg_value_ptr(const vtkv_segment *s, int layer) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   if (!s || !g_pool.segments.count(const_cast<vtkv_segment *>(s)) || layer < 0 || layer >= s->layer_num) {
     vtkv::fail(VTKV_EINVAL, "bad segment or layer %d", layer);
     return 0;
@@ -371,13 +501,13 @@ uint64_t vtkv_seg_value_ptr(const vtkv_segment *s, int layer) {
 }
 
 int64_t vtkv_seg_get_used(const vtkv_segment *s) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
   return s->used;
 }
 
 int vtkv_seg_set_used(vtkv_segment *s, int64_t used) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
   VTKV_REQUIRE(used >= 0 && used <= s->context_max, "used_bytes %lld outside [0, %lld]", (long long)used,
                (long long)s->context_max);
@@ -386,35 +516,39 @@ int vtkv_seg_set_used(vtkv_segment *s, int64_t used) {
 }
 
 int64_t vtkv_seg_mapped_bytes(const vtkv_segment *s) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
   return s->mapped;
 }
 
 int vtkv_seg_expand(vtkv_segment *s, int n) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
+  SEG_SETTLE(s);
   VTKV_REQUIRE(n >= 0, "num_chunks must be >= 0");
   return expand_locked(s, n);
 }
 
 int vtkv_seg_reserve(vtkv_segment *s, int64_t token_bytes, int64_t kv_size) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
+  SEG_SETTLE(s);
   VTKV_REQUIRE(token_bytes >= 0 && kv_size >= 0, "sizes must be >= 0");
   return reserve_locked(s, token_bytes, kv_size);
 }
 
 int vtkv_seg_ensure(vtkv_segment *s, int64_t token_bytes) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
+  SEG_SETTLE(s);
   VTKV_REQUIRE(token_bytes >= 0, "token_bytes must be >= 0");
   return ensure_locked(s, token_bytes);
 }
 
 int vtkv_seg_preempt(vtkv_segment *s) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
+  SEG_SETTLE(s);
   int rc = shrink_locked(s, 0);
   if (rc < 0) return rc;
   s->used = 0;
@@ -422,8 +556,9 @@ int vtkv_seg_preempt(vtkv_segment *s) {
 }
 
 int vtkv_seg_release(vtkv_segment *s) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
+  SEG_SETTLE(s);
   // vmm_allocator.cpp:393-420: keep the first expand_size bytes mapped when at least that much is
   // mapped, otherwise (fewer bytes mapped than expand_size) unmap everything.
   const int64_t keep = s->mapped >= s->expand_bytes ? s->expand_bytes : 0;
@@ -433,13 +568,44 @@ int vtkv_seg_release(vtkv_segment *s) {
   return VTKV_OK;
 }
 
+int vtkv_seg_eager_extend(vtkv_segment *s, int num_chunks) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  VTKV_REQUIRE(num_chunks >= 0, "num_chunks must be >= 0");
+  if (num_chunks == 0 || s->mapped >= s->context_max) return VTKV_OK;  // vmm_allocator.cpp:310: nothing left to map
+  if (!g_pool.worker.joinable()) g_pool.worker = std::thread(worker_main);
+  ++s->pending;
+  g_pool.requests.push_back({s, num_chunks});
+  g_pool.work_cv.notify_one();
+  return VTKV_OK;
+}
+
+int vtkv_seg_pending(const vtkv_segment *s) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(s);
+  return s->pending;
+}
+
+int vtkv_map_ahead_wait(void) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  g_pool.done_cv.wait(lk, [] {
+    if (!g_pool.requests.empty()) return false;
+    for (vtkv_segment *s : g_pool.segments)
+      if (s->pending) return false;
+    return true;
+  });
+  return VTKV_OK;
+}
+
 int vtkv_extend_kv_cache_batch(vtkv_segment *const *segs, int n, const int64_t *token_bytes,
                                const int64_t *set_used_tokens, int64_t kv_size, int gen, int64_t *slot_m_out) {
-  std::lock_guard<std::mutex> lk(g_pool.mu);
+  std::unique_lock<std::mutex> lk(g_pool.mu);
   VTKV_REQUIRE(n >= 0 && (n == 0 || (segs && token_bytes && slot_m_out)), "null argument");
   for (int i = 0; i < n; ++i) SEG_CHECK(segs[i]);
   for (int i = 0; i < n; ++i) {
     vtkv_segment *s = segs[i];
+    // a row that needs a chunk which is being mapped ahead waits for it here
+    if (s->pending && s->used + token_bytes[i] > s->mapped) SEG_SETTLE(s);
     if (set_used_tokens && set_used_tokens[i] > 0) s->used = set_used_tokens[i] * kv_size;
     slot_m_out[i] = s->used;
     if (gen) {
@@ -483,7 +649,7 @@ int vtkv_ptr_table_set(uint64_t table, int slot, uint64_t ptr) {
 int vtkv_ptr_table_fill(uint64_t table, vtkv_segment *const *segs, int n, int layer, int which) {
   std::vector<uint64_t> host(n > 0 ? n : 0);
   {
-    std::lock_guard<std::mutex> lk(g_pool.mu);
+    std::unique_lock<std::mutex> lk(g_pool.mu);
     VTKV_REQUIRE(table != 0 && n >= 0 && (n == 0 || segs), "bad table or segment list");
     for (int i = 0; i < n; ++i) {
       SEG_CHECK(segs[i]);

@@ -3,9 +3,12 @@
 (vmm_allocator/vmm_allocator.py:5-19), over the HIP virtual-memory pool of ``libvtkv.so``.
 
 Differences a caller can observe, all deliberate:
-  * growth during decode is done by the calling thread inside ``extend_kv_cache_batch`` /
-    ``eagerExtend`` instead of a detached thread, so ``query_shm`` / ``query_cycle`` always report
-    "ready" and there is nothing to spin on (llama.py:322-326 becomes a no-op);
+  * ``eagerExtend`` hands its request to a worker thread that sleeps on a condition variable (the
+    reference's thread spins on its queue and signals through POSIX shared memory); a row that needs
+    the chunk before the worker is done simply waits inside ``extend_kv_cache_batch``, so the spin
+    on ``query_shm`` at llama.py:322-326 is not needed (it still works);
+  * growth that was not requested ahead is done by the calling thread inside ``extend_kv_cache_batch``;
+  * unmapping is lazy: a released chunk stays mapped ("retired") until another sequence needs it;
   * pool exhaustion raises ``VtkvOutOfChunks`` instead of printing and carrying on
     (vmm_allocator.cpp:232-235,330-333);
   * segments can be destroyed (the reference never frees address ranges).
@@ -92,9 +95,15 @@ class KVcacheSegment:
         _C.check(_C.lib().vtkv_seg_reserve(self._h, int(token_size), int(kv_size)))
 
     def eagerExtend(self, token_size: int, seq_id: int) -> None:
-        """Map ahead so the next ``token_size`` bytes fit (vmm_allocator.cpp:307-320); done
-        in the calling thread."""
-        _C.check(_C.lib().vtkv_seg_ensure(self._h, int(token_size)))
+        """Ask the map-ahead worker for one more chunk per range and return at once
+        (vmm_allocator.cpp:307-320); ``query_shm([seq_id])`` tells when it is there."""
+        _eager_segments[int(seq_id)] = self
+        _C.check(_C.lib().vtkv_seg_eager_extend(self._h, 1))
+
+    @property
+    def pending(self) -> int:
+        """Map-ahead requests of this segment that have not finished."""
+        return int(_C.check(_C.lib().vtkv_seg_pending(self._h)))
 
     def preempt_seq(self, seq_id: int = -1) -> None:
         _C.check(_C.lib().vtkv_seg_preempt(self._h))
@@ -123,6 +132,8 @@ class KVcacheSegment:
 
     def destroy(self) -> None:
         if self._h:
+            for k in [k for k, v in _eager_segments.items() if v is self]:
+                del _eager_segments[k]
             _C.check(_C.lib().vtkv_seg_destroy(self._h))
             self._h = None
 
@@ -205,14 +216,28 @@ def copy_kv_cache(k_cache_batch: Sequence[KVCache], v_cache_batch: Sequence[KVCa
         _C.check(_C.lib().vtkv_ptr_table_fill(v.getKVCachePtr(), segs, len(segment), layer, 1))
 
 
-# Readiness queries of the reference's background mapper (vmm_allocator.cpp:74-111).  Mapping is
-# synchronous here, so every slot is always ready and nothing is pending.
+# Readiness queries of the reference's background mapper (vmm_allocator.cpp:74-111), answered from the
+# segments that eagerExtend was called on under these sequence ids.
+_eager_segments = {}
+
+
 def query_shm(seq_ids: Sequence[int]) -> bool:
+    """True when no map-ahead request of these sequences is outstanding."""
+    for i in seq_ids:
+        seg = _eager_segments.get(int(i))
+        if seg is not None and seg._h and seg.pending:
+            return False
     return True
 
 
 def query_cycle(seq_ids: Sequence[int]) -> bool:
-    return False
+    """The reference's "waited long enough, check again" signal; here simply: something is outstanding."""
+    return not query_shm(seq_ids)
+
+
+def wait_map_ahead() -> None:
+    """Block until every map-ahead request has been carried out."""
+    _C.check(_C.lib().vtkv_map_ahead_wait())
 
 
 def query_unmap(seq_ids: Sequence[int]) -> List[bool]:

@@ -107,6 +107,18 @@ int vtkv_seg_preempt(vtkv_segment *seg);
 /* Unmap all but the first expand_bytes, used = 0; replaces release_seq (vmm_allocator.cpp:383-421). */
 int vtkv_seg_release(vtkv_segment *seg);
 
+/* Map `num_chunks` more chunks into every range of the segment on a worker thread and return at once;
+ * replaces KVcacheSegment::eagerExtend and the eagerly_extend thread (vmm_allocator.cpp:40-72,307-320).
+ * Nothing happens if the ranges are fully mapped.  Any later call that changes the segment, and
+ * vtkv_extend_kv_cache_batch when a new row needs the chunk, first waits for the request; a failed
+ * request (pool exhausted) is reported by that call.  The driver calls run outside the pool's lock. */
+int vtkv_seg_eager_extend(vtkv_segment *s, int num_chunks);
+/* Map-ahead requests of the segment that are queued or running; 0 is the reference's "ready" flag
+ * (query_shm, vmm_allocator.cpp:86-92). <0 on error. */
+int vtkv_seg_pending(const vtkv_segment *s);
+/* Wait until every map-ahead request has been carried out.  No counterpart in the reference. */
+int vtkv_map_ahead_wait(void);
+
 /* Batched bookkeeping of one model step; replaces extend_kv_cache_batch (vmm_allocator.h:138-168).
  * For i < n: if set_used_tokens[i] > 0, used = set_used_tokens[i]*kv_size; slot_m_out[i] = used;
  * then gen ? (ensure mapped, used += token_bytes[i]) : reserve(token_bytes[i], kv_size).

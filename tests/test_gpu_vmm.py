@@ -184,3 +184,65 @@ def test_lazy_unmap_retire_revive_trim_reclaim(gpu_pool):
     b.destroy()
     a.destroy()
     assert vmm.showFreeBlocks() == free0 and vmm.retiredBlocks() == 0
+
+
+def test_map_ahead_requests_run_on_the_worker_and_settle(gpu_pool):
+    """eagerExtend returns at once; the chunk appears without further calls; operations on the segment
+    and rows that need the chunk wait for it; data written before and after is intact; a request that
+    cannot be served is reported by the next operation on the segment."""
+    import time
+
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    vmm.trim()
+    free0 = vmm.showFreeBlocks()
+    layers, row = 2, 2048
+    segs = [vmm.KVcacheSegment(layers, 6 * CHUNK, 0, False) for _ in range(8)]
+    for i, s in enumerate(segs):
+        s.expandMultiSegment(1)
+        s.set_used_size(CHUNK - 3 * row)              # three rows short of the first chunk's end
+        s.eagerExtend(row, 100 + i)
+    deadline = time.time() + 10
+    while not vmm.query_shm(range(100, 108)):
+        assert time.time() < deadline, "map-ahead requests did not finish"
+        time.sleep(0.001)
+    assert not vmm.query_cycle(range(100, 108))
+    assert all(s.actual_size == 2 * CHUNK and s.pending == 0 for s in segs)
+    assert vmm.showFreeBlocks() == free0 - 8 * 2 * layers * 2
+    # rows crossing into the chunk that was mapped ahead: no growth in the calling thread
+    for _ in range(6):
+        slot_m = vmm.extend_kv_cache_batch(None, None, list(range(8)), [row] * 8, segs, [0] * 8, row, True)
+    assert slot_m == [CHUNK + 2 * row] * 8 and all(s.actual_size == 2 * CHUNK for s in segs)
+    blob = np.random.default_rng(5).integers(0, 256, 2 * CHUNK, dtype=np.uint8)
+    _C.check(_C.lib().vtkv_memcpy_h2d(segs[3].getKeyDevicePtr(1), blob.ctypes.data_as(C.c_void_p), blob.nbytes))
+    # a burst of requests followed at once by operations that must wait for them
+    for s in segs:
+        s.eagerExtend(row, 0)
+        s.eagerExtend(row, 0)
+    segs[0].preempt_seq(0)                            # waits for both requests, then gives everything up
+    assert segs[0].actual_size == 0
+    segs[1].expandMultiSegment(1)                     # waits, then grows in the calling thread
+    assert segs[1].actual_size == 5 * CHUNK
+    vmm.wait_map_ahead()
+    assert all(s.actual_size == 4 * CHUNK for s in segs[2:])
+    back = np.empty(2 * CHUNK, np.uint8)
+    _C.check(_C.lib().vtkv_memcpy_d2h(back.ctypes.data_as(C.c_void_p), segs[3].getKeyDevicePtr(1), back.nbytes))
+    assert np.array_equal(back, blob)
+    # fully mapped ranges: a request is a no-op (vmm_allocator.cpp:310)
+    segs[2].expandMultiSegment(2)
+    segs[2].eagerExtend(row, 0)
+    vmm.wait_map_ahead()
+    assert segs[2].actual_size == 6 * CHUNK
+    # a request the pool cannot serve: reported by the next call on that segment, nothing half-mapped
+    hog = vmm.KVcacheSegment(1, (vmm.showFreeBlocks() // 2 + 2) * CHUNK, 0, False)
+    hog.expandMultiSegment((vmm.showFreeBlocks() - 2) // 2)      # leaves fewer chunks than segs[4] needs
+    segs[4].eagerExtend(row, 0)
+    vmm.wait_map_ahead()
+    with pytest.raises(_C.VtkvOutOfChunks):
+        segs[4].expandMultiSegment(1)
+    assert segs[4].actual_size == 4 * CHUNK
+    hog.destroy()
+    for s in segs:
+        s.destroy()
+    assert vmm.showFreeBlocks() == free0
