@@ -57,6 +57,8 @@ SIGNATURES = {
     "vtkv_seg_ensure": (_i, [_p, _i64]),
     "vtkv_seg_preempt": (_i, [_p]),
     "vtkv_seg_release": (_i, [_p]),
+    "vtkv_seg_share_prefix": (_i, [_p, _p, _i64, _p]),
+    "vtkv_pool_shared_chunks": (_i64, []),
     "vtkv_seg_eager_extend": (_i, [_p, _i]),
     "vtkv_seg_pending": (_i, [_p]),
     "vtkv_map_ahead_wait": (_i, []),

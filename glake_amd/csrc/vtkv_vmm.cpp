@@ -30,6 +30,7 @@
 #include <deque>
 #include <mutex>
 #include <thread>
+#include <unordered_map>
 #include <unordered_set>
 #include <vector>
 
@@ -63,6 +64,8 @@ struct Pool {
   std::vector<hipMemGenericAllocationHandle_t> free_chunks;
   int64_t total = 0;
   int64_t retired = 0;  // chunks still mapped at the top of shrunken segments; they count as free
+  // chunks that are mapped into more than one segment (shared prefixes): handle -> number of mappings
+  std::unordered_map<hipMemGenericAllocationHandle_t, int> shared;
   // map-ahead worker (started on the first request, joined by vtkv_pool_destroy or at exit)
   struct Request { vtkv_segment *seg; int chunks; };
   std::deque<Request> requests;
@@ -143,6 +146,16 @@ int map_chunks_locked(vtkv_segment *s, int n) {
   return VTKV_OK;
 }
 
+// One mapping of `h` is gone: the chunk is free again unless another segment still maps it.
+void release_handle_locked(hipMemGenericAllocationHandle_t h) {
+  auto it = g_pool.shared.find(h);
+  if (it == g_pool.shared.end()) {
+    g_pool.free_chunks.push_back(h);
+  } else if (--it->second == 1) {
+    g_pool.shared.erase(it);
+  }
+}
+
 // Physically unmap the retired chunks of `s` at offsets >= max(keep_held, mapped), top down, at most
 // `max_rows` chunk rows (one row = one chunk of every range; < 0: all).  Returns rows unmapped or < 0.
 int64_t trim_segment_locked(vtkv_segment *s, int64_t keep_held, int64_t max_rows) {
@@ -156,7 +169,7 @@ int64_t trim_segment_locked(vtkv_segment *s, int64_t keep_held, int64_t max_rows
         char *base = which ? s->v_base[l] : s->k_base[l];
         // one call per mapping: each chunk was mapped on its own
         VTKV_HIP(hipMemUnmap(base + top * kChunk, kChunk));
-        g_pool.free_chunks.push_back(list.back());
+        release_handle_locked(list.back());
         list.pop_back();
       }
     }
@@ -211,8 +224,18 @@ int expand_locked(vtkv_segment *s, int n) {
 int shrink_locked(vtkv_segment *s, int64_t keep_bytes) {
   if (keep_bytes >= s->mapped) return VTKV_OK;
   const int64_t keep_n = keep_bytes / kChunk;
+  // Chunks that another segment maps as well cannot be counted as free while they sit here retired:
+  // if any of the chunks given up is shared, everything above `keep` is unmapped right away.
+  bool any_shared = false;
+  if (!g_pool.shared.empty())
+    for (int l = 0; l < s->layer_num && !any_shared; ++l)
+      for (int which = 0; which < 2 && !any_shared; ++which) {
+        const auto &list = which ? s->v_chunks[l] : s->k_chunks[l];
+        for (int64_t j = keep_n; j < s->mapped / kChunk && !any_shared; ++j) any_shared = g_pool.shared.count(list[j]) != 0;
+      }
   g_pool.retired += 2ll * s->layer_num * (s->mapped / kChunk - keep_n);
   s->mapped = keep_n * kChunk;
+  if (any_shared && trim_segment_locked(s, keep_bytes, -1) < 0) return VTKV_EHIP;
   return VTKV_OK;
 }
 
@@ -566,6 +589,79 @@ int vtkv_seg_release(vtkv_segment *s) {
   if (rc < 0) return rc;
   s->used = 0;
   return VTKV_OK;
+}
+
+int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, void *stream) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  SEG_CHECK(dst);
+  SEG_CHECK(src);
+  SEG_SETTLE(dst);
+  SEG_SETTLE(src);
+  VTKV_REQUIRE(dst != src && dst->layer_num == src->layer_num, "segments must differ and have the same layer count");
+  VTKV_REQUIRE(bytes >= 0 && bytes <= src->used && src->used <= src->mapped, "prefix of %lld bytes exceeds the source's %lld",
+               (long long)bytes, (long long)src->used);
+  VTKV_REQUIRE(dst->mapped == 0 && dst->used == 0, "the destination segment must be empty");
+  const int64_t whole = bytes / kChunk, tail = bytes % kChunk;
+  VTKV_REQUIRE((whole + (tail ? 1 : 0)) * kChunk <= dst->context_max, "prefix does not fit the destination's range");
+  if (trim_segment_locked(dst, 0, -1) < 0) return VTKV_EHIP;  // its retired chunks would be in the way
+  if (tail && (int64_t)g_pool.free_chunks.size() + g_pool.retired < 2ll * dst->layer_num)
+    return vtkv::fail(VTKV_ENOMEM, "chunk pool exhausted: need %lld, free %lld", 2ll * dst->layer_num,
+                      (long long)((int64_t)g_pool.free_chunks.size() + g_pool.retired));
+  // whole chunks: the same physical chunk at the same offset of the destination's range
+  hipMemAccessDesc ad = {};
+  ad.location.type = hipMemLocationTypeDevice;
+  ad.location.id = g_pool.device;
+  ad.flags = hipMemAccessFlagsProtReadWrite;
+  struct Done { char *va; std::vector<hipMemGenericAllocationHandle_t> *list; hipMemGenericAllocationHandle_t h; };
+  std::vector<Done> done;
+  hipError_t err = hipSuccess;
+  for (int l = 0; l < dst->layer_num && err == hipSuccess; ++l)
+    for (int which = 0; which < 2 && err == hipSuccess; ++which) {
+      auto &from = which ? src->v_chunks[l] : src->k_chunks[l];
+      auto &to = which ? dst->v_chunks[l] : dst->k_chunks[l];
+      char *base = which ? dst->v_base[l] : dst->k_base[l];
+      for (int64_t j = 0; j < whole && err == hipSuccess; ++j) {
+        char *va = base + j * kChunk;
+        err = hipMemMap(va, kChunk, 0, from[j], 0);
+        if (err != hipSuccess) break;
+        to.push_back(from[j]);
+        done.push_back({va, &to, from[j]});
+        err = hipMemSetAccess(va, kChunk, &ad, 1);
+      }
+    }
+  if (err != hipSuccess) {
+    for (auto it = done.rbegin(); it != done.rend(); ++it) {
+      (void)hipMemUnmap(it->va, kChunk);
+      it->list->pop_back();
+    }
+    return vtkv::fail(VTKV_EHIP, "mapping a shared chunk failed: %s", hipGetErrorString(err));
+  }
+  for (const Done &d : done) {
+    auto it = g_pool.shared.find(d.h);
+    if (it == g_pool.shared.end()) g_pool.shared[d.h] = 2; else ++it->second;
+  }
+  dst->held = dst->mapped = whole * kChunk;
+  if (tail) {
+    // the partly filled chunk is the destination's own: both sequences go on writing behind the prefix
+    int rc = expand_locked(dst, 1);
+    if (rc < 0) {
+      (void)shrink_locked(dst, 0);
+      return rc;
+    }
+    for (int l = 0; l < dst->layer_num; ++l)
+      for (int which = 0; which < 2; ++which) {
+        char *to = (which ? dst->v_base[l] : dst->k_base[l]) + whole * kChunk;
+        const char *from = (which ? src->v_base[l] : src->k_base[l]) + whole * kChunk;
+        VTKV_HIP(hipMemcpyAsync(to, from, (size_t)tail, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+      }
+  }
+  dst->used = bytes;
+  return VTKV_OK;
+}
+
+int64_t vtkv_pool_shared_chunks(void) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  return (int64_t)g_pool.shared.size();
 }
 
 int vtkv_seg_eager_extend(vtkv_segment *s, int num_chunks) {

@@ -39,6 +39,11 @@ def totalBlocks() -> int:
     return int(_C.check(_C.lib().vtkv_pool_total_chunks()))
 
 
+def sharedBlocks() -> int:
+    """Physical chunks that are mapped into more than one segment (shared prefixes)."""
+    return int(_C.check(_C.lib().vtkv_pool_shared_chunks()))
+
+
 def retiredBlocks() -> int:
     """Free chunks that are still mapped at the top of a shrunken segment (unmapping is lazy)."""
     return int(_C.check(_C.lib().vtkv_pool_retired_chunks()))
@@ -99,6 +104,12 @@ class KVcacheSegment:
         (vmm_allocator.cpp:307-320); ``query_shm([seq_id])`` tells when it is there."""
         _eager_segments[int(seq_id)] = self
         _C.check(_C.lib().vtkv_seg_eager_extend(self._h, 1))
+
+    def share_prefix(self, src: "KVcacheSegment", nbytes: int, stream: int = 0) -> None:
+        """Begin this (empty) sequence with the first ``nbytes`` bytes of every range of ``src``: whole
+        chunks are mapped a second time instead of copied, the partly filled one is copied on ``stream``
+        (a raw HIP stream handle, 0 = the null stream)."""
+        _C.check(_C.lib().vtkv_seg_share_prefix(self._h, src._h, int(nbytes), C.c_void_p(stream)))
 
     @property
     def pending(self) -> int:

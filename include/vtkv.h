@@ -107,6 +107,17 @@ int vtkv_seg_preempt(vtkv_segment *seg);
 /* Unmap all but the first expand_bytes, used = 0; replaces release_seq (vmm_allocator.cpp:383-421). */
 int vtkv_seg_release(vtkv_segment *seg);
 
+/* Start `dst` (which must hold no rows) as a sequence that shares the first `bytes` bytes of every range
+ * of `src`: whole chunks below that mark are mapped into dst's ranges as well (one physical chunk, two
+ * addresses: no copy, no chunk taken from the pool), the partly filled chunk, if any, is copied into a
+ * chunk of dst's own on `stream`, and dst's used size becomes `bytes`.  Both sequences only ever append
+ * behind the prefix, so neither writes to a shared chunk.  A shared chunk returns to the pool when the
+ * last segment that maps it gives it up.  Stands in for the prefix reuse that the reference's radix cache
+ * plans but leaves unimplemented (vmm_allocator/radix_cache.py:184 `split_and_copy`). */
+int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, void *stream);
+/* Physical chunks currently mapped into more than one segment.  No counterpart in the reference. */
+int64_t vtkv_pool_shared_chunks(void);
+
 /* Map `num_chunks` more chunks into every range of the segment on a worker thread and return at once;
  * replaces KVcacheSegment::eagerExtend and the eagerly_extend thread (vmm_allocator.cpp:40-72,307-320).
  * Nothing happens if the ranges are fully mapped.  Any later call that changes the segment, and

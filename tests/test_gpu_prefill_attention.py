@@ -118,3 +118,48 @@ def test_prefill_row_equals_decode_of_the_same_position(gpu_pool):
     torch.cuda.synchronize()
     gpu.close()
     assert (pre - dec).abs().max().item() <= 2e-5 + 2e-5 * dec.abs().max().item()
+
+
+def test_prompt_behind_a_shared_prefix(gpu_pool):
+    """Prefix reuse end to end: a second sequence maps the first one's whole chunks instead of
+    recomputing them, writes only its own rows (multi-token reshape_and_cache) and attends over prefix +
+    own rows; the first sequence is untouched."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(8)
+    hq, hkv, d = 32, 8, 128
+    row = hkv * d * 2
+    shared_rows, own_rows = 2050, 60                      # 2 whole chunks (2048 rows) + 2 rows copied
+    gpu = GpuSeqs(gpu_pool, 2, hkv, d, 2, 4096)
+    k_a, v_a = bf16_randn(rng, (2100, hkv, d)), bf16_randn(rng, (2100, hkv, d))
+    gpu.upload(0, k_a, v_a)
+    gpu.segs[1].share_prefix(gpu.segs[0], shared_rows * row, torch.cuda.current_stream().cuda_stream)
+    assert gpu_pool.sharedBlocks() == 4                   # two chunks of K and of V
+    nk, nv = bf16_randn(rng, (own_rows, hkv, d)), bf16_randn(rng, (own_rows, hkv, d))
+    q = bf16_randn(rng, (own_rows, hq, d))
+    kt, vt = gpu.table_tensors()
+    slot_t = torch.tensor([1], dtype=torch.int64, device="cuda")
+    # the step prologue reserves room for the new rows (maps a third chunk) and returns where they go
+    slot_m = gpu_pool.extend_kv_cache_batch(None, None, [1], [own_rows * row], [gpu.segs[1]], [0], row, False)
+    assert slot_m == [shared_rows * row]
+    ops.reshape_and_cache(torch_bf16_from_bits(nk), torch_bf16_from_bits(nv), kt, vt,
+                          torch.tensor(slot_m, dtype=torch.int64, device="cuda"), slot_t,
+                          torch.tensor([own_rows], dtype=torch.int32, device="cuda"),
+                          torch.zeros(1, dtype=torch.int32, device="cuda"), own_rows, hkv, d)
+    out = torch.empty(own_rows, hq, d, dtype=torch.float32, device="cuda")
+    ops.prefill_attention(out, torch_bf16_from_bits(q), kt, vt, hkv, d ** -0.5, [own_rows], [shared_rows + own_rows], slot_t)
+    torch.cuda.synchronize()
+    k_b = np.concatenate([k_a[:shared_rows], nk])
+    v_b = np.concatenate([v_a[:shared_rows], nv])
+    n = (shared_rows + own_rows) * row
+    assert np.array_equal(gpu.download(1, n, which="k", dtype=np.uint16), k_b.reshape(-1))
+    assert np.array_equal(gpu.download(1, n, which="v", dtype=np.uint16), v_b.reshape(-1))
+    assert np.array_equal(gpu.download(0, 2100 * row, which="k", dtype=np.uint16), k_a.reshape(-1))
+    expect = O.prefill_attention(O.bf16_to_f32(q), O.VTensorCache([k_a, k_b], [v_a, v_b], [1], hkv, d), d ** -0.5,
+                                 [own_rows], [shared_rows + own_rows])
+    got = out.cpu().numpy()
+    gpu.close()
+    assert np.all(np.abs(got - expect) <= 2e-3 + 2e-3 * np.abs(expect))
+    assert gpu_pool.sharedBlocks() == 0

@@ -246,3 +246,70 @@ def test_map_ahead_requests_run_on_the_worker_and_settle(gpu_pool):
     for s in segs:
         s.destroy()
     assert vmm.showFreeBlocks() == free0
+
+
+def test_shared_prefix_maps_whole_chunks_twice_and_copies_the_tail(gpu_pool):
+    """A new sequence that starts with another one's prefix: whole chunks become visible at a second
+    address without taking chunks from the pool, the partly filled chunk is copied, both sequences go on
+    independently, and a shared chunk returns to the pool only when its last user lets go."""
+    import torch
+
+    from glake_amd import _C
+
+    def read(ptr, n):
+        out = np.empty(n, np.uint8)
+        _C.check(_C.lib().vtkv_memcpy_d2h(out.ctypes.data_as(C.c_void_p), ptr, n))
+        return out
+
+    def write(ptr, data):
+        _C.check(_C.lib().vtkv_memcpy_h2d(ptr, data.ctypes.data_as(C.c_void_p), data.nbytes))
+
+    vmm = gpu_pool
+    vmm.trim()
+    free0 = vmm.showFreeBlocks()
+    layers = 2
+    rng = np.random.default_rng(9)
+    src = vmm.KVcacheSegment(layers, 8 * CHUNK, 0, False)
+    src.expandMultiSegment(3)
+    used = 2 * CHUNK + 12345 * 16
+    blobs = {}
+    for l in range(layers):
+        for which, ptr in (("k", src.getKeyDevicePtr(l)), ("v", src.getValueDevicePtr(l))):
+            blobs[(l, which)] = rng.integers(0, 256, used, dtype=np.uint8)
+            write(ptr, blobs[(l, which)])
+    src.set_used_size(used)
+    prefix = 2 * CHUNK + 4000 * 16                       # two whole chunks and a partly filled one
+    dst = vmm.KVcacheSegment(layers, 8 * CHUNK, 0, False)
+    dst.share_prefix(src, prefix, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert dst.used_size == prefix and dst.actual_size == 3 * CHUNK
+    assert vmm.sharedBlocks() == 2 * 2 * layers           # two chunks of each of the 2*layers ranges
+    assert vmm.showFreeBlocks() == free0 - 3 * 2 * layers - 1 * 2 * layers   # only the tail chunks are new
+    for l in range(layers):
+        for which, ptr in (("k", dst.getKeyDevicePtr(l)), ("v", dst.getValueDevicePtr(l))):
+            assert np.array_equal(read(ptr, prefix), blobs[(l, which)][:prefix])
+    # both go on writing behind the prefix without seeing each other
+    mine = rng.integers(0, 256, 4096, dtype=np.uint8)
+    write(dst.getKeyDevicePtr(0) + prefix, mine)
+    assert np.array_equal(read(src.getKeyDevicePtr(0) + prefix, 4096), blobs[(0, "k")][prefix:prefix + 4096])
+    dst.expandMultiSegment(1)
+    assert dst.actual_size == 4 * CHUNK
+    # a third sequence shares with the second one: the first two chunks now have three users
+    third = vmm.KVcacheSegment(layers, 8 * CHUNK, 0, False)
+    third.share_prefix(dst, 2 * CHUNK)
+    assert third.actual_size == 2 * CHUNK and vmm.sharedBlocks() == 2 * 2 * layers
+    free_before = vmm.showFreeBlocks()
+    src.preempt_seq(0)                                     # the owner leaves first
+    assert src.actual_size == 0 and vmm.retiredBlocks() == 0
+    assert vmm.showFreeBlocks() == free_before + 1 * 2 * layers     # only its unshared third chunk came back
+    for seg in (dst, third):
+        assert np.array_equal(read(seg.getValueDevicePtr(1), 2 * CHUNK), blobs[(1, "v")][:2 * CHUNK])
+    assert np.array_equal(read(dst.getKeyDevicePtr(0) + prefix, 4096), mine)
+    dst.destroy()
+    assert vmm.sharedBlocks() == 0 and np.array_equal(read(third.getKeyDevicePtr(1), 2 * CHUNK), blobs[(1, "k")][:2 * CHUNK])
+    third.release_seq(0)
+    with pytest.raises(_C.VtkvError):
+        third.share_prefix(src, 1)                         # the source holds no rows any more
+    src.destroy()
+    third.destroy()
+    assert vmm.showFreeBlocks() == free0 and vmm.retiredBlocks() == 0
