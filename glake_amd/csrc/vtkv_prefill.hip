@@ -145,13 +145,36 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
 #pragma unroll
       for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const u32x4 *>(k_tile + k_lds_offset(n, 4 * c + g));
       const bool masked = t0 + kTile > wave_first_limit;  // wave-uniform: the tile reaches some column's limit
-      bf16x8 pop[kNB];
+      // Order within the tile: all S MFMAs first, then per column block its softmax followed by its P.V
+      // MFMAs, so that the matrix pipe works on one block's P.V while the vector unit does the next
+      // block's softmax.
+      f32x4 sacc[kNB];
 #pragma unroll
       for (int nb = 0; nb < kNB; ++nb) {
-        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        sacc[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
-          s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[ks]), qop[nb][ks], s, 0, 0, 0);
+          sacc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[ks]), qop[nb][ks], sacc[nb], 0,
+                                                             0, 0);
+      }
+      // transposed V operands, read once for both column blocks
+      u32x4 vop[8];
+      {
+        const int row = 4 * g + (n >> 2);
+        const int base = row * kRowBytes + ((n & 1) << 3);
+        const int swz = (row & 7) << 1;
+#pragma unroll
+        for (int db = 0; db < 8; ++db) {
+          const int off = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
+          const s16x4 quad =
+              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(v_tile + off));
+          const u32x2 qd = __builtin_bit_cast(u32x2, quad);
+          vop[db] = (u32x4){qd[0], qd[1], qd[0], qd[1]};
+        }
+      }
+#pragma unroll
+      for (int nb = 0; nb < kNB; ++nb) {
+        const f32x4 s = sacc[nb];
         float x[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -164,7 +187,10 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
             if (t0 + 4 * g + r >= limit[nb]) x[r] = -INFINITY;
         }
         const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
-        const float m_new = fmaxf(m_run[nb], tmax);
+        // The reference point of the exponentials only follows the running maximum when that has grown by
+        // more than 8 (a factor 256 in the weights, harmless in fp32): the rescale of the accumulators,
+        // which otherwise runs whenever any of the wave's 32 columns sees a new maximum, becomes rare.
+        const float m_new = tmax > m_run[nb] + 8.f ? tmax : m_run[nb];
         // (a column can have a whole tile masked; the reference point 0 keeps exp2(-inf - ref) = 0)
         const float m_ref = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_ref);
@@ -189,32 +215,11 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
         }
         pb[2] = pack_bf16x2(plo[0], plo[1]);
         pb[3] = pack_bf16x2(plo[2], plo[3]);
-        pop[nb] = __builtin_bit_cast(bf16x8, pb);
-      }
-      // O^T += V^T.P^T: each transposed V operand is read once and used for both column blocks
-      {
-        const int row = 4 * g + (n >> 2);
-        const int base = row * kRowBytes + ((n & 1) << 3);
-        const int swz = (row & 7) << 1;
+        const bf16x8 pop = __builtin_bit_cast(bf16x8, pb);
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          u32x4 vop[4];
-#pragma unroll
-          for (int d4 = 0; d4 < 4; ++d4) {
-            const int db = 4 * half + d4;
-            const int off = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
-            const s16x4 quad =
-                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(v_tile + off));
-            const u32x2 qd = __builtin_bit_cast(u32x2, quad);
-            vop[d4] = (u32x4){qd[0], qd[1], qd[0], qd[1]};
-          }
-#pragma unroll
-          for (int nb = 0; nb < kNB; ++nb)
-#pragma unroll
-            for (int d4 = 0; d4 < 4; ++d4)
-              acc[nb][4 * half + d4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  __builtin_bit_cast(bf16x8, vop[d4]), pop[nb], acc[nb][4 * half + d4], 0, 0, 0);
-        }
+        for (int db = 0; db < 8; ++db)
+          acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[db]), pop, acc[nb][db], 0,
+                                                                0, 0);
       }
     }
     lstore((kb + 1) & 1);  // nobody reads that stage: its readers finished before the last barrier
