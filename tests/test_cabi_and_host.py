@@ -116,3 +116,32 @@ def test_product_package_never_touches_the_oracle():
 def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_prefill_units_cover_every_query_token_once():
+    """Host logic of the prompt attention: the unit table (sequence, first query row, tokens, position of
+    the first token) covers each packed query row exactly once, keeps units inside one sequence, respects
+    the per-unit limit, places chunk queries at the end of their sequence and lists longest contexts first."""
+    import numpy as np
+
+    from glake_amd._custom_ops import prefill_units
+
+    query_lens, seq_lens = [5, 0, 130, 1, 64], [5, 9, 400, 77, 64]
+    for per_unit in (1, 4, 16, 32, 128):
+        u = prefill_units(query_lens, seq_lens, per_unit)
+        assert u.dtype == np.int32 and u.shape[1] == 4 and (u[:, 2] >= 1).all() and (u[:, 2] <= per_unit).all()
+        seen = np.zeros(sum(query_lens), int)
+        starts = np.concatenate([[0], np.cumsum(query_lens)])
+        for b, row0, ntok, pos0 in u.tolist():
+            seen[row0:row0 + ntok] += 1
+            assert starts[b] <= row0 and row0 + ntok <= starts[b + 1]                 # inside its sequence
+            assert pos0 == seq_lens[b] - query_lens[b] + (row0 - starts[b])           # lower-right aligned
+        assert (seen == 1).all()
+        reach = u[:, 2] + u[:, 3]
+        assert (np.diff(reach) <= 0).all()
+    assert prefill_units([], [], 4).shape == (0, 4)
+    import pytest
+
+    from glake_amd import _C
+    with pytest.raises(_C.VtkvError):
+        prefill_units([5], [4], 4)                                                     # more queries than rows
