@@ -168,9 +168,6 @@ def decode_append_attention(
         ws.numel(), int(partition_tokens), _stream()))
 
 
-_MAX_UNITS = 1024  # units one vtkv_prefill_attention call takes
-
-
 def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], per_unit: int):
     """Cut each sequence's query tokens into runs of up to ``per_unit`` consecutive tokens: int32 rows
     [sequence index, first query row, tokens, position of the first token], longest context first."""
@@ -232,20 +229,13 @@ def prefill_attention(
     units = prefill_units(query_lens, seq_lens, per_unit)
     if len(units) == 0:
         return
-    need = lib.vtkv_prefill_attention_workspace_bytes(min(len(units), _MAX_UNITS), num_kv_heads, head_size)
-    ws = _workspace(need, query.device)
     if alibi_slopes is not None:
         alibi_slopes = alibi_slopes.to(device=query.device, dtype=torch.float32)
     units_t = torch.from_numpy(units).to(query.device)
-    max_len = max(seq_lens)
-    per_call = _MAX_UNITS if kvd == _C.FP8_E4M3 else len(units)
-    for lo in range(0, len(units), per_call):
-        n = min(per_call, len(units) - lo)
-        _C.check(lib.vtkv_prefill_attention(
-            _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping),
-            C.c_void_p(units_t.data_ptr() + 16 * lo), n, num_heads, num_kv_heads, head_size, query.stride(0),
-            float(scale), int(max_len), _ptr(alibi_slopes), qd, _dt(out), kvd,
-            float(kv_scale), float(kv_scale if v_scale is None else v_scale), _ptr(ws), ws.numel(), _stream()))
+    _C.check(lib.vtkv_prefill_attention(
+        _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping), _ptr(units_t), len(units),
+        num_heads, num_kv_heads, head_size, query.stride(0), float(scale), int(max(seq_lens)), _ptr(alibi_slopes), qd,
+        _dt(out), kvd, float(kv_scale), float(kv_scale if v_scale is None else v_scale), _stream()))
 
 
 def paged_attention_v2(

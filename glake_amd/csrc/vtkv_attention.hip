@@ -61,13 +61,6 @@ static_assert(VTKV_ATTN_STAGES >= 1 && VTKV_ATTN_STAGES <= 4, "1 to 4 register t
 #include "vtkv_attn_common.h"
 #include "vtkv_fp8.h"
 
-namespace vtkv {
-int prefill_attention_bf16(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
-                           const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
-                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
-                           const float *alibi_slopes, int q_dtype, int out_dtype, void *stream);
-}
-
 namespace {
 
 using namespace vtkv_attn;
@@ -108,9 +101,6 @@ struct AttnParams {
   const char *new_k, *new_v;
   int64_t new_k_stride, new_v_stride;
   int inline_lens;  // sequence lengths come with the kernel arguments instead of from seq_lens
-  // prefill: [num_seqs][4] = {sequence, first query row, query tokens, position of the first token};
-  // num_seqs then counts these units instead of sequences
-  const int32_t *units;
 };
 
 // Sequence lengths passed by value (no upload, no dependent global load at the start of the kernel).
@@ -134,17 +124,10 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // own at the end of the sequence's tile list, loaded from new_k / new_v, and the wave that handles it
 // also stores the row into the cache.  One launch then does reshape_and_cache and attention, and each
 // byte of the new rows is read once.
-//
-// PREFILL: the 16 columns are not the G heads of one query token but up to 16/G consecutive query tokens
-// of one sequence times their G heads ("unit"; p.units lists them and takes the place of the
-// sequences).  The token at position t sees rows 0..t of the cache, which already holds the prompt's own
-// rows; each lane applies its column's limit to the logits, everything else is as in decode.  A unit's
-// rows are read once for all its tokens, i.e. 16/G times less often than one decode call per token would.
-template <bool ALIBI, bool FP8, bool APPEND, bool PREFILL>
+template <bool ALIBI, bool FP8, bool APPEND>
 __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
   static_assert(!(FP8 && APPEND), "the fused append copies bf16 rows");
-  static_assert(!(PREFILL && APPEND), "prefill rows are written by reshape_and_cache");
   // wave-private V tiles (4 KiB each); reused at the end of a segment for the cross-wave merge
   // then the merge statistics (1 KiB) and the wave-private K tiles
   __shared__ __attribute__((aligned(16))) char smem[2 * kWaves * kTile * kRowBytes + 1024];
@@ -160,11 +143,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
   const int G = p.group;
   const int Hkv = p.num_kv_heads;
   const int B = p.num_seqs;
-  auto len_of = [&](int idx) {
-    if (PREFILL) return p.units[4 * idx + 3] + p.units[4 * idx + 2];  // rows the unit's last token sees
-    return p.inline_lens ? il.v[idx] : p.seq_lens[idx];
-  };
-  const int cstride = PREFILL ? 16 : G;  // columns per partial slot
+  auto len_of = [&](int idx) { return p.inline_lens ? il.v[idx] : p.seq_lens[idx]; };
   // tiles of one kv head of a sequence: its cached rows in 16s, plus the new row's own tile
   auto tiles_of = [](int len) {
     if (len <= 0) return 0;
@@ -208,11 +187,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
 
   // ---- this workgroup's span [g_cur, g_end) of the global tile order
   const int span = span_of(p, total_tiles);
-  // Which span this workgroup takes.  Workgroups are dealt to the 8 XCDs round-robin by their index;
-  // in prefill consecutive spans belong to consecutive units of one sequence, which read the same rows,
-  // so there the workgroups of one XCD take consecutive spans and meet in that XCD's L2 (the grid is a
-  // multiple of 8 then).  Decode reads nothing twice and keeps the plain order.
-  const int wg = PREFILL ? (int)((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : (int)blockIdx.x;
+  const int wg = blockIdx.x;
   int g_cur = wg * span;
   if (g_cur >= total_tiles) return;
   const int g_end = min(total_tiles, g_cur + span);
@@ -250,20 +225,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
 
     // the tables hold plain integers: say explicitly that they are global-memory addresses, otherwise
     // the loads become flat loads that also count on the LDS wait counter and defeat the prefetch
-    // prefill: the unit's sequence, first query row, number of tokens, position of its first token
-    int u_tok0 = b, u_ntok = 1, u_pos0 = seq_len - 1, u_seq = b;
-    if (PREFILL) {
-      u_seq = uniform(p.units[4 * b]);
-      u_tok0 = uniform(p.units[4 * b + 1]);
-      u_ntok = uniform(p.units[4 * b + 2]);
-      u_pos0 = uniform(p.units[4 * b + 3]);
-    }
-    const int ncols = PREFILL ? u_ntok * G : G;        // columns in use
-    const int col_tok = PREFILL ? n / G : 0;           // this lane's column: query token of the unit ...
-    const int col_head = PREFILL ? n % G : n;          // ... and head of the group
-    // rows this lane's column may see (rows below the limit); unused columns see everything (q = 0)
-    const int limit = PREFILL ? (n < ncols ? u_pos0 + col_tok + 1 : 0x7fffffff) : seq_len;
-    const int64_t slot = p.slot_ids[u_seq];
+    const int64_t slot = p.slot_ids[b];
     gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
     gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
     gptr nk_base = k_base, nv_base = v_base;
@@ -278,18 +240,17 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
     // padded heads.
     bf16x8 qop[4];
     {
-      const uint16_t *qrow = p.q + (int64_t)(u_tok0 + (n < ncols ? col_tok : 0)) * p.q_stride +
-                             (int64_t)(kvh * G + (n < ncols ? col_head : 0)) * kD;
+      const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * kD;
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const int d0 = FP8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
         u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + d0);
-        if (n >= ncols) raw = (u32x4){0, 0, 0, 0};
+        if (n >= G) raw = (u32x4){0, 0, 0, 0};
         qop[ks] = __builtin_bit_cast(bf16x8, raw);
       }
     }
     float slope_log2 = 0.f;
-    if (ALIBI) slope_log2 = n < ncols ? p.alibi_slopes[kvh * G + col_head] * kLog2e : 0.f;
+    if (ALIBI) slope_log2 = n < G ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
 
     f32x4 acc[8];
 #pragma unroll
@@ -335,9 +296,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
       for (int j = 0; j < kLoads; ++j) {
         uint32_t off = (last ? t_off_last[j] : t_off[j]) & mask;
         if (APPEND) off |= t_off_new & mask_new;
-        // decode reads every byte once: streaming loads; prefill units of one sequence read the same rows
-        // at about the same time: ordinary loads, so that they meet in L2
-        regs[j] = PREFILL ? *(gvec)(src + row0 + off) : __builtin_nontemporal_load((gvec)(src + row0 + off));
+        regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off));
       }
     };
     auto load_k = [&](int i, u32x4 *kr) { load_tile(k_base, nk_base, i, kr); };
@@ -401,12 +360,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         x[r] = s[r] * p.scale_log2;
-        if (ALIBI) x[r] += slope_log2 * (float)(t0 + 4 * g + r - limit + 1);
-      }
-      if (PREFILL && t0 + kTile > u_pos0 + 1) {  // wave-uniform: the tile reaches past the first token's limit
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (t0 + 4 * g + r >= limit) x[r] = -INFINITY;
+        if (ALIBI) x[r] += slope_log2 * (float)(t0 + 4 * g + r - seq_len + 1);
       }
       if (valid < kTile) {  // wave-uniform: only a sequence's ragged last tile, or the new row's tile
 #pragma unroll
@@ -415,14 +369,11 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
       }
       const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
       const float m_new = fmaxf(m_run, tmax);
-      // (prefill: a column can have all its rows of this tile masked before it has seen any row; the
-      // reference point 0 then keeps the exponentials at exp2(-inf) = 0 instead of exp2(nan))
-      const float m_ref = PREFILL && m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);  // 0 on the first tile (m_run = -inf)
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
       m_run = m_new;
       float pr[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_ref);
+      for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
       l_run = l_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
@@ -520,8 +471,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
       sm_l[wave * 16 + n] = l_run;
     }
     __syncthreads();
-    float m_wg = fmaxf(fmaxf(sm_m[n], sm_m[16 + n]), fmaxf(sm_m[32 + n], sm_m[48 + n]));
-    if (PREFILL && m_wg == -INFINITY) m_wg = 0.f;           // a column none of whose rows lie in this piece
+    const float m_wg = fmaxf(fmaxf(sm_m[n], sm_m[16 + n]), fmaxf(sm_m[32 + n], sm_m[48 + n]));
     const float f = __builtin_amdgcn_exp2f(m_run - m_wg);  // 0 for a wave that saw no row
     // slot of this (workgroup, segment): both indices only grow along the tile order, so the sum is unique
     const int64_t slot_idx = (int64_t)wg + (int64_t)b * Hkv + kvh;
@@ -530,18 +480,17 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
     const int first_tile = uniform(s_cum[b]) * Hkv + kvh * nt_b;
     const int w0 = first_tile / span, w1 = (first_tile + nt_b - 1) / span;
     const bool whole = p.fused_merge && w0 == w1;  // no other workgroup: the result is final
-    auto store_out = [&](int col, int d, float r) {
-      const int64_t oi = PREFILL ? ((int64_t)(u_tok0 + col / G) * p.num_heads + kvh * G + col % G) * kD + d
-                                 : ((int64_t)b * p.num_heads + kvh * G + col) * kD + d;
+    auto store_out = [&](int head, int d, float r) {
+      const int64_t oi = ((int64_t)b * p.num_heads + kvh * G + head) * kD + d;
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
         reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
     };
     // G <= 8 fits the 16 KiB; for larger groups the merge runs in two halves of 8 heads
-    for (int h0 = 0; h0 < ncols; h0 += 8) {
+    for (int h0 = 0; h0 < G; h0 += 8) {
       if (h0 > 0) __syncthreads();
-      if (n >= h0 && n < min(ncols, h0 + 8)) {
+      if (n >= h0 && n < min(G, h0 + 8)) {
 #pragma unroll
         for (int db = 0; db < 8; ++db)
 #pragma unroll
@@ -549,29 +498,23 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
             sm_o[(wave * 8 + (n - h0)) * kD + db * 16 + 4 * g + i] = acc[db][i] * f;
       }
       __syncthreads();
-      const int nh = min(ncols, h0 + 8) - h0;
+      const int nh = min(G, h0 + 8) - h0;
       for (int idx = threadIdx.x; idx < nh * kD; idx += kThreads) {
         const int hh = idx / kD, d = idx % kD;
         const int head = h0 + hh;
-        float mw = fmaxf(fmaxf(sm_m[head], sm_m[16 + head]), fmaxf(sm_m[32 + head], sm_m[48 + head]));
-        const bool none = PREFILL && mw == -INFINITY;  // no row of this piece is visible to the column
-        if (none) mw = 0.f;
+        const float mw = fmaxf(fmaxf(sm_m[head], sm_m[16 + head]), fmaxf(sm_m[32 + head], sm_m[48 + head]));
         float lsum = 0.f, o = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
           lsum += sm_l[w * 16 + head] * __builtin_amdgcn_exp2f(sm_m[w * 16 + head] - mw);
           o += sm_o[(w * 8 + hh) * kD + d];
         }
-        if (none) {  // an empty piece: weight 0 in the merge
-          mw = -INFINITY;
-          lsum = 0.f;
-        }
-        const float o_norm = none ? 0.f : o / lsum;
+        const float o_norm = o / lsum;
         if (whole) {
           store_out(head, d, o_norm * p.v_scale);
           continue;
         }
-        const int64_t pidx = slot_idx * cstride + head;
+        const int64_t pidx = slot_idx * G + head;
         if (p.fused_merge) {
           store_device_coherent(&p.part_out[pidx * kD + d], o_norm);
           if (d == 0) {
@@ -603,7 +546,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
       }
       __syncthreads();
       if (s_last) {
-        for (int idx = threadIdx.x; idx < ncols * kD; idx += kThreads) {
+        for (int idx = threadIdx.x; idx < G * kD; idx += kThreads) {
           const int head = idx / kD, d = idx % kD;
           // four pieces at a time, all their loads in flight together; running (max, sum, out) across batches
           float m = -INFINITY, wsum = 0.f, o = 0.f;
@@ -611,7 +554,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
             float pm[4], ps[4], po[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              const int64_t pidx = (min(wb + j, w1) + seg) * cstride + head;
+              const int64_t pidx = (min(wb + j, w1) + seg) * G + head;
               pm[j] = load_device_coherent(&p.part_max[pidx]);
               ps[j] = load_device_coherent(&p.part_sum[pidx]);
               po[j] = load_device_coherent(&p.part_out[pidx * kD + d]);
@@ -620,13 +563,12 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
 #pragma unroll
             for (int j = 1; j < 4; ++j) bm = fmaxf(bm, pm[j]);
             const float m_new = fmaxf(m, bm);
-            const float m_ref = PREFILL && m_new == -INFINITY ? 0.f : m_new;  // only empty pieces so far
-            const float keep = __builtin_amdgcn_exp2f(m - m_ref);  // 0 for the first batch
+            const float keep = __builtin_amdgcn_exp2f(m - m_new);  // 0 for the first batch
             wsum *= keep;
             o *= keep;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              const float wt = wb + j <= w1 ? ps[j] * __builtin_amdgcn_exp2f(pm[j] - m_ref) : 0.f;
+              const float wt = wb + j <= w1 ? ps[j] * __builtin_amdgcn_exp2f(pm[j] - m_new) : 0.f;
               wsum += wt;
               o += po[j] * wt;
             }
@@ -700,7 +642,7 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 10;  // instantiations of the streaming kernel
+constexpr int kVariants = 6;  // instantiations of the streaming kernel
 struct Residency {
   std::mutex mu;
   int device = -1;
@@ -750,12 +692,10 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
                    int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
                    const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale, float v_scale,
                    void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream, const void *new_key,
-                   const void *new_value, int64_t key_stride, int64_t value_stride, const int32_t *units = nullptr) {
+                   const void *new_value, int64_t key_stride, int64_t value_stride) {
   const bool append = new_key != nullptr;
-  const bool prefill = units != nullptr;
   VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids, "null argument");
-  VTKV_REQUIRE(prefill || (seq_lens != nullptr) != (host_seq_lens != nullptr),
-               "pass either device or host sequence lengths");
+  VTKV_REQUIRE((seq_lens != nullptr) != (host_seq_lens != nullptr), "pass either device or host sequence lengths");
   VTKV_REQUIRE(num_seqs >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
   VTKV_REQUIRE(num_seqs <= kMaxSeqs, "at most %d sequences per call, got %d", kMaxSeqs, num_seqs);
@@ -789,21 +729,16 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
 
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   const bool alibi = alibi_slopes != nullptr;
-  // kernel variant: bit 0 fp8, bit 1 alibi; 4 + alibi for the fused append; 6.. for prefill
-  const int variant = prefill ? 6 + (alibi ? 2 : 0) + (fp8 ? 1 : 0)
-                              : append ? 4 + (alibi ? 1 : 0) : (alibi ? 2 : 0) + (fp8 ? 1 : 0);
+  // kernel variant: bit 0 fp8, bit 1 alibi, 4 + alibi for the fused append
+  const int variant = append ? 4 + (alibi ? 1 : 0) : (alibi ? 2 : 0) + (fp8 ? 1 : 0);
   void (*kernel)(AttnParams, InlineLens) = nullptr;
   switch (variant) {
-    case 0: kernel = decode_attn_stream_kernel<false, false, false, false>; break;
-    case 1: kernel = decode_attn_stream_kernel<false, true, false, false>; break;
-    case 2: kernel = decode_attn_stream_kernel<true, false, false, false>; break;
-    case 3: kernel = decode_attn_stream_kernel<true, true, false, false>; break;
-    case 4: kernel = decode_attn_stream_kernel<false, false, true, false>; break;
-    case 5: kernel = decode_attn_stream_kernel<true, false, true, false>; break;
-    case 6: kernel = decode_attn_stream_kernel<false, false, false, true>; break;
-    case 7: kernel = decode_attn_stream_kernel<false, true, false, true>; break;
-    case 8: kernel = decode_attn_stream_kernel<true, false, false, true>; break;
-    default: kernel = decode_attn_stream_kernel<true, true, false, true>; break;
+    case 0: kernel = decode_attn_stream_kernel<false, false, false>; break;
+    case 1: kernel = decode_attn_stream_kernel<false, true, false>; break;
+    case 2: kernel = decode_attn_stream_kernel<true, false, false>; break;
+    case 3: kernel = decode_attn_stream_kernel<true, true, false>; break;
+    case 4: kernel = decode_attn_stream_kernel<false, false, true>; break;
+    default: kernel = decode_attn_stream_kernel<true, false, true>; break;
   }
   int64_t grid;
   if (partition_tokens > 0) {
@@ -813,10 +748,9 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   } else {
     const int g = resident_grid(kernel, variant);
     if (g <= 0) return vtkv::fail(VTKV_EHIP, "cannot query the kernel's occupancy");
-    grid = prefill ? std::max(8, g / 8 * 8) : g;  // prefill deals spans to XCDs in eighths of the grid
+    grid = g;
   }
-  // (prefill keeps 16 columns per slot and kv head instead of the group's heads)
-  const int64_t n_float = scratch_floats(grid, num_seqs, prefill ? 16 * num_kv_heads : num_heads, head_size);
+  const int64_t n_float = scratch_floats(grid, num_seqs, num_heads, head_size);
   const int64_t count_bytes = counter_bytes(num_seqs, num_heads);
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
   const int64_t need = n_float * (int64_t)sizeof(float) + cum_bytes + count_bytes;
@@ -832,7 +766,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.slot_ids = slot_ids;
   p.seq_lens = seq_lens;
   p.alibi_slopes = alibi_slopes;
-  const int64_t n_stat = grid * 16 + (int64_t)num_seqs * (prefill ? 16 * num_kv_heads : num_heads);  // (slot, column) pairs
+  const int64_t n_stat = grid * 16 + (int64_t)num_seqs * num_heads;  // (slot, head) pairs
   // the counters come first, at a place that does not depend on the sizes of a call
   p.seg_count = (uint32_t *)workspace;
   // Merging inside the streaming kernel saves the second launch, but the workgroup that arrives last
@@ -840,8 +774,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   // most (sequence, kv head) segments lie inside one workgroup and need no merge at all (measured: +4.5 %
   // per step at 2048 segments on 512 workgroups, +1.5 % at 1024, -1.6 % at 512), so it is the default
   // from two segments per workgroup on.
-  p.fused_merge = prefill || g_fused_merge == 1 ||
-                  (g_fused_merge < 0 && (int64_t)num_seqs * num_kv_heads >= 2 * grid);  // (prefill has no merge kernel)
+  p.fused_merge = g_fused_merge == 1 || (g_fused_merge < 0 && (int64_t)num_seqs * num_kv_heads >= 2 * grid);
   p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
   p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);
   p.part_max = p.part_out + n_stat * kD;
@@ -863,7 +796,6 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.new_k_stride = key_stride * 2;
   p.new_v_stride = value_stride * 2;
   p.inline_lens = host_seq_lens != nullptr;
-  p.units = units;
   InlineLens il;
   if (host_seq_lens) memcpy(il.v, host_seq_lens, (size_t)num_seqs * sizeof(int32_t));
 
@@ -916,29 +848,6 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
   return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, nullptr, num_seqs, num_heads, num_kv_heads,
                         head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
                         v_scale, workspace, workspace_bytes, partition_tokens, stream, nullptr, nullptr, 0, 0);
-}
-
-int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
-                           const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
-                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
-                           const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
-                           float v_scale, void *workspace, int64_t workspace_bytes, void *stream) {
-  VTKV_REQUIRE(units, "null argument");
-  if (kv_dtype == VTKV_BF16)  // the dedicated kernel (vtkv_prefill.hip); it needs no workspace
-    return vtkv::prefill_attention_bf16(out, q, k_ptrs, v_ptrs, slot_ids, units, num_units, num_heads, num_kv_heads,
-                                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype,
-                                        stream);
-  // fp8 cache: units of up to 16/G tokens through the streaming kernel
-  return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, nullptr, nullptr, num_units, num_heads, num_kv_heads,
-                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
-                        v_scale, workspace, workspace_bytes, 0, stream, nullptr, nullptr, 0, 0, units);
-}
-
-int64_t vtkv_prefill_attention_workspace_bytes(int num_units, int num_kv_heads, int head_size) {
-  if (num_units <= 0 || num_kv_heads <= 0 || head_size <= 0) return 0;
-  const int64_t cum_bytes = ((int64_t)(num_units + 1) * 4 + 15) / 16 * 16;
-  return scratch_floats(kDefaultMaxGrid, num_units, 16 * num_kv_heads, head_size) * (int64_t)sizeof(float) +
-         cum_bytes + counter_bytes(num_units, num_kv_heads);
 }
 
 int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,

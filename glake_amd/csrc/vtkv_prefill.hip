@@ -1,4 +1,4 @@
-// Prompt (prefill) attention over per-sequence contiguous KV ranges for gfx950, bf16 cache.
+// Prompt (prefill) attention over per-sequence contiguous KV ranges for gfx950, bf16 or fp8-e4m3 cache.
 //
 // The query token at position t of its sequence attends to rows 0..t of the sequence's K and V
 // ranges, which already hold the prompt's own rows.  Unlike decode this is not bound by HBM: a block
@@ -15,6 +15,10 @@
 //    rescale), with each lane applying its column's causal limit to the logits of the tiles that reach it.
 //  * The kv head is the fastest index of the grid: with 8 kv heads the workgroups of one kv head all land
 //    on one XCD, whose L2 then serves the re-reads of that head's rows by later query blocks.
+//
+//  * fp8 cache: rows are e4m3fn codes (128 bytes per head row); they are widened to bf16 (exactly) on the
+//    way into the LDS stage, so everything after the stage is the bf16 kernel; the K scale folds into the
+//    logit scale and the V scale into the final normalisation.
 //
 // Numerics as in the decode kernel (vtkv_attention.hip); the reference computes this with xformers /
 // an external flash-attention kernel (vllm/attention/backends/xformers.py:331-386).
@@ -42,12 +46,13 @@ struct PrefillParams {
   int out_f32;
   int64_t q_stride;
   int num_heads, num_kv_heads, group;
-  float scale_log2;
+  float scale_log2;  // scale * log2(e) [* k_scale for an fp8 cache]
+  float v_scale;     // 1 for a bf16 cache
 };
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-template <bool ALIBI>
+template <bool ALIBI, bool FP8>
 __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kStageBytes];
   const int lane = threadIdx.x & 63;
@@ -65,9 +70,10 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   typedef const __attribute__((address_space(1))) char *gptr;
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
   const int64_t slot = p.slot_ids[u_seq];
-  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kRowBytes;
-  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kRowBytes;
-  const uint32_t row_stride = (uint32_t)Hkv * kRowBytes;
+  constexpr int kKvRowBytes = FP8 ? kD : kRowBytes;  // bytes of one head row in the cache
+  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
+  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
+  const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;
 
   // ---- this wave's columns: block nb, column n -> (token, head); unused columns get q = 0
   bf16x8 qop[kNB][4];
@@ -107,15 +113,18 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     for (int i = 0; i < 8; ++i) acc[nb][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- cooperative stage loads: thread t takes piece t%16 of rows t/16 + 16j of a 64-row block
-  const int ld_piece = threadIdx.x & 15, ld_row = threadIdx.x >> 4;
+  // ---- cooperative stage loads of a 64-row block.  bf16 rows: thread t takes piece t%16 of rows
+  // t/16 + 16j, j < 4.  fp8 rows have 8 pieces of 16 codes: thread t takes piece t%8 of rows t/8 + 32j,
+  // j < 2, and widens it to two bf16 pieces on the way into LDS.
+  constexpr int kLd = FP8 ? 2 : 4;
+  const int ld_piece = FP8 ? threadIdx.x & 7 : threadIdx.x & 15, ld_row = FP8 ? threadIdx.x >> 3 : threadIdx.x >> 4;
   const int nblocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
-  u32x4 kst[kSub], vst[kSub];
+  u32x4 kst[kLd], vst[kLd];
   auto gload = [&](int kb) {
 #pragma unroll
-    for (int j = 0; j < kSub; ++j) {
+    for (int j = 0; j < kLd; ++j) {
       // rows past the end are redirected to the last row; they are masked for every column in use
-      const int row = min(kb * kKeyBlock + j * kTile + ld_row, kv_len - 1);
+      const int row = min(kb * kKeyBlock + j * (kKeyBlock / kLd) + ld_row, kv_len - 1);
       const int64_t off = (int64_t)row * row_stride + ld_piece * 16;
       kst[j] = *(gvec)(k_base + off);
       vst[j] = *(gvec)(v_base + off);
@@ -124,9 +133,18 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   auto lstore = [&](int buf) {
     char *kb_ = smem + buf * kStageBytes, *vb_ = kb_ + kKeyBlock * kRowBytes;
 #pragma unroll
-    for (int j = 0; j < kSub; ++j) {
-      *reinterpret_cast<u32x4 *>(kb_ + j * kTile * kRowBytes + k_lds_offset(ld_row, ld_piece)) = kst[j];
-      *reinterpret_cast<u32x4 *>(vb_ + j * kTile * kRowBytes + v_lds_offset(ld_row, ld_piece)) = vst[j];
+    for (int j = 0; j < kLd; ++j) {
+      if constexpr (FP8) {
+        const int row = j * 32 + ld_row, tile = row >> 4, r = row & 15;
+        char *kt = kb_ + tile * kTile * kRowBytes, *vt = vb_ + tile * kTile * kRowBytes;
+        *reinterpret_cast<u32x4 *>(kt + k_lds_offset(r, 2 * ld_piece)) = fp8x8_to_bf16x8(kst[j][0], kst[j][1]);
+        *reinterpret_cast<u32x4 *>(kt + k_lds_offset(r, 2 * ld_piece + 1)) = fp8x8_to_bf16x8(kst[j][2], kst[j][3]);
+        *reinterpret_cast<u32x4 *>(vt + v_lds_offset(r, 2 * ld_piece)) = fp8x8_to_bf16x8(vst[j][0], vst[j][1]);
+        *reinterpret_cast<u32x4 *>(vt + v_lds_offset(r, 2 * ld_piece + 1)) = fp8x8_to_bf16x8(vst[j][2], vst[j][3]);
+      } else {
+        *reinterpret_cast<u32x4 *>(kb_ + j * kTile * kRowBytes + k_lds_offset(ld_row, ld_piece)) = kst[j];
+        *reinterpret_cast<u32x4 *>(vb_ + j * kTile * kRowBytes + v_lds_offset(ld_row, ld_piece)) = vst[j];
+      }
     }
   };
 
@@ -231,7 +249,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   for (int nb = 0; nb < kNB; ++nb) {
     const float l = sum_over_row_groups(l_run[nb]);
     if (col_tok[nb] < 0) continue;
-    const float inv = 1.f / l;
+    const float inv = p.v_scale / l;
     const int64_t o0 = ((int64_t)(u_row0 + col_tok[nb]) * p.num_heads + kvh * G + col_head[nb]) * kD + 4 * g;
 #pragma unroll
     for (int db = 0; db < 8; ++db) {
@@ -254,24 +272,24 @@ int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype) {
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return 0;
   const int group = num_heads / num_kv_heads;
   if (group > 16) return 0;
-  return kv_dtype == VTKV_FP8_E4M3 ? std::max(1, 16 / group) : kCols / group;
+  (void)kv_dtype;  // the same kernel serves both cache types
+  return kCols / group;
 }
 
-}  // extern "C"
-
-namespace vtkv {
-
-// bf16 cache: the kernel above.  Called by vtkv_prefill_attention (vtkv_attention.hip).
-int prefill_attention_bf16(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
-                                const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
-                                int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
-                                const float *alibi_slopes, int q_dtype, int out_dtype, void *stream) {
+int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                           const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
+                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                           const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                           float v_scale, void *stream) {
   VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids && units, "null argument");
   VTKV_REQUIRE(num_units >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
   VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
   VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
   VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
+  VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be BF16 or FP8_E4M3");
+  const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
+  if (fp8) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
   const int group = num_heads / num_kv_heads;
   VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
@@ -293,14 +311,20 @@ int prefill_attention_bf16(void *out, const void *q, const int64_t *k_ptrs, cons
   p.num_heads = num_heads;
   p.num_kv_heads = num_kv_heads;
   p.group = group;
-  p.scale_log2 = scale * kLog2e;
+  p.scale_log2 = scale * kLog2e * (fp8 ? k_scale : 1.f);
+  p.v_scale = fp8 ? v_scale : 1.f;
   const dim3 grid((unsigned)((int64_t)num_units * num_kv_heads)), block(kThreads);
-  if (alibi_slopes)
-    hipLaunchKernelGGL(prefill_attn_kernel<true>, grid, block, 0, (hipStream_t)stream, p);
+  hipStream_t st = (hipStream_t)stream;
+  if (alibi_slopes && fp8)
+    hipLaunchKernelGGL((prefill_attn_kernel<true, true>), grid, block, 0, st, p);
+  else if (alibi_slopes)
+    hipLaunchKernelGGL((prefill_attn_kernel<true, false>), grid, block, 0, st, p);
+  else if (fp8)
+    hipLaunchKernelGGL((prefill_attn_kernel<false, true>), grid, block, 0, st, p);
   else
-    hipLaunchKernelGGL(prefill_attn_kernel<false>, grid, block, 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL((prefill_attn_kernel<false, false>), grid, block, 0, st, p);
   VTKV_HIP(hipGetLastError());
   return VTKV_OK;
 }
 
-}  // namespace vtkv
+}  // extern "C"

@@ -254,6 +254,10 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                           float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
                           void *stream);
 
+/* Query tokens one unit may hold: 128 / (num_heads/num_kv_heads) (one workgroup per unit and kv head).
+ * 0 for unsupported shapes. */
+int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
+
 /* Causal attention of prompt (or chunked-prefill) tokens over the contiguous ranges, which already hold
  * the tokens' own rows (vtkv_reshape_and_cache runs first, as at vllm/attention/backends/xformers.py:
  * 301-312).  Replaces the prompt-run branch of the backend (xformers.py:331-386: the xformers call for a
@@ -263,22 +267,15 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
  *   units    device int32[num_units][4] = {sequence index into slot_ids, first query row, number of query
  *            tokens (1 .. vtkv_prefill_unit_tokens(...)), position of the first of them in its sequence}:
  *            consecutive query tokens of one sequence that share one pass over its rows; every query
- *            token belongs to exactly one unit; longest units first balances the load best; for an fp8
- *            cache at most 1024 units per call
+ *            token belongs to exactly one unit; longest units first balances the load best
  *   max_seq_len  host upper bound of position + 1 over all query tokens
- *   workspace    as for vtkv_decode_attention (zero-filled once), at least
- *            vtkv_prefill_attention_workspace_bytes(num_units, num_kv_heads, head_size) bytes
- * Other arguments as for vtkv_decode_attention. */
-/* Query tokens one unit may hold: 128 / (num_heads/num_kv_heads) for a bf16 cache (one workgroup per unit
- * and kv head), 16 / (num_heads/num_kv_heads), at least 1, for an fp8 cache.  0 for unsupported shapes. */
-int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
-/* Workspace needed for an fp8 cache (a bf16 cache needs none; NULL / 0 may be passed then). */
-int64_t vtkv_prefill_attention_workspace_bytes(int num_units, int num_kv_heads, int head_size);
+ * No scratch is needed.  Other arguments as for vtkv_decode_attention (kv_dtype VTKV_BF16 or
+ * VTKV_FP8_E4M3 with k_scale / v_scale). */
 int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                            const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
                            int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
                            const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
-                           float v_scale, void *workspace, int64_t workspace_bytes, void *stream);
+                           float v_scale, void *stream);
 
 /* reshape_and_cache (decode form: one new row per sequence) fused into the attention launch; replaces
  * the pair of calls at vllm/attention/backends/xformers.py:310-312 and :357-371 for a decode step.
