@@ -133,7 +133,10 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
   __shared__ __attribute__((aligned(16))) char smem[2 * kWaves * kTile * kRowBytes + 1024];
   __shared__ int s_cum[kMaxSeqs + 1];  // s_cum[b] = tiles (of one kv head) of sequences before b
   __shared__ int s_wave_tot[kWaves];
-  __shared__ int s_last;  // this workgroup delivered the last piece of the current (sequence, kv head)
+  // pieces of shared (sequence, kv head) segments this workgroup has written: segment, first and last
+  // workgroup of the segment, and whether this workgroup delivered the last piece
+  __shared__ int s_pend[2][4];
+  __shared__ int s_npend;
 
   const int lane = threadIdx.x & 63;
   // everything that decides control flow and base addresses is kept wave-uniform (scalar registers)
@@ -150,6 +153,7 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
     return APPEND ? (len - 1 + kTile - 1) / kTile + 1 : (len + kTile - 1) / kTile;
   };
 
+  if (threadIdx.x == 0) s_npend = 0;
   // ---- exclusive prefix sums of the per-sequence tile counts (every workgroup computes its own copy)
   {
     constexpr int kPer = kMaxSeqs / kThreads;
@@ -530,53 +534,15 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
         }
       }
     }
-    if (p.fused_merge && !whole) {
-      // Count the arrival and let the workgroup that arrives last merge all pieces (the rule of
-      // decode_attn_reduce_kernel below).  Pieces come from other CUs and other L2s: they were written
-      // with device-coherent stores, every wave waits until its stores have completed before the
-      // arrival is counted, and the merging workgroup reads them with device-coherent loads.
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-      const int64_t seg = (int64_t)b * Hkv + kvh;
-      if (threadIdx.x == 0) {
-        const unsigned old = __hip_atomic_fetch_add(&p.seg_count[seg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const bool last_piece = old + 1 == (unsigned)(w1 - w0 + 1);
-        if (last_piece) __hip_atomic_store(&p.seg_count[seg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = last_piece;
-      }
-      __syncthreads();
-      if (s_last) {
-        for (int idx = threadIdx.x; idx < G * kD; idx += kThreads) {
-          const int head = idx / kD, d = idx % kD;
-          // four pieces at a time, all their loads in flight together; running (max, sum, out) across batches
-          float m = -INFINITY, wsum = 0.f, o = 0.f;
-          for (int wb = w0; wb <= w1; wb += 4) {
-            float pm[4], ps[4], po[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const int64_t pidx = (min(wb + j, w1) + seg) * G + head;
-              pm[j] = load_device_coherent(&p.part_max[pidx]);
-              ps[j] = load_device_coherent(&p.part_sum[pidx]);
-              po[j] = load_device_coherent(&p.part_out[pidx * kD + d]);
-            }
-            float bm = pm[0];
-#pragma unroll
-            for (int j = 1; j < 4; ++j) bm = fmaxf(bm, pm[j]);
-            const float m_new = fmaxf(m, bm);
-            const float keep = __builtin_amdgcn_exp2f(m - m_new);  // 0 for the first batch
-            wsum *= keep;
-            o *= keep;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const float wt = wb + j <= w1 ? ps[j] * __builtin_amdgcn_exp2f(pm[j] - m_new) : 0.f;
-              wsum += wt;
-              o += po[j] * wt;
-            }
-            m = m_new;
-          }
-          store_out(head, d, o / wsum * p.v_scale);
-        }
-      }
+    if (p.fused_merge && !whole && threadIdx.x == 0) {
+      // A piece of a (sequence, kv head) that other workgroups share.  Its arrival is counted at the end
+      // of this workgroup's span, not here, so that the streaming goes on without waiting for the
+      // stores.  Only the first and the last segment of a span can be such pieces.
+      const int k = s_npend;
+      s_pend[k][0] = b * Hkv + kvh;
+      s_pend[k][1] = w0;
+      s_pend[k][2] = w1;
+      s_npend = k + 1;
     }
 
     // ---- next segment of the span
@@ -594,6 +560,68 @@ __global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
         }
       }
       __syncthreads();  // the merge area is the next segment's V tiles
+    }
+  }
+
+  // ---- arrivals and merges of the shared segments (the rule of decode_attn_reduce_kernel below).
+  // Pieces come from other CUs and other L2s: they were written with device-coherent stores, every wave
+  // waits until its stores have completed before the arrivals are counted, and the pieces are read with
+  // device-coherent loads.  The workgroup that delivers the last piece of a segment merges it and leaves
+  // the counter at zero for the next launch.
+  if (p.fused_merge) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const int np = uniform(s_npend);
+    if (np == 0) return;
+    if (lane == 0 && wave < np) {
+      const int seg = s_pend[wave][0];
+      const unsigned pieces = (unsigned)(s_pend[wave][2] - s_pend[wave][1] + 1);
+      const unsigned old = __hip_atomic_fetch_add(&p.seg_count[seg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last_piece = old + 1 == pieces;
+      if (last_piece) __hip_atomic_store(&p.seg_count[seg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_pend[wave][3] = last_piece;
+    }
+    __syncthreads();
+    const int per_seg = G * kD;
+    for (int idx = threadIdx.x; idx < np * per_seg; idx += kThreads) {
+      const int j = idx / per_seg;
+      if (!s_pend[j][3]) continue;
+      const int head = (idx - j * per_seg) / kD, d = idx % kD;
+      const int64_t seg = s_pend[j][0];
+      const int w0 = s_pend[j][1], w1 = s_pend[j][2];
+      // four pieces at a time, all their loads in flight together; running (max, sum, out) across batches
+      float m = -INFINITY, wsum = 0.f, o = 0.f;
+      for (int wb = w0; wb <= w1; wb += 4) {
+        float pm[4], ps[4], po[4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int64_t pidx = (min(wb + jj, w1) + seg) * G + head;
+          pm[jj] = load_device_coherent(&p.part_max[pidx]);
+          ps[jj] = load_device_coherent(&p.part_sum[pidx]);
+          po[jj] = load_device_coherent(&p.part_out[pidx * kD + d]);
+        }
+        float bm = pm[0];
+#pragma unroll
+        for (int jj = 1; jj < 4; ++jj) bm = fmaxf(bm, pm[jj]);
+        const float m_new = fmaxf(m, bm);
+        const float keep = __builtin_amdgcn_exp2f(m - m_new);  // 0 for the first batch
+        wsum *= keep;
+        o *= keep;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const float wt = wb + jj <= w1 ? ps[jj] * __builtin_amdgcn_exp2f(pm[jj] - m_new) : 0.f;
+          wsum += wt;
+          o += po[jj] * wt;
+        }
+        m = m_new;
+      }
+      const float r = o / wsum * p.v_scale;
+      // segment = sequence * Hkv + kv head, so (segment * G + head) is (sequence * Hq + query head)
+      const int64_t oi = (seg * G + head) * kD + d;
+      if (p.out_f32)
+        reinterpret_cast<float *>(p.out)[oi] = r;
+      else
+        reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
     }
   }
 }
