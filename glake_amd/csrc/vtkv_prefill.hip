@@ -7,7 +7,7 @@
 //  * A workgroup (four wave64) takes one unit = up to 128/G consecutive query tokens of one sequence
 //    and one kv head, i.e. 128 columns (token, head of the group); a wave owns 32 of them as two
 //    blocks of 16 and walks over ALL rows its columns may see, so there is nothing to merge at the end.
-//  * K and V rows are loaded once per workgroup, 64 rows at a time, as whole rows with ordinary
+//  * K and V rows are loaded once per workgroup, 32 rows at a time, as whole rows with ordinary
 //    (cached) loads into a double-buffered LDS stage in the swizzled tile layouts of the decode kernel;
 //    every wave reads each 16-row tile from LDS once and uses it for both of its column blocks.
 //  * S^T = K_tile . Q^T and O^T += V_tile^T . P^T run on v_mfma_f32_16x16x32_bf16 exactly as in the
@@ -31,9 +31,16 @@ using namespace vtkv_attn;
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
-constexpr int kNB = 2;                        // column blocks of 16 per wave
+#ifndef VTKV_PREFILL_NB
+#define VTKV_PREFILL_NB 2
+#endif
+#ifndef VTKV_PREFILL_KEYS
+#define VTKV_PREFILL_KEYS 32
+#endif
+constexpr int kNB = VTKV_PREFILL_NB;          // column blocks of 16 per wave
 constexpr int kCols = kWaves * kNB * 16;      // columns per workgroup
-constexpr int kKeyBlock = 64;                 // rows per LDS stage
+constexpr int kKeyBlock = VTKV_PREFILL_KEYS;  // rows per LDS stage (32 or 64)
+static_assert(kKeyBlock == 32 || kKeyBlock == 64, "the stage loads cover 32 or 64 rows");
 constexpr int kSub = kKeyBlock / kTile;       // 16-row tiles per stage
 constexpr int kStageBytes = 2 * kKeyBlock * kRowBytes;  // K then V
 
@@ -113,10 +120,10 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     for (int i = 0; i < 8; ++i) acc[nb][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- cooperative stage loads of a 64-row block.  bf16 rows: thread t takes piece t%16 of rows
-  // t/16 + 16j, j < 4.  fp8 rows have 8 pieces of 16 codes: thread t takes piece t%8 of rows t/8 + 32j,
-  // j < 2, and widens it to two bf16 pieces on the way into LDS.
-  constexpr int kLd = FP8 ? 2 : 4;
+  // ---- cooperative stage loads of a block of kKeyBlock rows.  bf16 rows: thread t takes piece t%16 of
+  // rows t/16 + 16j.  fp8 rows have 8 pieces of 16 codes: thread t takes piece t%8 of rows t/8 + 32j and
+  // widens it to two bf16 pieces on the way into LDS.
+  constexpr int kLd = FP8 ? kKeyBlock / 32 : kKeyBlock / 16;
   const int ld_piece = FP8 ? threadIdx.x & 7 : threadIdx.x & 15, ld_row = FP8 ? threadIdx.x >> 3 : threadIdx.x >> 4;
   const int nblocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
   u32x4 kst[kLd], vst[kLd];
