@@ -700,9 +700,10 @@ int vtkv_extend_kv_cache_batch(vtkv_segment *const *segs, int n, const int64_t *
   for (int i = 0; i < n; ++i) SEG_CHECK(segs[i]);
   for (int i = 0; i < n; ++i) {
     vtkv_segment *s = segs[i];
-    // a row that needs a chunk which is being mapped ahead waits for it here
-    if (s->pending && s->used + token_bytes[i] > s->mapped) SEG_SETTLE(s);
     if (set_used_tokens && set_used_tokens[i] > 0) s->used = set_used_tokens[i] * kv_size;
+    // rows that need a chunk which is being mapped ahead wait for it here (a prompt always does: its
+    // reservation looks 100 rows ahead)
+    if (s->pending && (!gen || s->used + token_bytes[i] > s->mapped)) SEG_SETTLE(s);
     slot_m_out[i] = s->used;
     if (gen) {
       int rc = ensure_locked(s, token_bytes[i]);
