@@ -51,12 +51,6 @@
 #ifndef VTKV_ATTN_STAGES
 #define VTKV_ATTN_STAGES 2
 #endif
-// register budget of the streaming kernel: N waves per SIMD (it fits 128 VGPRs with one register tile)
-#ifdef VTKV_ATTN_WAVES_PER_EU
-#define VTKV_ATTN_OCCUPANCY __attribute__((amdgpu_waves_per_eu(VTKV_ATTN_WAVES_PER_EU)))
-#else
-#define VTKV_ATTN_OCCUPANCY
-#endif
 static_assert(VTKV_ATTN_STAGES >= 1 && VTKV_ATTN_STAGES <= 4, "1 to 4 register tiles per wave");
 #include "vtkv_attn_common.h"
 #include "vtkv_fp8.h"
@@ -68,7 +62,7 @@ using namespace vtkv_attn;
 
 constexpr int kWaves = 4;          // waves per workgroup
 constexpr int kThreads = kWaves * 64;
-constexpr int kStages = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
+constexpr int kStagesBf16 = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
 constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
 constexpr int kMinSpan = 4;        // a workgroup takes at least one tile per wave
 constexpr int kDefaultMaxGrid = 4096;  // upper bound of the resident-workgroup grid, sizes the scratch
@@ -125,8 +119,12 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // also stores the row into the cache.  One launch then does reshape_and_cache and attention, and each
 // byte of the new rows is read once.
 template <bool ALIBI, bool FP8, bool APPEND>
-__global__ void VTKV_ATTN_OCCUPANCY __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FP8 ? 3 : 2)))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
+  // An fp8 tile is half the bytes of a bf16 tile for the same chain of dependent steps, so that variant
+  // is bound by latency, not by HBM: it runs three waves per SIMD (it fits 168 registers with one
+  // register tile per wave, refilled as soon as its contents have gone to LDS) instead of two.
+  constexpr int kStages = FP8 ? 1 : kStagesBf16;
   static_assert(!(FP8 && APPEND), "the fused append copies bf16 rows");
   // wave-private V tiles (4 KiB each); reused at the end of a segment for the cross-wave merge
   // then the merge statistics (1 KiB) and the wave-private K tiles
