@@ -51,6 +51,9 @@
 #ifndef VTKV_ATTN_STAGES
 #define VTKV_ATTN_STAGES 2
 #endif
+#ifndef VTKV_ATTN_BF16_WAVES
+#define VTKV_ATTN_BF16_WAVES 2  // waves per SIMD of the bf16 variants (3 spills)
+#endif
 static_assert(VTKV_ATTN_STAGES >= 1 && VTKV_ATTN_STAGES <= 4, "1 to 4 register tiles per wave");
 #include "vtkv_attn_common.h"
 #include "vtkv_fp8.h"
@@ -119,7 +122,7 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // also stores the row into the cache.  One launch then does reshape_and_cache and attention, and each
 // byte of the new rows is read once.
 template <bool ALIBI, bool FP8, bool APPEND>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FP8 ? 3 : 2)))
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FP8 ? 3 : VTKV_ATTN_BF16_WAVES)))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
   // An fp8 tile is half the bytes of a bf16 tile for the same chain of dependent steps, so that variant
   // is bound by latency, not by HBM: it runs three waves per SIMD (it fits 168 registers with one
