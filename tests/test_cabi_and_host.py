@@ -146,15 +146,3 @@ def test_prefill_units_cover_every_query_token_once():
     with pytest.raises(_C.VtkvError):
         prefill_units([5], [4], 4)                                                     # more queries than rows
 
-
-def test_bench_refuses_more_than_one_gpu():
-    """Nothing on this path communicates: the benchmark runs on one GPU and says so when asked for more
-    (the check comes before anything touches a GPU)."""
-    import os
-    import subprocess
-    import sys
-
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
-                         timeout=120)
-    assert res.returncode == 2 and "one GPU" in res.stderr and res.stdout.strip() == ""
