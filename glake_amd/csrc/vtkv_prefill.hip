@@ -10,20 +10,26 @@
 //  * K and V rows are loaded once per workgroup, 32 rows at a time, as whole rows with ordinary
 //    (cached) loads into a double-buffered LDS stage in the swizzled tile layouts of the decode kernel;
 //    every wave reads each 16-row tile from LDS once and uses it for both of its column blocks.
-//  * S^T = K_tile . Q^T and O^T += V_tile^T . P^T run on v_mfma_f32_16x16x32_bf16 exactly as in the
-//    decode kernel (P as bf16 head + tail in one K=32 MFMA, softmax statistics in registers, online
-//    rescale), with each lane applying its column's causal limit to the logits of the tiles that reach it.
+//  * S^T = K_tile . Q^T runs on v_mfma_f32_16x16x32_bf16 as in the decode kernel.  O^T += V^T . P^T runs
+//    on v_mfma_f32_16x16x32_f16 over the stage's 32 rows at once: V is converted to fp16 on its way into
+//    LDS and the softmax weights are rounded to fp16 (2^-12 relative per weight, 16 times finer than the
+//    bf16 weights of flash-attention kernels; the decode kernel's bf16 head + tail is finer still but costs
+//    twice the P.V MFMAs).  bf16 V values convert exactly for magnitudes in [2^-24, 65504]; smaller ones
+//    lose low bits (absolute error below 2^-25), larger ones saturate at 65504.  Softmax statistics live in
+//    registers, each lane applies its column's causal limit to the logits of the stages that reach it.
 //  * The kv head is the fastest index of the grid: with 8 kv heads the workgroups of one kv head all land
 //    on one XCD, whose L2 then serves the re-reads of that head's rows by later query blocks.
 //
-//  * fp8 cache: rows are e4m3fn codes (128 bytes per head row); they are widened to bf16 (exactly) on the
-//    way into the LDS stage, so everything after the stage is the bf16 kernel; the K scale folds into the
-//    logit scale and the V scale into the final normalisation.
+//  * fp8 cache: rows are e4m3fn codes (128 bytes per head row); on the way into the LDS stage K is widened
+//    to bf16 and V to fp16 (both exactly), so everything after the stage is the bf16 kernel; the K scale
+//    folds into the logit scale and the V scale into the final normalisation.
 //
-// Numerics as in the decode kernel (vtkv_attention.hip); the reference computes this with xformers /
+// Otherwise numerics as in the decode kernel (vtkv_attention.hip); the reference computes this with xformers /
 // an external flash-attention kernel (vllm/attention/backends/xformers.py:331-386).
 #include "vtkv_attn_common.h"
 #include "vtkv_common.h"
+
+#include <type_traits>
 
 namespace {
 
@@ -34,14 +40,10 @@ constexpr int kThreads = kWaves * 64;
 #ifndef VTKV_PREFILL_NB
 #define VTKV_PREFILL_NB 2
 #endif
-#ifndef VTKV_PREFILL_KEYS
-#define VTKV_PREFILL_KEYS 32
-#endif
+
 constexpr int kNB = VTKV_PREFILL_NB;          // column blocks of 16 per wave
 constexpr int kCols = kWaves * kNB * 16;      // columns per workgroup
-constexpr int kKeyBlock = VTKV_PREFILL_KEYS;  // rows per LDS stage (32 or 64)
-static_assert(kKeyBlock == 32 || kKeyBlock == 64, "the stage loads cover 32 or 64 rows");
-constexpr int kSub = kKeyBlock / kTile;       // 16-row tiles per stage
+constexpr int kKeyBlock = 32;                 // rows per LDS stage = rows of one P.V reduction (two 16-row tiles)
 constexpr int kStageBytes = 2 * kKeyBlock * kRowBytes;  // K then V
 
 struct PrefillParams {
@@ -57,7 +59,63 @@ struct PrefillParams {
   float v_scale;     // 1 for a bf16 cache
 };
 
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// Two floats to two fp16 in one register.  Round toward zero: a value beyond the fp16 range becomes the
+// largest finite fp16 instead of infinity.
+__device__ __forceinline__ unsigned pack_f16x2_sat(float a, float b) {
+  return __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+// Round to nearest (for the softmax weights, which lie in [0, 256]).
+__device__ __forceinline__ unsigned pack_f16x2(float a, float b) {
+  f16x2 v = {(_Float16)a, (_Float16)b};
+  return __builtin_bit_cast(unsigned, v);
+}
+// l + the two fp16 halves of w, in fp32.
+__device__ __forceinline__ float add_f16x2(unsigned w, float l) {
+  const f16x2 ones = {(_Float16)1.f, (_Float16)1.f};
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, l, false);
+}
+// Maxima as single instructions.  fmaxf() first quiets its operands (one more instruction each) wherever the
+// compiler cannot prove them canonical, which it cannot after selects and lane swaps.
+__device__ __forceinline__ float fmax2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float fmax3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// Maximum over the four row groups of a column: lanes n, n+16, n+32, n+48.
+__device__ __forceinline__ float wave_max_over_row_groups(float v) {
+  float a, b;
+  swap_rows16(v, a, b);
+  swap_rows32(fmax2(a, b), a, b);
+  return fmax2(a, b);
+}
+// Eight bf16 values (one 16-byte piece of a V row) to eight fp16 values.  Exact for magnitudes in
+// [2^-24, 65504]; larger ones saturate.
+__device__ __forceinline__ u32x4 bf16x8_to_f16x8(u32x4 v) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    r[i] = pack_f16x2_sat(__builtin_bit_cast(float, v[i] << 16), __builtin_bit_cast(float, v[i] & 0xffff0000u));
+  return r;
+}
+// Eight e4m3fn codes (two dwords) to eight fp16 values; exact.
+__device__ __forceinline__ u32x4 fp8x8_to_f16x8(unsigned lo, unsigned hi) {
+  u32x4 r;
+  r[0] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false));
+  r[1] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true));
+  r[2] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false));
+  r[3] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true));
+  return r;
+}
 
 template <bool ALIBI, bool FP8>
 __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p) {
@@ -122,133 +180,187 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
 
   // ---- cooperative stage loads of a block of kKeyBlock rows.  bf16 rows: thread t takes piece t%16 of
   // rows t/16 + 16j.  fp8 rows have 8 pieces of 16 codes: thread t takes piece t%8 of rows t/8 + 32j and
-  // widens it to two bf16 pieces on the way into LDS.
+  // widens it to two 16-bit pieces on the way into LDS.  A thread's byte offset into the K range is also
+  // its offset into the V range; it advances by 32 rows per stage and is clamped to the same piece of the
+  // last row (rows past the end are masked for every column in use, so any finite in-bounds data will do).
   constexpr int kLd = FP8 ? kKeyBlock / 32 : kKeyBlock / 16;
   const int ld_piece = FP8 ? threadIdx.x & 7 : threadIdx.x & 15, ld_row = FP8 ? threadIdx.x >> 3 : threadIdx.x >> 4;
   const int nblocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
+  const uint32_t last_off = (uint32_t)(kv_len - 1) * row_stride + ld_piece * 16;
+  const uint32_t stage_step = kKeyBlock * row_stride;
+  uint32_t ld_off[kLd];
+#pragma unroll
+  for (int j = 0; j < kLd; ++j) ld_off[j] = (uint32_t)(j * (kKeyBlock / kLd) + ld_row) * row_stride + ld_piece * 16;
   u32x4 kst[kLd], vst[kLd];
-  auto gload = [&](int kb) {
+  auto gload = [&]() {  // loads the next stage's rows and moves on
 #pragma unroll
     for (int j = 0; j < kLd; ++j) {
-      // rows past the end are redirected to the last row; they are masked for every column in use
-      const int row = min(kb * kKeyBlock + j * (kKeyBlock / kLd) + ld_row, kv_len - 1);
-      const int64_t off = (int64_t)row * row_stride + ld_piece * 16;
+      const uint32_t off = min(ld_off[j], last_off);
       kst[j] = *(gvec)(k_base + off);
       vst[j] = *(gvec)(v_base + off);
+      ld_off[j] += stage_step;
     }
   };
-  auto lstore = [&](int buf) {
-    char *kb_ = smem + buf * kStageBytes, *vb_ = kb_ + kKeyBlock * kRowBytes;
+  // LDS byte offsets that do not depend on the stage, so that the stage's buffer and tile add as immediates
+  int st_k[kLd], st_v[kLd];  // where lstore puts this thread's pieces (fp8: the first of each pair)
+#pragma unroll
+  for (int j = 0; j < kLd; ++j) {
+    if constexpr (FP8) {
+      const int row = j * 32 + ld_row, tile = row >> 4, r = row & 15;
+      st_k[j] = tile * kTile * kRowBytes + k_lds_offset(r, 2 * ld_piece);
+      st_v[j] = kKeyBlock * kRowBytes + tile * kTile * kRowBytes + v_lds_offset(r, 2 * ld_piece);
+    } else {
+      st_k[j] = j * kTile * kRowBytes + k_lds_offset(ld_row, ld_piece);
+      st_v[j] = kKeyBlock * kRowBytes + j * kTile * kRowBytes + v_lds_offset(ld_row, ld_piece);
+    }
+  }
+  auto lstore = [&](auto bufc) {
+    char *base = smem + decltype(bufc)::value * kStageBytes;
 #pragma unroll
     for (int j = 0; j < kLd; ++j) {
       if constexpr (FP8) {
-        const int row = j * 32 + ld_row, tile = row >> 4, r = row & 15;
-        char *kt = kb_ + tile * kTile * kRowBytes, *vt = vb_ + tile * kTile * kRowBytes;
-        *reinterpret_cast<u32x4 *>(kt + k_lds_offset(r, 2 * ld_piece)) = fp8x8_to_bf16x8(kst[j][0], kst[j][1]);
-        *reinterpret_cast<u32x4 *>(kt + k_lds_offset(r, 2 * ld_piece + 1)) = fp8x8_to_bf16x8(kst[j][2], kst[j][3]);
-        *reinterpret_cast<u32x4 *>(vt + v_lds_offset(r, 2 * ld_piece)) = fp8x8_to_bf16x8(vst[j][0], vst[j][1]);
-        *reinterpret_cast<u32x4 *>(vt + v_lds_offset(r, 2 * ld_piece + 1)) = fp8x8_to_bf16x8(vst[j][2], vst[j][3]);
+        // pieces 2p and 2p+1 of a row sit 16 bytes apart before the swizzle, which flips bit 4 or leaves it
+        *reinterpret_cast<u32x4 *>(base + st_k[j]) = fp8x8_to_bf16x8(kst[j][0], kst[j][1]);
+        *reinterpret_cast<u32x4 *>(base + (st_k[j] ^ 16)) = fp8x8_to_bf16x8(kst[j][2], kst[j][3]);
+        *reinterpret_cast<u32x4 *>(base + st_v[j]) = fp8x8_to_f16x8(vst[j][0], vst[j][1]);
+        *reinterpret_cast<u32x4 *>(base + (st_v[j] ^ 16)) = fp8x8_to_f16x8(vst[j][2], vst[j][3]);
       } else {
-        *reinterpret_cast<u32x4 *>(kb_ + j * kTile * kRowBytes + k_lds_offset(ld_row, ld_piece)) = kst[j];
-        *reinterpret_cast<u32x4 *>(vb_ + j * kTile * kRowBytes + v_lds_offset(ld_row, ld_piece)) = vst[j];
+        *reinterpret_cast<u32x4 *>(base + st_k[j]) = kst[j];
+        *reinterpret_cast<u32x4 *>(base + st_v[j]) = bf16x8_to_f16x8(vst[j]);
       }
     }
   };
+  // A operands of S^T = K.Q^T: lane (n, g) takes row n, bytes [16g, +16) of each 64-byte quarter c
+  int ka_off[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) ka_off[c] = k_lds_offset(n, 4 * c + g);
+  // A operands of O^T += V^T.P^T: the lane's transposed quad of dims [16db, +16)
+  int vq_off[8];
+  {
+    const int row = 4 * g + (n >> 2);
+    const int base = kKeyBlock * kRowBytes + row * kRowBytes + ((n & 1) << 3);
+    const int swz = (row & 7) << 1;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) vq_off[db] = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
+  }
+  const float sl = p.scale_log2;
+  // The reference point of the exponentials only follows the running maximum when that has grown by more
+  // than 8 in log2 units (a factor 256 in the weights, harmless in fp32 and fp16): the rescale of the
+  // accumulators, which otherwise runs whenever any of the wave's 32 columns sees a new maximum, becomes
+  // rare.  Without ALiBi the maximum is tracked on the raw dot products (the scale is positive) and the
+  // scale is applied inside the exponent's fused multiply-add.
+  const float lazy = ALIBI ? 8.f : 8.f / sl;
 
-  gload(0);
-  lstore(0);
-  __syncthreads();
-  for (int kb = 0; kb < nblocks; ++kb) {
-    gload(min(kb + 1, nblocks - 1));  // always issued: the last block is loaded once more and not used
-    const char *kstage = smem + (kb & 1) * kStageBytes, *vstage = kstage + kKeyBlock * kRowBytes;
-    for (int sub = 0; sub < kSub; ++sub) {
-      const int t0 = kb * kKeyBlock + sub * kTile;
-      if (t0 >= wave_end) break;  // wave-uniform: nothing this wave's columns may see
-      const char *k_tile = kstage + sub * kTile * kRowBytes, *v_tile = vstage + sub * kTile * kRowBytes;
-      // A operand of S^T = K.Q^T: lane (n, g) takes row n, bytes [16g, +16) of each 64-byte quarter
-      u32x4 ka[4];
+  auto stage = [&](auto bufc, int kb) {
+    constexpr int buf = decltype(bufc)::value;
+    gload();  // always issued: past the last stage it re-reads the last row and nobody uses it
+    const char *st = smem + buf * kStageBytes;
+    const int t0 = kb * kKeyBlock;
+    if (t0 < wave_end) {  // wave-uniform: else nothing this wave's columns may see
+      u32x4 ka[2][4];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) ka[c] = *reinterpret_cast<const u32x4 *>(k_tile + k_lds_offset(n, 4 * c + g));
-      const bool masked = t0 + kTile > wave_first_limit;  // wave-uniform: the tile reaches some column's limit
-      // Order within the tile: all S MFMAs first, then per column block its softmax followed by its P.V
-      // MFMAs, so that the matrix pipe works on one block's P.V while the vector unit does the next
-      // block's softmax.
-      f32x4 sacc[kNB];
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int nb = 0; nb < kNB; ++nb) {
-        sacc[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < 4; ++c)
+          ka[t][c] = *reinterpret_cast<const u32x4 *>(st + t * kTile * kRowBytes + ka_off[c]);
+      const bool masked = t0 + kKeyBlock > wave_first_limit;  // wave-uniform: the stage reaches some column's limit
+      // all S MFMAs first, then per column block its softmax followed by its P.V MFMAs, so that the matrix
+      // pipe works on one block's P.V while the vector unit does the next block's softmax
+      f32x4 sacc[kNB][2];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-          sacc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[ks]), qop[nb][ks], sacc[nb], 0,
-                                                             0, 0);
-      }
-      // transposed V operands, read once for both column blocks
+      for (int nb = 0; nb < kNB; ++nb)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          sacc[nb][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks)
+            sacc[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[t][ks]), qop[nb][ks],
+                                                                  sacc[nb][t], 0, 0, 0);
+        }
+      // reduction slot (g, j) of the K=32 P.V MFMA stands for row 4g+j of the first tile (j < 4) and row
+      // 4g+j-4 of the second (j >= 4), so a lane's A operand is its transposed quad of the first tile
+      // followed by that of the second; read once for both column blocks
       u32x4 vop[8];
-      {
-        const int row = 4 * g + (n >> 2);
-        const int base = row * kRowBytes + ((n & 1) << 3);
-        const int swz = (row & 7) << 1;
 #pragma unroll
-        for (int db = 0; db < 8; ++db) {
-          const int off = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
-          const s16x4 quad =
-              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(v_tile + off));
-          const u32x2 qd = __builtin_bit_cast(u32x2, quad);
-          vop[db] = (u32x4){qd[0], qd[1], qd[0], qd[1]};
-        }
+      for (int db = 0; db < 8; ++db) {
+        const u32x2 qa = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                                       (__attribute__((address_space(3))) s16x4 *)(st + vq_off[db])));
+        const u32x2 qb = __builtin_bit_cast(
+            u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                       (__attribute__((address_space(3))) s16x4 *)(st + kTile * kRowBytes + vq_off[db])));
+        vop[db] = (u32x4){qa[0], qa[1], qb[0], qb[1]};
       }
 #pragma unroll
       for (int nb = 0; nb < kNB; ++nb) {
-        const f32x4 s = sacc[nb];
-        float x[4];
+        // x[4t + r] belongs to row t0 + 16t + 4g + r of the lane's column: with ALiBi the logit in log2
+        // units, else the raw dot product
+        float x[8];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          x[r] = s[r] * p.scale_log2;
-          if (ALIBI) x[r] += slope_log2[nb] * (float)(t0 + 4 * g + r - limit[nb] + 1);
-        }
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            if (ALIBI)
+              x[4 * t + r] = __builtin_fmaf(sacc[nb][t][r], sl,
+                                            slope_log2[nb] * (float)(t0 + 16 * t + 4 * g + r - limit[nb] + 1));
+            else
+              x[4 * t + r] = sacc[nb][t][r];
+          }
         if (masked) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (t0 + 4 * g + r >= limit[nb]) x[r] = -INFINITY;
-        }
-        const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
-        // The reference point of the exponentials only follows the running maximum when that has grown by
-        // more than 8 (a factor 256 in the weights, harmless in fp32): the rescale of the accumulators,
-        // which otherwise runs whenever any of the wave's 32 columns sees a new maximum, becomes rare.
-        const float m_new = tmax > m_run[nb] + 8.f ? tmax : m_run[nb];
-        // (a column can have a whole tile masked; the reference point 0 keeps exp2(-inf - ref) = 0)
-        const float m_ref = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_ref);
-        m_run[nb] = m_new;
-        float pr[4];
+          for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_ref);
-        l_run[nb] = l_run[nb] * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+            for (int r = 0; r < 4; ++r)
+              if (t0 + 16 * t + 4 * g + r >= limit[nb]) x[4 * t + r] = -INFINITY;
+        }
+        const float tmax = wave_max_over_row_groups(fmax2(fmax3(x[0], x[1], x[2]), fmax3(fmax3(x[3], x[4], x[5]), x[6], x[7])));
+        const bool grow = tmax > m_run[nb] + lazy;
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // rare: some column of the block moves its reference point
+          const float m_new = grow ? tmax : m_run[nb];
+          // (a column that has seen only masked rows keeps -inf and rescales its zeros by 1)
+          const float alpha = grow ? __builtin_amdgcn_exp2f(ALIBI ? m_run[nb] - m_new : (m_run[nb] - m_new) * sl) : 1.f;
+          m_run[nb] = m_new;
+          l_run[nb] *= alpha;
 #pragma unroll
           for (int d = 0; d < 8; ++d) acc[nb][d] *= alpha;
         }
-        // P^T as a bf16 head plus a bf16 tail in the two halves of the K=32 reduction (as in decode)
-        float plo[4];
-        u32x4 pb;
-        pb[0] = pack_bf16x2(pr[0], pr[1]);
-        pb[1] = pack_bf16x2(pr[2], pr[3]);
+        // (a column can have everything so far masked; the reference point 0 keeps exp2(-inf - ref) = 0)
+        const float m_ref = m_run[nb] == -INFINITY ? 0.f : m_run[nb];
+        float pr[8];
+        if (ALIBI) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const unsigned hi_bits = (r & 1) ? (pb[r >> 1] & 0xffff0000u) : (pb[r >> 1] << 16);
-          plo[r] = pr[r] - __builtin_bit_cast(float, hi_bits);
+          for (int r = 0; r < 8; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_ref);
+        } else {
+          const float mr = -m_ref * sl;
+#pragma unroll
+          for (int r = 0; r < 8; ++r) pr[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], sl, mr));
         }
-        pb[2] = pack_bf16x2(plo[0], plo[1]);
-        pb[3] = pack_bf16x2(plo[2], plo[3]);
-        const bf16x8 pop = __builtin_bit_cast(bf16x8, pb);
+        // P^T as fp16 (11 significant bits: the rounding stays below 2^-12 relative, which a bf16 P would
+        // miss by a factor 16); the normaliser sums the same rounded weights
+        u32x4 pb;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pb[r] = pack_f16x2(pr[2 * r], pr[2 * r + 1]);
+        float l = l_run[nb];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) l = add_f16x2(pb[r], l);
+        l_run[nb] = l;
+        const f16x8 pop = __builtin_bit_cast(f16x8, pb);
 #pragma unroll
         for (int db = 0; db < 8; ++db)
-          acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[db]), pop, acc[nb][db], 0,
-                                                                0, 0);
+          acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, vop[db]), pop, acc[nb][db], 0, 0,
+                                                               0);
       }
     }
-    lstore((kb + 1) & 1);  // nobody reads that stage: its readers finished before the last barrier
+    // the other stage: its readers finished before the last barrier
+    lstore(std::integral_constant<int, buf ^ 1>{});
     __syncthreads();
+  };
+
+  gload();
+  lstore(std::integral_constant<int, 0>{});
+  __syncthreads();
+  for (int kb = 0; kb < nblocks; kb += 2) {
+    stage(std::integral_constant<int, 0>{}, kb);
+    if (kb + 1 < nblocks) stage(std::integral_constant<int, 1>{}, kb + 1);
   }
 
   // ---- normalise and store: lane (n, g) holds O[column n][d = 16*db + 4g + i]
@@ -294,6 +406,7 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
   VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
   VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
+  VTKV_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
   VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be BF16 or FP8_E4M3");
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   if (fp8) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
@@ -302,7 +415,9 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                    (uintptr_t)out % 16 == 0,
                "q rows must be 16-byte aligned and at least num_heads*head_size apart");
-  VTKV_REQUIRE(max_seq_len > 0 && (int64_t)max_seq_len * num_kv_heads * head_size * 2 < (1ll << 40), "bad max_seq_len");
+  // (the kernel addresses a sequence's rows with 32-bit byte offsets)
+  VTKV_REQUIRE(max_seq_len > 0 && ((int64_t)max_seq_len + 64) * num_kv_heads * head_size * 2 < (1ll << 31),
+               "max_seq_len %d: a sequence's K or V range must stay below 2 GiB", max_seq_len);
   VTKV_REQUIRE((int64_t)num_units * num_kv_heads < (1ll << 31), "too many units");
   if (num_units == 0) return VTKV_OK;
   PrefillParams p;

@@ -97,8 +97,9 @@ def test_long_prompt_needs_several_calls(gpu_pool):
 
 
 def test_prefill_row_equals_decode_of_the_same_position(gpu_pool):
-    """Cross-check without the oracle: every prompt token's output equals (up to fp32 summation order)
-    what decode attention gives for a context cut at that token."""
+    """Cross-check without the oracle: every prompt token's output equals what decode attention gives for
+    a context cut at that token, up to the rounding of the prompt kernel's softmax weights to fp16
+    (2^-12 relative per weight; the decode kernel carries them as a bf16 head and tail, 2^-17)."""
     import torch
 
     from glake_amd import _custom_ops as ops
@@ -117,7 +118,7 @@ def test_prefill_row_equals_decode_of_the_same_position(gpu_pool):
                            t, None, "auto", 1.0, torch.zeros(t, dtype=torch.int64, device="cuda"))
     torch.cuda.synchronize()
     gpu.close()
-    assert (pre - dec).abs().max().item() <= 2e-5 + 2e-5 * dec.abs().max().item()
+    assert (pre - dec).abs().max().item() <= 2e-5 + 2.0 ** -12 * dec.abs().max().item()
 
 
 def test_prompt_behind_a_shared_prefix(gpu_pool):
