@@ -58,7 +58,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 rate
 def prompt_run(args, cfg) -> int:
     """One step = one prompt run of one layer: reshape_and_cache of every prompt row, then causal
     attention of all prompt tokens over the ranges.  Reported in TFLOP/s (4*Hq*D flop per visible
-    (query, key) pair) against the dense bf16 MFMA peak; this kernel is a first version."""
+    (query, key) pair) against the dense bf16 MFMA peak."""
     import torch
 
     from glake_amd import _custom_ops as ops, vmm_allocator as vmm
@@ -125,7 +125,7 @@ def prompt_run(args, cfg) -> int:
         "tokens_per_s": round(n_tok / dt, 1),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "decode_attn_stream_kernel (prefill units)", "avg_call_ms": round(attn_ms, 4),
+                     "kernel": "prefill_attn_kernel", "avg_call_ms": round(attn_ms, 4),
                      "algorithmic_flops_per_call": flops},
     }
     print(json.dumps(result))
