@@ -13,7 +13,8 @@ from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from
 pytestmark = pytest.mark.gpu
 
 
-def run_case(vmm, seed, query_lens, seq_lens, hq, hkv, d=128, alibi=False, fp8=False, tol=2e-3):
+def run_case(vmm, seed, query_lens, seq_lens, hq, hkv, d=128, alibi=False, fp8=False, tol=2e-3, shape_inputs=None,
+             out_scale=1.0):
     import torch
 
     from glake_amd import _custom_ops as ops
@@ -36,9 +37,12 @@ def run_case(vmm, seed, query_lens, seq_lens, hq, hkv, d=128, alibi=False, fp8=F
             k_host[s], v_host[s] = O.fp8_encode(k_f[i], k_scale), O.fp8_encode(v_f[i], v_scale)
         else:
             k_host[s], v_host[s] = bf16_randn(rng, (t, hkv, d)), bf16_randn(rng, (t, hkv, d))
-        gpu.upload(s, k_host[s], v_host[s])
     n_tok = sum(query_lens)
     q = bf16_randn(rng, (n_tok, hq, d))
+    if shape_inputs is not None:  # bf16 bit patterns, edited in place
+        shape_inputs(q, [k_host[int(s)] for s in slots], [v_host[int(s)] for s in slots])
+    for s in slots:
+        gpu.upload(int(s), k_host[int(s)], v_host[int(s)])
     scale = float(d) ** -0.5
     slopes = (rng.standard_normal(hq) * 0.1).astype(np.float32) if alibi else None
     if fp8:  # exact dequantisation in fp32, which is what the kernel computes with
@@ -62,7 +66,7 @@ def run_case(vmm, seed, query_lens, seq_lens, hq, hkv, d=128, alibi=False, fp8=F
     assert np.isfinite(got).all()
     assert np.array_equal(bits_from_torch_bf16(out16), O.f32_to_bf16(got)), "bf16 output is not RNE(fp32 output)"
     err = np.abs(got - expect)
-    bound = tol + tol * np.abs(expect)
+    bound = tol * out_scale + tol * np.abs(expect)   # out_scale: the magnitude of the V values, 1 by default
     worst = np.unravel_index(np.argmax(err - bound), err.shape)
     assert np.all(err <= bound), (f"max err {err.max():.3e} at (token, head, d)={worst}: got {got[worst]!r} "
                                   f"want {expect[worst]!r}")
@@ -164,3 +168,54 @@ def test_prompt_behind_a_shared_prefix(gpu_pool):
     gpu.close()
     assert np.all(np.abs(got - expect) <= 2e-3 + 2e-3 * np.abs(expect))
     assert gpu_pool.sharedBlocks() == 0
+
+
+def test_logit_peaks_move_the_reference_point_mid_sequence(gpu_pool):
+    """Rows whose logits tower over everything before them (by 15 to 60 in log2 units, far beyond the 8 the
+    kernel tolerates before it moves a column's reference point), placed at the start, inside and at the end
+    of stages and growing along the sequence: the accumulators are rescaled several times mid-sequence,
+    for some columns of a wave and not for others (queries before a peak do not see it)."""
+    d = 128
+    u = np.where(np.arange(d) % 3 == 0, -1.0, 1.0).astype(np.float32)
+
+    def peaks(q, ks, vs):
+        qf = O.bf16_to_f32(q)
+        qf += 3.0 * u                                     # every query leans towards u
+        q[...] = O.f32_to_bf16(qf)
+        for k in ks:
+            for pos, c in ((0, 0.1), (31, 0.2), (32, 0.35), (200, 0.55), (333, 0.8), (511, 1.0)):
+                if pos < k.shape[0]:
+                    k[pos] = O.f32_to_bf16(np.broadcast_to(c * u, k[pos].shape))
+
+    run_case(gpu_pool, 7, [512, 90, 300], [512, 90 + 260, 300], 32, 8, shape_inputs=peaks)
+    run_case(gpu_pool, 8, [400], [400], 16, 8, alibi=True, shape_inputs=peaks)
+
+
+def test_large_values_stay_finite(gpu_pool):
+    """V travels as fp16 inside the prompt kernel: values up to 6e4 are exact to bf16 precision there, and
+    a value beyond the fp16 range saturates at 65504 instead of becoming infinite."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    def clip(q, ks, vs):
+        for v in vs:
+            v[...] = O.f32_to_bf16(np.clip(O.bf16_to_f32(v) * 1.5e4, -6.0e4, 6.0e4))
+
+    run_case(gpu_pool, 9, [70, 33], [70, 33 + 64], 32, 8, shape_inputs=clip, out_scale=1.5e4)
+
+    # one key, value 1e5: the output is the saturated value
+    rng = np.random.default_rng(10)
+    hq, hkv = 8, 8
+    gpu = GpuSeqs(gpu_pool, 1, hkv, d := 128, 2, 1)
+    v = O.f32_to_bf16(np.full((1, hkv, d), 1.0e5, np.float32))
+    gpu.upload(0, bf16_randn(rng, (1, hkv, d)), v)
+    kt, vt = gpu.table_tensors()
+    out = torch.empty(1, hq, d, dtype=torch.float32, device="cuda")
+    ops.prefill_attention(out, torch_bf16_from_bits(bf16_randn(rng, (1, hq, d))), kt, vt, hkv, d ** -0.5, [1], [1],
+                          torch.zeros(1, dtype=torch.int64, device="cuda"))
+    torch.cuda.synchronize()
+    gpu.close()
+    # (round toward zero lands on the largest finite fp16)
+    assert torch.all(out == 65504.0)
+
