@@ -231,7 +231,9 @@ def prefill_attention(
         return
     if alibi_slopes is not None:
         alibi_slopes = alibi_slopes.to(device=query.device, dtype=torch.float32)
-    units_t = torch.from_numpy(units).to(query.device)
+    # through pinned memory and without waiting: a copy from pageable memory would hold the host until the
+    # GPU has caught up with everything queued before it
+    units_t = torch.from_numpy(units).pin_memory().to(query.device, non_blocking=True)
     _C.check(lib.vtkv_prefill_attention(
         _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping), _ptr(units_t), len(units),
         num_heads, num_kv_heads, head_size, query.stride(0), float(scale), int(max(seq_lens)), _ptr(alibi_slopes), qd,
