@@ -10,7 +10,8 @@
 // request queue and touches the pool from two threads without a lock, vmm_allocator.cpp:43-48,
 // 222-228); growth in the decode step is done in the calling thread instead of a detached busy-
 // spinning thread signalling through POSIX shared memory (vmm_allocator.cpp:40-72,113-151);
-// failed growth leaves the segment unchanged instead of half-mapped; ranges are freed on destroy.
+// failed growth leaves the segment unchanged instead of half-mapped; the ranges of a destroyed segment
+// are kept for the next segment of the same size and freed with the pool.
 //
 // Unmapping is lazy.  hipMemUnmap costs about 260 us per 2 MiB chunk on this hardware (mapping one
 // costs about 55 us), so a segment that shrinks (preempt, release, swap-out) only gives its chunks
@@ -81,8 +82,29 @@ struct Pool {
     if (worker.joinable()) worker.join();
   }
   std::unordered_set<vtkv_segment *> segments;
+  // Address ranges of destroyed segments, by size, kept for the next segment of that size.  A range is
+  // reserved once and freed when the pool is destroyed: with this runtime, freeing a range and reserving it
+  // again leaves stale bookkeeping behind if the first incarnation had chunks mapped (seen as a crash
+  // inside hipMemAddressFree of the second incarnation, and as hipMemMap failing with "invalid argument").
+  // The reference never frees its ranges at all (vmm_allocator.cpp:177-212).
+  std::unordered_map<int64_t, std::vector<char *>> spare_ranges;
 };
 Pool g_pool;
+
+// An address range of `bytes` for a segment: a spare one of that size, else a new reservation.
+hipError_t take_range_locked(int64_t bytes, char **out) {
+  auto it = g_pool.spare_ranges.find(bytes);
+  if (it != g_pool.spare_ranges.end() && !it->second.empty()) {
+    *out = it->second.back();
+    it->second.pop_back();
+    return hipSuccess;
+  }
+  void *p = nullptr;
+  const hipError_t e = hipMemAddressReserve(&p, bytes, kChunk, nullptr, 0);
+  *out = (char *)p;
+  return e;
+}
+void give_range_locked(char *p, int64_t bytes) { g_pool.spare_ranges[bytes].push_back(p); }
 
 }  // namespace
 }  // namespace vtkv
@@ -117,13 +139,18 @@ int map_chunks_locked(vtkv_segment *s, int n) {
   struct Done { char *va; hipMemGenericAllocationHandle_t h; std::vector<hipMemGenericAllocationHandle_t> *list; };
   std::vector<Done> done;
   hipError_t err = hipSuccess;
+  char where[128] = "";
   for (int l = 0; l < s->layer_num && err == hipSuccess; ++l) {
     for (int j = 0; j < n && err == hipSuccess; ++j) {
       for (int which = 0; which < 2 && err == hipSuccess; ++which) {
         char *va = (which ? s->v_base[l] : s->k_base[l]) + s->held + (int64_t)j * kChunk;
         hipMemGenericAllocationHandle_t h = g_pool.free_chunks.back();
         err = hipMemMap(va, kChunk, 0, h, 0);
-        if (err != hipSuccess) break;
+        if (err != hipSuccess) {
+          snprintf(where, sizeof(where), " (hipMemMap, %s range of layer %d, offset %lld of %lld)", which ? "V" : "K", l,
+                   (long long)(s->held + (int64_t)j * kChunk), (long long)s->context_max);
+          break;
+        }
         g_pool.free_chunks.pop_back();
         auto *list = which ? &s->v_chunks[l] : &s->k_chunks[l];
         list->push_back(h);
@@ -139,7 +166,7 @@ int map_chunks_locked(vtkv_segment *s, int n) {
       it->list->pop_back();
       g_pool.free_chunks.push_back(it->h);
     }
-    return vtkv::fail(VTKV_EHIP, "mapping a chunk failed: %s", hipGetErrorString(err));
+    return vtkv::fail(VTKV_EHIP, "mapping a chunk failed: %s%s", hipGetErrorString(err), where);
   }
   s->held += (int64_t)n * kChunk;
   s->mapped = s->held;
@@ -422,6 +449,9 @@ int vtkv_pool_destroy(void) {
     lk.lock();
     g_pool.stop = false;
   }
+  for (auto &kv : g_pool.spare_ranges)
+    for (char *p : kv.second) VTKV_HIP(hipMemAddressFree(p, kv.first));
+  g_pool.spare_ranges.clear();
   for (auto h : g_pool.free_chunks) VTKV_HIP(hipMemRelease(h));
   g_pool.free_chunks.clear();
   g_pool.total = 0;
@@ -448,25 +478,25 @@ vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t 
   s->k_chunks.resize(layer_num);
   s->v_chunks.resize(layer_num);
   auto unwind = [&](hipError_t e) {
-    for (char *p : s->k_base) (void)hipMemAddressFree(p, context_max_bytes);
-    for (char *p : s->v_base) (void)hipMemAddressFree(p, context_max_bytes);
+    for (char *p : s->k_base) vtkv::give_range_locked(p, context_max_bytes);
+    for (char *p : s->v_base) vtkv::give_range_locked(p, context_max_bytes);
     delete s;
     vtkv::fail(VTKV_EHIP, "hipMemAddressReserve failed: %s", hipGetErrorString(e));
     return (vtkv_segment *)nullptr;
   };
   for (int l = 0; l < layer_num; ++l) {
-    void *k = nullptr, *v = nullptr;
-    hipError_t e = hipMemAddressReserve(&k, context_max_bytes, kChunk, nullptr, 0);
+    char *k = nullptr, *v = nullptr;
+    hipError_t e = vtkv::take_range_locked(context_max_bytes, &k);
     if (e != hipSuccess) return unwind(e);
-    s->k_base.push_back((char *)k);
-    e = hipMemAddressReserve(&v, context_max_bytes, kChunk, nullptr, 0);
+    s->k_base.push_back(k);
+    e = vtkv::take_range_locked(context_max_bytes, &v);
     if (e != hipSuccess) return unwind(e);
-    s->v_base.push_back((char *)v);
+    s->v_base.push_back(v);
   }
   if (expand && expand_bytes > 0) {
     if (expand_locked(s, (int)(expand_bytes / kChunk)) < 0) {
-      for (char *p : s->k_base) (void)hipMemAddressFree(p, context_max_bytes);
-      for (char *p : s->v_base) (void)hipMemAddressFree(p, context_max_bytes);
+      for (char *p : s->k_base) vtkv::give_range_locked(p, context_max_bytes);
+      for (char *p : s->v_base) vtkv::give_range_locked(p, context_max_bytes);
       delete s;
       return nullptr;
     }
@@ -498,8 +528,9 @@ int vtkv_seg_destroy(vtkv_segment *s) {
   int rc = shrink_locked(s, 0);
   if (rc < 0) return rc;
   if (trim_segment_locked(s, 0, -1) < 0) return VTKV_EHIP;
-  for (char *p : s->k_base) VTKV_HIP(hipMemAddressFree(p, s->context_max));
-  for (char *p : s->v_base) VTKV_HIP(hipMemAddressFree(p, s->context_max));
+  // every chunk is unmapped; the ranges wait for the next segment of this size
+  for (char *p : s->k_base) vtkv::give_range_locked(p, s->context_max);
+  for (char *p : s->v_base) vtkv::give_range_locked(p, s->context_max);
   g_pool.segments.erase(s);
   delete s;
   return VTKV_OK;

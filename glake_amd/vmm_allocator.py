@@ -16,6 +16,7 @@ Differences a caller can observe, all deliberate:
 from __future__ import annotations
 
 import ctypes as C
+import sys
 from typing import List, Sequence
 
 import numpy as np
@@ -148,9 +149,10 @@ class KVcacheSegment:
             _C.check(_C.lib().vtkv_seg_destroy(self._h))
             self._h = None
 
-    def __del__(self):  # best effort: the pool may already be gone at interpreter exit
-        try:
-            self.destroy()
+    def __del__(self):  # best effort; at interpreter exit the HIP runtime may be gone already, and the
+        try:            # process gives everything back anyway
+            if not sys.is_finalizing():
+                self.destroy()
         except Exception:
             pass
 
@@ -182,7 +184,8 @@ class KVCache:
 
     def __del__(self):
         try:
-            self.destroy()
+            if not sys.is_finalizing():
+                self.destroy()
         except Exception:
             pass
 

@@ -313,3 +313,37 @@ def test_shared_prefix_maps_whole_chunks_twice_and_copies_the_tail(gpu_pool):
     src.destroy()
     third.destroy()
     assert vmm.showFreeBlocks() == free0 and vmm.retiredBlocks() == 0
+
+
+def test_slots_are_created_and_destroyed_over_and_over(gpu_pool):
+    """Churn: sets of slots of one size are created, some of them written and read, and all destroyed,
+    hundreds of times.  The address ranges of destroyed slots are handed to the next slots of that size,
+    so a slot that was never mapped follows one that was at the same addresses and the other way round
+    (freeing and reserving the ranges anew instead ran into stale bookkeeping of the HIP runtime: a
+    crash inside hipMemAddressFree or a failing hipMemMap after a few cycles)."""
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    free0 = vmm.showFreeBlocks()
+    rng = np.random.default_rng(5)
+    bases = set()
+    for cycle in range(300):
+        size = int(rng.integers(1, 4)) * CHUNK
+        segs = [vmm.KVcacheSegment(1, size, 0, False) for _ in range(6)]
+        for s in segs:
+            bases.add((size, s.getKeyDevicePtr(0)))
+            bases.add((size, s.getValueDevicePtr(0)))
+        used = rng.permutation(6)[:3]
+        for i in used:
+            segs[i].expandMultiSegment(size // CHUNK)
+            payload = rng.integers(0, 256, 4096, dtype=np.uint8)
+            dst = segs[i].getValueDevicePtr(0) + size - 4096
+            _C.check(_C.lib().vtkv_memcpy_h2d(dst, payload.ctypes.data_as(C.c_void_p), 4096))
+            back = np.empty(4096, np.uint8)
+            _C.check(_C.lib().vtkv_memcpy_d2h(back.ctypes.data_as(C.c_void_p), dst, 4096))
+            assert np.array_equal(back, payload)
+        for s in segs:
+            s.destroy()
+        assert vmm.showFreeBlocks() == free0
+    # three sizes, six slots, two ranges each: the same 36 ranges (at most) served all 300 cycles
+    assert len(bases) <= 36
