@@ -19,7 +19,8 @@ pytestmark = pytest.mark.gpu
 ATOL = RTOL = 2e-3
 
 
-def run_case(vmm, seed, seq_lens, hq, hkv, d=128, partition_tokens=0, alibi=False, shuffle_slots=True, version="v1"):
+def run_case(vmm, seed, seq_lens, hq, hkv, d=128, partition_tokens=0, alibi=False, shuffle_slots=True, version="v1",
+             bf16_step_check=True):
     import torch
 
     from glake_amd import _custom_ops as ops
@@ -73,6 +74,8 @@ def run_case(vmm, seed, seq_lens, hq, hkv, d=128, partition_tokens=0, alibi=Fals
     def key(bits):
         b = bits.astype(np.int32)
         return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
+    if not bf16_step_check:
+        return got, want
     steps = np.abs(key(got_bits) - key(expect))
     big = np.abs(expect32) >= 2.0 ** -6   # below that a bf16 step is < 3.1e-5 and the absolute bound rules
     assert steps[big].max(initial=0) <= 1, f"{(steps[big] > 1).sum()} elements differ by more than one bf16 step"

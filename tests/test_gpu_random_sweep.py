@@ -1,0 +1,53 @@
+"""A seeded random sweep of decode and prompt attention against the oracle: head counts (GQA groups 1 to
+16, odd head counts), batch sizes, length mixes (all short, mixed, one very long sequence among short
+ones), fixed partitions and stream-K spans, ALiBi, fp8, and the three merge modes.  Every case builds its
+own sequence slots and destroys them again.  Same tolerances as the dedicated tests; with ALiBi the check
+on bf16 steps is left out (slopes drawn from N(0,1) times positions in the thousands give biases whose
+fp32 rounding alone exceeds a bf16 step of a small output, inside the tolerance on the fp32 values)."""
+import numpy as np
+import pytest
+
+import test_gpu_attention as A
+import test_gpu_prefill_attention as P
+
+pytestmark = pytest.mark.gpu
+
+HEADS = [(32, 8), (64, 8), (8, 8), (16, 1), (12, 4), (8, 2), (16, 16), (48, 8), (128, 8), (7, 7), (10, 2)]
+
+
+@pytest.mark.parametrize("seed", [101, 202, 303])
+def test_random_sweep(gpu_pool, seed):
+    from glake_amd import _C
+
+    lib = _C.lib()
+    rng = np.random.default_rng(seed)
+    try:
+        for case in range(40):
+            hq, hkv = HEADS[rng.integers(len(HEADS))]
+            b = int(rng.integers(1, 24))
+            kind = rng.integers(4)
+            if kind == 0:
+                lens = rng.integers(1, 40, b)
+            elif kind == 1:
+                lens = rng.integers(1, 700, b)
+            elif kind == 2:
+                lens = rng.integers(1, 3000, max(1, b // 3))
+            else:
+                lens = np.concatenate([rng.integers(1, 20, b), rng.integers(2000, 6000, 1)])
+            lens = [int(x) for x in lens]
+            pt = int(rng.choice([0, 0, 0, 64, 128, 256, 512, 1024]))
+            alibi = bool(rng.integers(4) == 0)
+            merge = int(rng.integers(-1, 2))
+            sub = int(rng.integers(1 << 30))
+            _C.check(lib.vtkv_set_fused_merge(merge))
+            print(f"decode case {case}: seed {sub} heads {hq}/{hkv} lens {lens} partition {pt} alibi {alibi} merge {merge}",
+                  flush=True)
+            A.run_case(gpu_pool, sub, lens, hq, hkv, partition_tokens=pt, alibi=alibi, bf16_step_check=not alibi)
+            if rng.integers(3) == 0:
+                seq = [int(x) for x in rng.integers(1, 600, int(rng.integers(1, 6)))]
+                ql = [int(rng.integers(1, s + 1)) if rng.integers(2) else s for s in seq]
+                fp8, al = bool(rng.integers(4) == 0), bool(rng.integers(4) == 0)
+                print(f"prompt case {case}: seed {sub} heads {hq}/{hkv} queries {ql} rows {seq} fp8 {fp8} alibi {al}", flush=True)
+                P.run_case(gpu_pool, sub, ql, seq, hq, hkv, alibi=al, fp8=fp8, tol=3e-2 if fp8 else 2e-3)
+    finally:
+        _C.check(lib.vtkv_set_fused_merge(-1))
