@@ -43,6 +43,7 @@ SIGNATURES = {
     "vtkv_pool_free_chunks": (_i64, []),
     "vtkv_pool_total_chunks": (_i64, []),
     "vtkv_pool_retired_chunks": (_i64, []),
+    "vtkv_pool_recreated_chunks": (_i64, []),
     "vtkv_pool_trim": (_i64, [_i64]),
     "vtkv_pool_destroy": (_i, []),
     "vtkv_seg_create": (_p, [_i, _i64, _i64, _i]),

@@ -67,6 +67,9 @@ struct Pool {
   int64_t retired = 0;  // chunks still mapped at the top of shrunken segments; they count as free
   // chunks that are mapped into more than one segment (shared prefixes): handle -> number of mappings
   std::unordered_map<hipMemGenericAllocationHandle_t, int> shared;
+  // map/unmap cycles a chunk has been through since it was created (see kCyclesPerChunk)
+  std::unordered_map<hipMemGenericAllocationHandle_t, int> cycles;
+  int64_t recreated = 0;
   // map-ahead worker (started on the first request, joined by vtkv_pool_destroy or at exit)
   struct Request { vtkv_segment *seg; int chunks; };
   std::deque<Request> requests;
@@ -173,14 +176,36 @@ int map_chunks_locked(vtkv_segment *s, int n) {
   return VTKV_OK;
 }
 
+// A physical chunk is created anew after this many map/unmap cycles.  The runtime keeps something per
+// (chunk, address) pair a chunk has ever been mapped at and gives it up only with the chunk: a pure HIP
+// program that maps 96 chunks at the top of 250 ranges in turn gets "invalid argument" from
+// hipMemSetAccess and "out of memory" from hipMemCreate after 330 000 mappings with 300 GB free, and
+// runs on without limit when it re-creates its chunks now and then.  A server maps a chunk at a new
+// address at every 2 MiB boundary a sequence crosses, so it would get there within hours.
+constexpr int kCyclesPerChunk = 256;
+
 // One mapping of `h` is gone: the chunk is free again unless another segment still maps it.
 void release_handle_locked(hipMemGenericAllocationHandle_t h) {
   auto it = g_pool.shared.find(h);
-  if (it == g_pool.shared.end()) {
-    g_pool.free_chunks.push_back(h);
-  } else if (--it->second == 1) {
-    g_pool.shared.erase(it);
+  if (it != g_pool.shared.end()) {
+    if (--it->second == 1) g_pool.shared.erase(it);
+    return;
   }
+  if (++g_pool.cycles[h] >= kCyclesPerChunk) {
+    hipMemAllocationProp prop = {};
+    prop.type = hipMemAllocationTypePinned;
+    prop.location.type = hipMemLocationTypeDevice;
+    prop.location.id = g_pool.device;
+    hipMemGenericAllocationHandle_t fresh;
+    // (if the new chunk cannot be had now, the old one serves on and is tried again after its next cycle)
+    if (hipMemCreate(&fresh, kChunk, &prop, 0) == hipSuccess) {
+      g_pool.cycles.erase(h);
+      (void)hipMemRelease(h);
+      h = fresh;
+      ++g_pool.recreated;
+    }
+  }
+  g_pool.free_chunks.push_back(h);
 }
 
 // Physically unmap the retired chunks of `s` at offsets >= max(keep_held, mapped), top down, at most
@@ -414,6 +439,11 @@ int64_t vtkv_pool_free_chunks(void) {
   return (int64_t)g_pool.free_chunks.size() + g_pool.retired;
 }
 
+int64_t vtkv_pool_recreated_chunks(void) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  return g_pool.recreated;
+}
+
 int64_t vtkv_pool_retired_chunks(void) {
   std::unique_lock<std::mutex> lk(g_pool.mu);
   return g_pool.retired;
@@ -454,6 +484,7 @@ int vtkv_pool_destroy(void) {
   g_pool.spare_ranges.clear();
   for (auto h : g_pool.free_chunks) VTKV_HIP(hipMemRelease(h));
   g_pool.free_chunks.clear();
+  g_pool.cycles.clear();
   g_pool.total = 0;
   g_pool.device = -1;
   return VTKV_OK;

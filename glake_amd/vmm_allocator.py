@@ -45,6 +45,11 @@ def sharedBlocks() -> int:
     return int(_C.check(_C.lib().vtkv_pool_shared_chunks()))
 
 
+def recreatedBlocks() -> int:
+    """Physical chunks replaced by new ones so far (each after 256 map/unmap cycles)."""
+    return int(_C.check(_C.lib().vtkv_pool_recreated_chunks()))
+
+
 def retiredBlocks() -> int:
     """Free chunks that are still mapped at the top of a shrunken segment (unmapping is lazy)."""
     return int(_C.check(_C.lib().vtkv_pool_retired_chunks()))

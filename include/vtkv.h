@@ -62,6 +62,10 @@ int vtkv_pool_init(int device, int64_t num_chunks);
 int64_t vtkv_pool_free_chunks(void);
 /* How many of the free chunks are retired, i.e. still mapped.  No counterpart in the reference. */
 int64_t vtkv_pool_retired_chunks(void);
+/* Physical chunks the pool has released and created anew so far: a chunk is replaced after 256 map/unmap
+ * cycles, because the HIP runtime keeps per-chunk state for every address a chunk was ever mapped at and
+ * runs out of it otherwise.  No counterpart in the reference. */
+int64_t vtkv_pool_recreated_chunks(void);
 /* Unmap retired chunks now, until at least `max_chunks` are unmapped or none is left (< 0: all; whole
  * rows, i.e. one chunk of every range of a segment, at a time), so that later growth finds them on the
  * free list; meant for idle moments of the host thread.  Returns the number unmapped, < 0 on error.

@@ -347,3 +347,29 @@ def test_slots_are_created_and_destroyed_over_and_over(gpu_pool):
         assert vmm.showFreeBlocks() == free0
     # three sizes, six slots, two ranges each: the same 36 ranges (at most) served all 300 cycles
     assert len(bases) <= 36
+
+
+def test_chunks_are_replaced_after_many_map_unmap_cycles(gpu_pool):
+    """One slot grows by a chunk and gives it back to the driver 700 times: the chunk on top of the free
+    list goes through all of these cycles and is replaced by a newly created one after every 256 (the
+    HIP runtime runs out of per-chunk state otherwise, after some 10^5 mappings at changing addresses).
+    The books stay balanced and the memory works."""
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    free0, total0, made0 = vmm.showFreeBlocks(), vmm.totalBlocks(), vmm.recreatedBlocks()
+    seg = vmm.KVcacheSegment(1, 2 * CHUNK, 0, False)
+    payload = np.arange(4096, dtype=np.uint8)
+    back = np.empty_like(payload)
+    for cycle in range(700):
+        seg.expandMultiSegment(1)
+        if cycle % 50 == 0:
+            dst = seg.getKeyDevicePtr(0) + CHUNK - 4096
+            _C.check(_C.lib().vtkv_memcpy_h2d(dst, payload.ctypes.data_as(C.c_void_p), 4096))
+            _C.check(_C.lib().vtkv_memcpy_d2h(back.ctypes.data_as(C.c_void_p), dst, 4096))
+            assert np.array_equal(back, payload)
+        seg.preempt_seq(0)
+        assert vmm.trim() == 2            # the K chunk and the V chunk really go back to the driver
+    assert vmm.recreatedBlocks() - made0 >= 4     # two chunks per cycle, each replaced at 256 and 512 cycles
+    seg.destroy()
+    assert vmm.showFreeBlocks() == free0 and vmm.totalBlocks() == total0
