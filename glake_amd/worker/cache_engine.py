@@ -102,12 +102,24 @@ class CacheEngine:
         stream, then unmap the slots (their chunks return to the pool).  Returns bytes moved."""
         src, dst, nbytes = [], [], []
         total = 0
+        if len(set(slots)) != len(slots):
+            raise _C.VtkvError(_C.EINVAL, "swap_out: a slot is listed twice")
         for slot in slots:
             if slot in self._swapped:
                 raise _C.VtkvError(_C.ESTATE, f"slot {slot} is already swapped out")
+        # room for all of them first: a full arena must leave every slot as it was
+        placed: List[Tuple[int, int, int]] = []
+        try:
+            for slot in slots:
+                used = self.vmm_kvcache_segment[slot].used_size
+                placed.append((slot, self._arena.alloc(2 * self.num_layers * used) if used else 0, used))
+        except _C.VtkvError:
+            for _, off, used in placed:
+                if used:
+                    self._arena.release(off, 2 * self.num_layers * used)
+            raise
+        for slot, off, used in placed:
             seg = self.vmm_kvcache_segment[slot]
-            used = seg.used_size
-            off = self._arena.alloc(2 * self.num_layers * used) if used else 0
             self._swapped[slot] = (off, used)
             for l in range(self.num_layers):
                 for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):

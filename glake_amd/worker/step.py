@@ -26,7 +26,8 @@ def prepare_step(attn_metadata, kv_caches: Sequence) -> None:
         decode_seq_len = None
     else:
         # llama.py:321-337: the reference spins on its background mapper here and then queues
-        # eagerExtend requests; mapping is synchronous in this library, so only the requests remain
+        # eagerExtend requests; here a row that needs a chunk which is still being mapped waits inside
+        # extend_kv_cache_batch, so only the requests remain
         decode_seq_len = torch.ones(n, dtype=torch.int32, device=attn_metadata.slot_mapping.device)
         kv_size_list = [kv_size] * n
         for idx, slot_id in enumerate(attn_metadata.extend_seq_list):

@@ -118,3 +118,50 @@ def test_swap_ranges_piece_and_stream_variants_are_exact(gpu_pool):
         torch.cuda.synchronize()
         assert torch.equal(src, back)
     _C.check(_C.lib().vtkv_host_free(C.c_void_p(host)))
+
+
+def test_swap_out_into_a_full_arena_changes_nothing(gpu_pool):
+    """The host arena holds one of two sequences: swapping both out fails as a whole, both stay resident
+    with their bytes, the arena stays empty, and each can still be swapped out (and in) alone."""
+    import torch
+
+    from glake_amd import _C
+    from glake_amd.worker.cache_engine import CacheEngine
+
+    hkv, d = 8, 128
+    row = hkv * d * 2
+    eng = CacheEngine(num_layers=2, num_kv_heads=hkv, head_size=d, dtype=torch.bfloat16, max_num_seqs=2,
+                      max_num_batched_tokens=600, swap_space_bytes=2 * 2 * 300 * row + 4096)
+    rng = np.random.default_rng(3)
+    data = {}
+    for slot, tokens in ((0, 300), (1, 250)):
+        seg = eng.vmm_kvcache_segment[slot]
+        seg.expandMultiSegment(1)
+        seg.set_used_size(tokens * row)
+        for l in range(2):
+            for which, base in (("k", seg.getKeyDevicePtr(l)), ("v", seg.getValueDevicePtr(l))):
+                buf = rng.integers(0, 256, tokens * row, dtype=np.uint8)
+                _C.check(_C.lib().vtkv_memcpy_h2d(base, buf.ctypes.data, buf.nbytes))
+                data[(slot, l, which)] = buf
+
+    def resident_bytes_intact():
+        for (slot, l, which), buf in data.items():
+            seg = eng.vmm_kvcache_segment[slot]
+            base = seg.getKeyDevicePtr(l) if which == "k" else seg.getValueDevicePtr(l)
+            back = np.empty_like(buf)
+            _C.check(_C.lib().vtkv_memcpy_d2h(back.ctypes.data, base, buf.nbytes))
+            assert np.array_equal(back, buf), (slot, l, which)
+
+    with pytest.raises(_C.VtkvOutOfChunks):
+        eng.swap_out([0, 1])
+    assert eng._swapped == {} and eng._arena.free == [(0, eng._arena.nbytes)]
+    assert [s.actual_size for s in eng.vmm_kvcache_segment] == [2 << 20, 2 << 20]
+    resident_bytes_intact()
+    with pytest.raises(_C.VtkvError):
+        eng.swap_out([0, 0])
+    for slot in (0, 1):
+        eng.swap_out([slot])
+        assert eng.vmm_kvcache_segment[slot].actual_size == 0
+        eng.swap_in([slot])
+    resident_bytes_intact()
+    eng.close()
