@@ -56,16 +56,24 @@ def _require_cuda(*tensors) -> None:
             raise _C.VtkvError(_C.EINVAL, "tensor must live on the GPU")
 
 
-# scratch for the attention's partial results, grown on demand, one per device.  The library wants it
-# zero-filled before its first use (it keeps arrival counters there that it resets itself).
+# Scratch for the attention's partial results, grown on demand: one per device and stream, because calls
+# that run at the same time must not share it (they would mix their partial results and arrival counters).
+# The library wants it zero-filled before its first use (it keeps the counters there and resets them itself).
 _workspaces = {}
 
 
 def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
-    ws = _workspaces.get(device)
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None and torch.cuda.is_current_stream_capturing():
+        # a graph is being recorded: use the scratch an eager call on this device has made before, so that the
+        # graph neither allocates nor clears 35 MiB at every replay (replay it on that call's stream)
+        for (dev, _), other in _workspaces.items():
+            if dev == device and other.numel() >= nbytes:
+                return other
     if ws is None or ws.numel() < nbytes:
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[device] = ws
+        _workspaces[key] = ws
     return ws
 
 

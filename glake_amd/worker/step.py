@@ -103,7 +103,8 @@ class DecodeStepPlan:
         self._recorded = [False, False]
         self._row = 0
         need = self._lib.vtkv_decode_attention_workspace_bytes(n, self.num_heads, self.head_size, 1, 0)
-        self._ws = ops._workspace(need, self.device)
+        # its own scratch (zero-filled once, as the library asks): plans may run on different streams at once
+        self._ws = torch.zeros(max(int(need), 1 << 20), dtype=torch.uint8, device=self.device)
         self._ws_p, self._ws_n = C.c_void_p(self._ws.data_ptr()), self._ws.numel()
         self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
         self.fused = bool(fused) and self._kv_dt == _C.BF16 and self._src_dt == _C.BF16

@@ -146,3 +146,50 @@ def test_merge_inside_and_outside_the_kernel(gpu_pool, mode):
         run_case(gpu_pool, 1001, rng.integers(512, 4097, 64).tolist(), 32, 8)
     finally:
         _C.check(lib.vtkv_set_fused_merge(-1))
+
+
+def test_calls_on_two_streams_do_not_share_scratch(gpu_pool):
+    """Two batches attend at the same time on two streams, twenty times over; each result equals the one
+    the same call gives when it runs alone (the wrapper keeps one scratch buffer per device and stream)."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(21)
+    hq, hkv, d = 32, 8, 128
+    scale = d ** -0.5
+    batches = []
+    for lens in ([900, 1500, 700, 64, 2100], [1300, 40, 1800, 1000]):
+        gpu = GpuSeqs(gpu_pool, len(lens), hkv, d, 2, max(lens))
+        for i, t in enumerate(lens):
+            gpu.upload(i, bf16_randn(rng, (t, hkv, d)), bf16_randn(rng, (t, hkv, d)))
+        kt, vt = gpu.table_tensors()
+        q = torch_bf16_from_bits(bf16_randn(rng, (len(lens), hq, d)))
+        sl = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        slot = torch.arange(len(lens), dtype=torch.int64, device="cuda")
+        batches.append(dict(gpu=gpu, kt=kt, vt=vt, q=q, sl=sl, slot=slot, max=max(lens),
+                            out=torch.empty(len(lens), hq, d, dtype=torch.float32, device="cuda")))
+
+    def attend(b, out):
+        ops.paged_attention_v1(out, b["q"], b["kt"], b["vt"], hkv, scale, b["sl"], 1, b["max"], None, "auto", 1.0,
+                               b["slot"])
+
+    alone = []
+    for b in batches:
+        ref = torch.empty_like(b["out"])
+        attend(b, ref)
+        alone.append(ref)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for _ in range(20):
+        for b, st in zip(batches, streams):
+            b["out"].fill_(float("nan"))
+        torch.cuda.synchronize()
+        for b, st in zip(batches, streams):
+            with torch.cuda.stream(st):
+                attend(b, b["out"])
+        torch.cuda.synchronize()
+        for b, ref in zip(batches, alone):
+            assert torch.equal(b["out"], ref)
+    for b in batches:
+        b["gpu"].close()
