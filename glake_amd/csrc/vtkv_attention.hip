@@ -65,6 +65,10 @@ using namespace vtkv_attn;
 
 constexpr int kWaves = 4;          // waves per workgroup
 constexpr int kThreads = kWaves * 64;
+#ifndef VTKV_ATTN_FP8_STAGES
+#define VTKV_ATTN_FP8_STAGES 1
+#endif
+constexpr int kStagesFp8 = VTKV_ATTN_FP8_STAGES;  // likewise for the fp8 variant (see the kernel)
 constexpr int kStagesBf16 = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
 constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
 constexpr int kMinSpan = 4;        // a workgroup takes at least one tile per wave
@@ -127,7 +131,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
   // An fp8 tile is half the bytes of a bf16 tile for the same chain of dependent steps, so that variant
   // is bound by latency, not by HBM: it runs three waves per SIMD (it fits 168 registers with one
   // register tile per wave, refilled as soon as its contents have gone to LDS) instead of two.
-  constexpr int kStages = FP8 ? 1 : kStagesBf16;
+  constexpr int kStages = FP8 ? kStagesFp8 : kStagesBf16;
   static_assert(!(FP8 && APPEND), "the fused append copies bf16 rows");
   // wave-private V tiles (4 KiB each); reused at the end of a segment for the cross-wave merge
   // then the merge statistics (1 KiB) and the wave-private K tiles
