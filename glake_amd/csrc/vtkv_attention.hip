@@ -634,33 +634,66 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
 // Merge the partials of one (sequence, head): out = sum_j o_j w_j / sum_j w_j with
 // w_j = l_j * 2^(m_j - max m)  (csrc/attention/attention_kernels.cu:515-582).  The segment's tiles
 // [first, first + nt) of the global order were handled by workgroups first/span .. (first+nt-1)/span.
+// One workgroup per (kv head, sequence), thread d; the group's heads are taken four at a time and the
+// pieces four at a time, so that up to 48 loads of a thread are in flight together: the kernel is a chain
+// of three or four memory round trips (tile counts, then statistics and partial outputs of a batch), and
+// with one small workgroup per query head it was that chain times many more workgroups.
 __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
-  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const int G = p.group, Hkv = p.num_kv_heads;
   const int cum_b = p.cum_tiles[b];
   const int nt = p.cum_tiles[b + 1] - cum_b;
   if (nt <= 0) return;
   const int total_tiles = p.cum_tiles[p.num_seqs] * Hkv;
   const int span = span_of(p, total_tiles);
-  const int kvh = head / G, hg = head % G;
   const int first = cum_b * Hkv + kvh * nt;
   const int w0 = first / span, w1 = (first + nt - 1) / span;
   const int64_t seg = (int64_t)b * Hkv + kvh;
-  float m = -INFINITY;
-  for (int w = w0; w <= w1; ++w) m = fmaxf(m, p.part_max[(w + seg) * G + hg]);
-  float wsum = 0.f, o = 0.f;
-  for (int w = w0; w <= w1; ++w) {
-    const int64_t pidx = (w + seg) * G + hg;
-    const float wt = p.part_sum[pidx] * __builtin_amdgcn_exp2f(p.part_max[pidx] - m);
-    wsum += wt;
-    o += p.part_out[pidx * kD + d] * wt;
+  for (int h0 = 0; h0 < G; h0 += 4) {
+    float m[4], wsum[4], o[4];
+#pragma unroll
+    for (int hh = 0; hh < 4; ++hh) m[hh] = -INFINITY, wsum[hh] = 0.f, o[hh] = 0.f;
+    for (int wb = w0; wb <= w1; wb += 4) {
+      float pm[4][4], ps[4][4], po[4][4];
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+        for (int hh = 0; hh < 4; ++hh) {
+          // (pieces and heads past the end repeat the last one; their weights are set to zero below)
+          const int64_t pidx = (min(wb + jj, w1) + seg) * G + min(h0 + hh, G - 1);
+          pm[jj][hh] = p.part_max[pidx];
+          ps[jj][hh] = p.part_sum[pidx];
+          po[jj][hh] = p.part_out[pidx * kD + d];
+        }
+#pragma unroll
+      for (int hh = 0; hh < 4; ++hh) {
+        float bm = pm[0][hh];
+#pragma unroll
+        for (int jj = 1; jj < 4; ++jj) bm = fmaxf(bm, pm[jj][hh]);
+        const float m_new = fmaxf(m[hh], bm);
+        const float keep = __builtin_amdgcn_exp2f(m[hh] - m_new);  // 0 for the first batch
+        wsum[hh] *= keep;
+        o[hh] *= keep;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const float wt = wb + jj <= w1 ? ps[jj][hh] * __builtin_amdgcn_exp2f(pm[jj][hh] - m_new) : 0.f;
+          wsum[hh] += wt;
+          o[hh] += po[jj][hh] * wt;
+        }
+        m[hh] = m_new;
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < 4; ++hh) {
+      if (h0 + hh >= G) break;
+      const float r = o[hh] / wsum[hh] * p.v_scale;
+      const int64_t oi = ((int64_t)b * p.num_heads + kvh * G + h0 + hh) * kD + d;
+      if (p.out_f32)
+        reinterpret_cast<float *>(p.out)[oi] = r;
+      else
+        reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
+    }
   }
-  const float r = o / wsum * p.v_scale;
-  const int64_t oi = ((int64_t)b * p.num_heads + head) * kD + d;
-  if (p.out_f32)
-    reinterpret_cast<float *>(p.out)[oi] = r;
-  else
-    reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
 }
 
 // Optional per-kernel timing for benchmarks: when switched on, every vtkv_decode_attention call
@@ -847,7 +880,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, p, il);
   if (timed) VTKV_HIP(hipEventRecord(ev[1], st));
   if (!p.fused_merge)
-    hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_heads, num_seqs), dim3(kD), 0, st, p);
+    hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_kv_heads, num_seqs), dim3(kD), 0, st, p);
   if (timed) {
     VTKV_HIP(hipEventRecord(ev[2], st));
     ++g_timer.calls;
