@@ -135,13 +135,18 @@ def decode_append_attention(
     alibi_slopes: Optional[torch.Tensor],
     slot_mapping: torch.Tensor,
     partition_tokens: int = 0,
+    kv_cache_dtype: str = "auto",
+    kv_scale: float = 1.0,
+    v_scale: Optional[float] = None,
 ) -> None:
     """One launch for the two calls a decode step makes per layer, ``reshape_and_cache`` then
     ``paged_attention_v1`` (vllm/attention/backends/xformers.py:310-312 and :357-371): ``key`` /
     ``value`` hold one new row per sequence, ``seq_lens`` counts it, the row lands at position
     ``seq_lens[b] - 1`` of sequence b's ranges and attention runs over all ``seq_lens[b]`` rows.
     ``seq_lens`` is an int32 GPU tensor, or a host sequence of at most 512 ints (then nothing is
-    uploaded).  bf16 cache only.  No counterpart as a single op in the reference."""
+    uploaded).  The cache is bf16, or fp8 (``kv_cache_dtype="fp8"`` with ``kv_scale`` / ``v_scale``: the row is
+    stored quantised exactly as ``reshape_and_cache`` stores it).  No counterpart as a single op in the
+    reference."""
     _require_cuda(out, query, key, value, slot_mapping)
     num_seqs, num_heads, head_size = query.shape
     if not out.is_contiguous():
@@ -172,8 +177,9 @@ def decode_append_attention(
     _C.check(lib.vtkv_decode_append_attention(
         _ptr(out), _ptr(query), _ptr(key), _ptr(value), key.stride(0), value.stride(0), _ptr(key_cache),
         _ptr(value_cache), _ptr(slot_mapping), dev_lens, host_lens, num_seqs, num_heads, num_kv_heads, head_size,
-        query.stride(0), float(scale), int(max_seq_len), _ptr(alibi_slopes), qd, _dt(out), _dt(key), _ptr(ws),
-        ws.numel(), int(partition_tokens), _stream()))
+        query.stride(0), float(scale), int(max_seq_len), _ptr(alibi_slopes), qd, _dt(out),
+        _kv_dtype(kv_cache_dtype, _dt(key)), float(kv_scale), float(kv_scale if v_scale is None else v_scale),
+        _ptr(ws), ws.numel(), int(partition_tokens), _stream()))
 
 
 def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], per_unit: int):

@@ -140,7 +140,7 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
                              f"Supported head sizes are: {supported}.")
         if sliding_window is not None:
             raise ValueError("sliding-window attention is not supported by the vtensor backend")
-        # one launch for cache write + attention in pure decode steps on a bf16 cache; False = two launches
+        # one launch for cache write + attention in pure decode steps; False = two launches
         self.fuse_decode_append = True
 
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, key_cache, value_cache,
@@ -153,9 +153,8 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
         vs = kv_scale if v_scale is None else v_scale
 
         if (self.fuse_decode_append and key_cache is not None and attn_metadata.num_prefill_tokens == 0
-                and attn_metadata.decode_metadata is not None and self.kv_cache_dtype == "auto"
-                and query.dtype == torch.bfloat16):
-            # A pure decode step on a bf16 cache: the cache write (xformers.py:310-312) and the decode
+                and attn_metadata.decode_metadata is not None and query.dtype == torch.bfloat16):
+            # A pure decode step: the cache write (xformers.py:310-312) and the decode
             # attention (:357-371) are one launch.  The row goes to position seq_len - 1 of each range,
             # which is where slot_m points in the reference's flow (llama.py:340: the bytes used before
             # this step).
@@ -165,7 +164,7 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
                 output, query, key, value, attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
                 attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], self.num_kv_heads, self.scale,
                 attn_metadata.seq_lens_tensor, attn_metadata.max_seq_len, self.alibi_slopes,
-                attn_metadata.slot_mapping)
+                attn_metadata.slot_mapping, kv_cache_dtype=self.kv_cache_dtype, kv_scale=kv_scale, v_scale=vs)
             return output.view(-1, self.num_heads * self.head_size)
 
         if key_cache is not None:

@@ -101,6 +101,7 @@ struct AttnParams {
   // fused append: the step's new K/V rows, one per sequence, row b at new_k + b * new_k_stride (bytes)
   const char *new_k, *new_v;
   int64_t new_k_stride, new_v_stride;
+  float k_quant, v_quant;  // fp8 cache: the new rows are stored as e4m3fn(x / k_quant), e4m3fn(x / v_quant)
   int inline_lens;  // sequence lengths come with the kernel arguments instead of from seq_lens
 };
 
@@ -132,7 +133,6 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
   // is bound by latency, not by HBM: it runs three waves per SIMD (it fits 168 registers with one
   // register tile per wave, refilled as soon as its contents have gone to LDS) instead of two.
   constexpr int kStages = FP8 ? kStagesFp8 : kStagesBf16;
-  static_assert(!(FP8 && APPEND), "the fused append copies bf16 rows");
   // wave-private V tiles (4 KiB each); reused at the end of a segment for the cross-wave merge
   // then the merge statistics (1 KiB) and the wave-private K tiles
   __shared__ __attribute__((aligned(16))) char smem[2 * kWaves * kTile * kRowBytes + 1024];
@@ -278,7 +278,12 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
     // whole rows per load (fp8 rows are 128 bytes: a load then covers eight rows, lane l takes row
     // 8j + l/8, piece l%8).
     uint32_t t_off[kLoads], t_off_last[kLoads];
-    const uint32_t t_off_new = n * 16;  // the new row's tile: every row slot holds the one new row
+    // The new row's tile.  bf16 cache: every row slot holds the one new row, lane (g, n) its piece n.
+    // fp8 cache: the new row arrives as bf16 and is quantised in consume(): a lane's two loads fetch the
+    // two bf16 pieces that become its 16 codes, pieces 2*(lane%8) and 2*(lane%8)+1 of the 256-byte row.
+    uint32_t t_off_new[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) t_off_new[j] = FP8 ? ((lane & 7) * 2 + j) * 16 : n * 16;
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
       const int row = FP8 ? 8 * j + (lane >> 3) : 4 * j + g;
@@ -304,7 +309,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
 #pragma unroll
       for (int j = 0; j < kLoads; ++j) {
         uint32_t off = (last ? t_off_last[j] : t_off[j]) & mask;
-        if (APPEND) off |= t_off_new & mask_new;
+        if (APPEND) off |= t_off_new[j] & mask_new;
         regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off));
       }
     };
@@ -317,7 +322,37 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
       const bool is_new = APPEND && has_new && tile == seg_tiles - 1;
       const int t0 = is_new ? seq_len - 1 : seg_start + tile * kTile;                  // position of the tile's row 0
       const int valid = is_new ? 1 : (tile == n_tiles - 1 ? valid_last : kTile);       // rows that count
-      if (APPEND && is_new && g == 0) {
+      if constexpr (APPEND && FP8) {
+        if (is_new) {
+          // the lane's sixteen new bf16 values of K and of V become e4m3fn codes, as scatter_rows_fp8_kernel
+          // makes them (IEEE division by the scale, round to nearest even, saturate); the codes take the place
+          // of a loaded tile whose rows all hold the new row, and lanes 0..7 append them to the cache
+          auto quantise = [](const u32x4 &a, const u32x4 &b, float sc) {
+            u32x4 c;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              const u32x4 &src = w < 2 ? a : b;
+              uint32_t word = 0;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const uint32_t pair = src[(2 * w + e / 2) & 3];
+                const float x = __builtin_bit_cast(float, (e & 1) ? (pair & 0xffff0000u) : (pair << 16));
+                word |= (uint32_t)vtkv::fp8_e4m3fn_encode(x / sc) << (8 * e);
+              }
+              c[w] = word;
+            }
+            return c;
+          };
+          kreg[0] = kreg[1] = quantise(kreg[0], kreg[1], p.k_quant);
+          vreg[0] = vreg[1] = quantise(vreg[0], vreg[1], p.v_quant);
+          if (lane < 8) {
+            typedef __attribute__((address_space(1))) u32x4 *gvec_rw;
+            const int64_t dst = (int64_t)(seq_len - 1) * row_stride + lane * 16;
+            *(gvec_rw)((uintptr_t)k_base + dst) = kreg[0];
+            *(gvec_rw)((uintptr_t)v_base + dst) = vreg[0];
+          }
+        }
+      } else if (APPEND && is_new && g == 0) {
         // lanes 0..15 hold the sixteen 16-byte pieces of the new K and V rows: append them to the cache
         typedef __attribute__((address_space(1))) u32x4 *gvec_rw;
         const int64_t dst = (int64_t)(seq_len - 1) * row_stride + n * 16;
@@ -708,7 +743,7 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 6;  // instantiations of the streaming kernel
+constexpr int kVariants = 8;  // instantiations of the streaming kernel
 struct Residency {
   std::mutex mu;
   int device = -1;
@@ -785,7 +820,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
                "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
   if (append) {
     VTKV_REQUIRE(new_value != nullptr, "null argument");
-    VTKV_REQUIRE(kv_dtype == VTKV_BF16, "the fused append needs a bf16 cache (use vtkv_reshape_and_cache for fp8)");
+    VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "the fused append needs a bf16 or fp8 cache");
     const int64_t row = (int64_t)num_kv_heads * head_size;
     VTKV_REQUIRE(key_stride >= row && value_stride >= row && key_stride % 8 == 0 && value_stride % 8 == 0 &&
                      (uintptr_t)new_key % 16 == 0 && (uintptr_t)new_value % 16 == 0,
@@ -795,8 +830,8 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
 
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   const bool alibi = alibi_slopes != nullptr;
-  // kernel variant: bit 0 fp8, bit 1 alibi, 4 + alibi for the fused append
-  const int variant = append ? 4 + (alibi ? 1 : 0) : (alibi ? 2 : 0) + (fp8 ? 1 : 0);
+  // kernel variant: bit 0 fp8, bit 1 alibi, bit 2 fused append
+  const int variant = (append ? 4 : 0) + (alibi ? 2 : 0) + (fp8 ? 1 : 0);
   void (*kernel)(AttnParams, InlineLens) = nullptr;
   switch (variant) {
     case 0: kernel = decode_attn_stream_kernel<false, false, false>; break;
@@ -804,7 +839,9 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
     case 2: kernel = decode_attn_stream_kernel<true, false, false>; break;
     case 3: kernel = decode_attn_stream_kernel<true, true, false>; break;
     case 4: kernel = decode_attn_stream_kernel<false, false, true>; break;
-    default: kernel = decode_attn_stream_kernel<true, false, true>; break;
+    case 5: kernel = decode_attn_stream_kernel<false, true, true>; break;
+    case 6: kernel = decode_attn_stream_kernel<true, false, true>; break;
+    default: kernel = decode_attn_stream_kernel<true, true, true>; break;
   }
   int64_t grid;
   if (partition_tokens > 0) {
@@ -861,6 +898,8 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.new_v = (const char *)new_value;
   p.new_k_stride = key_stride * 2;
   p.new_v_stride = value_stride * 2;
+  p.k_quant = k_scale;
+  p.v_quant = v_scale;
   p.inline_lens = host_seq_lens != nullptr;
   InlineLens il;
   if (host_seq_lens) memcpy(il.v, host_seq_lens, (size_t)num_seqs * sizeof(int32_t));
@@ -921,12 +960,13 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
                                  const int64_t *slot_ids, const int32_t *seq_lens, const int32_t *host_seq_lens,
                                  int num_seqs, int num_heads, int num_kv_heads, int head_size, int64_t q_stride,
                                  float scale, int max_seq_len, const float *alibi_slopes, int q_dtype, int out_dtype,
-                                 int kv_dtype, void *workspace, int64_t workspace_bytes, int partition_tokens,
-                                 void *stream) {
+                                 int kv_dtype, float k_scale, float v_scale, void *workspace, int64_t workspace_bytes,
+                                 int partition_tokens, void *stream) {
   VTKV_REQUIRE(key && value, "null argument");
   return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, host_seq_lens, num_seqs, num_heads, num_kv_heads,
-                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, 1.f, 1.f,
-                        workspace, workspace_bytes, partition_tokens, stream, key, value, key_stride, value_stride);
+                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
+                        v_scale, workspace, workspace_bytes, partition_tokens, stream, key, value, key_stride,
+                        value_stride);
 }
 
 int vtkv_set_fused_merge(int on) {

@@ -51,7 +51,7 @@ class DecodeStepPlan:
     (``vtkv_extend_kv_cache_batch``, ``vtkv_reshape_and_cache``, ``vtkv_decode_attention``); what the
     plan saves is per-call Python: argument arrays, the device tables and the pinned staging ring are
     made once, the bookkeeping writes its offsets straight into pinned memory, and both metadata arrays
-    travel in one asynchronous copy.  With a bf16 cache and ``fused=True`` the append and the attention
+    travel in one asynchronous copy.  With ``fused=True`` (bf16 or fp8 cache) the append and the attention
     are one launch (``vtkv_decode_append_attention``) and, up to 512 sequences, the lengths travel with the
     kernel arguments, so a step is two kernels (attention and its merge) and no copy.  Build a new plan
     when the set of running sequences changes.
@@ -107,7 +107,7 @@ class DecodeStepPlan:
         self._ws = torch.zeros(max(int(need), 1 << 20), dtype=torch.uint8, device=self.device)
         self._ws_p, self._ws_n = C.c_void_p(self._ws.data_ptr()), self._ws.numel()
         self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
-        self.fused = bool(fused) and self._kv_dt == _C.BF16 and self._src_dt == _C.BF16
+        self.fused = bool(fused) and self._src_dt == _C.BF16 and self._kv_dt in (_C.BF16, _C.FP8_E4M3)
         self._inline = self.fused and n <= 512
         self._host_lens_p = [C.c_void_p(self._stage[i].data_ptr() + 8 * n) for i in range(ring)]
 
@@ -138,8 +138,8 @@ class DecodeStepPlan:
                 C_void_p(out.data_ptr()), C_void_p(query.data_ptr()), C_void_p(key.data_ptr()),
                 C_void_p(value.data_ptr()), key.stride(0), value.stride(0), self._k_table, self._v_table,
                 self._slot_p, None, self._host_lens_p[i], n, self.num_heads, self.num_kv_heads, self.head_size,
-                query.stride(0), self.scale, max_len, alibi_p, self._src_dt, out_dt, self._kv_dt, self._ws_p,
-                self._ws_n, 0, stream))
+                query.stride(0), self.scale, max_len, alibi_p, self._src_dt, out_dt, self._kv_dt, self.k_scale,
+                self.v_scale, self._ws_p, self._ws_n, 0, stream))
             return max_len
         check(lib.vtkv_memcpy_h2d_async(self._meta_addr, self._row_p[i], 12 * n, stream))
         if i == half - 1 or i == self._ring - 1:
@@ -151,8 +151,8 @@ class DecodeStepPlan:
                 C_void_p(out.data_ptr()), C_void_p(query.data_ptr()), C_void_p(key.data_ptr()),
                 C_void_p(value.data_ptr()), key.stride(0), value.stride(0), self._k_table, self._v_table,
                 self._slot_p, self._lens_p, None, n, self.num_heads, self.num_kv_heads, self.head_size,
-                query.stride(0), self.scale, max_len, alibi_p, self._src_dt, out_dt, self._kv_dt, self._ws_p,
-                self._ws_n, 0, stream))
+                query.stride(0), self.scale, max_len, alibi_p, self._src_dt, out_dt, self._kv_dt, self.k_scale,
+                self.v_scale, self._ws_p, self._ws_n, 0, stream))
             return max_len
         kstride = key.stride(0)
         vstride = value.stride(0)

@@ -289,15 +289,16 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
  * vtkv_reshape_and_cache followed by vtkv_decode_attention (the result up to fp32 summation order).
  * Lengths come either from the device (seq_lens) or from the host (host_seq_lens, at most 512 sequences;
  * copied into the kernel arguments during the call, so no upload is needed and the array may be reused
- * at once); pass NULL for the other.  kv_dtype must be VTKV_BF16.  Other arguments as for
- * vtkv_decode_attention. */
+ * at once); pass NULL for the other.  kv_dtype is VTKV_BF16, or VTKV_FP8_E4M3 with k_scale / v_scale: the new
+ * rows are then stored as e4m3fn(x / scale), bit for bit as vtkv_reshape_and_cache stores them, and attended
+ * to in that form.  Other arguments as for vtkv_decode_attention. */
 int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,
                                  int64_t value_stride, const int64_t *k_ptrs, const int64_t *v_ptrs,
                                  const int64_t *slot_ids, const int32_t *seq_lens, const int32_t *host_seq_lens,
                                  int num_seqs, int num_heads, int num_kv_heads, int head_size, int64_t q_stride,
                                  float scale, int max_seq_len, const float *alibi_slopes, int q_dtype, int out_dtype,
-                                 int kv_dtype, void *workspace, int64_t workspace_bytes, int partition_tokens,
-                                 void *stream);
+                                 int kv_dtype, float k_scale, float v_scale, void *workspace, int64_t workspace_bytes,
+                                 int partition_tokens, void *stream);
 
 /* Where the partial results of the workgroups that share a (sequence, kv head) are merged: 1 = inside the
  * attention kernel, by whichever of them finishes last; 0 = by a second kernel; -1 (the default) = inside

@@ -2,7 +2,8 @@
 land in the cache bit for bit where reshape_and_cache would put them, and the attention output over
 old rows + new row is within 2e-3 abs + 2e-3 rel of the oracle (fp32 output, see test_gpu_attention.py
 for why the comparison is made before the final bf16 store), for lengths from the host (kernel
-arguments) and from the device."""
+arguments) and from the device, for a bf16 cache and for an fp8 cache (the new row is then quantised
+inside the launch, to the same codes as reshape_and_cache writes)."""
 import numpy as np
 import pytest
 
@@ -15,7 +16,7 @@ pytestmark = pytest.mark.gpu
 TOL = 2e-3
 
 
-def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partition_tokens=0, d=128):
+def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partition_tokens=0, d=128, fp8=False):
     """seq_lens count the new token."""
     import torch
 
@@ -25,12 +26,20 @@ def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partit
     b = len(seq_lens)
     num_slots = b + 2
     slots = rng.permutation(num_slots)[:b]
-    row = hkv * d * 2
-    gpu = GpuSeqs(vmm, num_slots, hkv, d, 2, max(seq_lens) + 1)
+    eb = 1 if fp8 else 2
+    row = hkv * d * eb
+    k_scale, v_scale = (0.021, 0.033) if fp8 else (1.0, 1.0)
+    code_t = np.uint8 if fp8 else np.uint16
+
+    def stored(bits, sc):  # what the cache holds for bf16 source rows
+        return O.fp8_encode(O.bf16_to_f32(bits), sc) if fp8 else bits
+
+    gpu = GpuSeqs(vmm, num_slots, hkv, d, eb, max(seq_lens) + 1)
     k_host, v_host = {}, {}
     for i, t in enumerate(seq_lens):
         s = int(slots[i])
-        k_host[s], v_host[s] = bf16_randn(rng, (t - 1, hkv, d)), bf16_randn(rng, (t - 1, hkv, d))
+        k_host[s] = stored(bf16_randn(rng, (t - 1, hkv, d)), k_scale)
+        v_host[s] = stored(bf16_randn(rng, (t - 1, hkv, d)), v_scale)
         gpu.upload(s, k_host[s], v_host[s])
     # the step's bookkeeping maps the chunk a new row needs, as in the engine
     used = vmm.extend_kv_cache_batch(None, None, [int(s) for s in slots], [row] * b, [gpu.segs[int(s)] for s in slots],
@@ -50,18 +59,22 @@ def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partit
     al_t = None if slopes is None else torch.from_numpy(slopes).cuda()
     for o in (out32, out16):  # the second call appends the same rows again: idempotent
         ops.decode_append_attention(o, q_t, nk_t, nv_t, kt, vt, hkv, scale, lens_arg, max(seq_lens), al_t, slot_t,
-                                    partition_tokens=partition_tokens)
+                                    partition_tokens=partition_tokens, kv_cache_dtype="fp8" if fp8 else "auto",
+                                    kv_scale=k_scale, v_scale=v_scale)
     torch.cuda.synchronize()
 
     # cache: old rows untouched, new row in place
-    full_k = [np.zeros((1, hkv, d), np.uint16)] * num_slots
-    full_v = [np.zeros((1, hkv, d), np.uint16)] * num_slots
+    full_k = [np.zeros((1, hkv, d), code_t)] * num_slots
+    full_v = [np.zeros((1, hkv, d), code_t)] * num_slots
     for i, t in enumerate(seq_lens):
         s = int(slots[i])
-        full_k[s] = np.concatenate([k_host[s], nk[i:i + 1]])
-        full_v[s] = np.concatenate([v_host[s], nv[i:i + 1]])
-        assert np.array_equal(gpu.download(s, t * row, which="k", dtype=np.uint16), full_k[s].reshape(-1)), f"K of seq {i}"
-        assert np.array_equal(gpu.download(s, t * row, which="v", dtype=np.uint16), full_v[s].reshape(-1)), f"V of seq {i}"
+        full_k[s] = np.concatenate([k_host[s], stored(nk[i:i + 1], k_scale)])
+        full_v[s] = np.concatenate([v_host[s], stored(nv[i:i + 1], v_scale)])
+        assert np.array_equal(gpu.download(s, t * row, which="k", dtype=code_t), full_k[s].reshape(-1)), f"K of seq {i}"
+        assert np.array_equal(gpu.download(s, t * row, which="v", dtype=code_t), full_v[s].reshape(-1)), f"V of seq {i}"
+    if fp8:  # exact dequantisation in fp32, which is what the kernel computes with
+        full_k = [O.fp8_decode(c, k_scale) for c in full_k]
+        full_v = [O.fp8_decode(c, v_scale) for c in full_v]
     cache = O.VTensorCache(full_k, full_v, slots, hkv, d)
     expect32 = O.paged_attention_v1(O.bf16_to_f32(q), cache, scale, seq_lens, slopes)
     got = out32.cpu().numpy()
@@ -82,6 +95,17 @@ EDGE = [1, 2, 3, 16, 17, 18, 33, 64, 65, 66, 256, 257, 258, 1025, 1026]
 @pytest.mark.parametrize("lens_from", ["host", "device"])
 def test_edge_lengths(gpu_pool, hq, hkv, lens_from):
     run_case(gpu_pool, 11, EDGE, hq, hkv, lens_from=lens_from)
+
+
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (64, 8), (16, 1)])
+@pytest.mark.parametrize("lens_from", ["host", "device"])
+def test_fp8_cache_edge_lengths(gpu_pool, hq, hkv, lens_from):
+    run_case(gpu_pool, 13, EDGE + [2049, 2050], hq, hkv, lens_from=lens_from, fp8=True)
+
+
+def test_fp8_cache_alibi_and_partitions(gpu_pool):
+    run_case(gpu_pool, 14, [1, 34, 401, 1000], 32, 8, alibi=True, fp8=True)
+    run_case(gpu_pool, 15, [700, 65, 1, 1500, 2049, 17], 32, 8, partition_tokens=512, fp8=True, lens_from="device")
 
 
 def test_config2_shape(gpu_pool):
@@ -106,7 +130,7 @@ def test_long_sequence_many_workgroups_per_segment(gpu_pool):
     run_case(gpu_pool, 9, [40000, 1, 2, 5000], 32, 8, lens_from="device")
 
 
-def test_rejects_fp8_cache_and_too_many_host_lengths(gpu_pool):
+def test_rejects_other_cache_types_and_too_many_host_lengths(gpu_pool):
     import ctypes as C
 
     import torch
@@ -119,8 +143,13 @@ def test_rejects_fp8_cache_and_too_many_host_lengths(gpu_pool):
     host = (C.c_int32 * 600)(*([1] * 600))
     ws = torch.empty(lib.vtkv_decode_attention_workspace_bytes(600, 8, 128, 16, 0), dtype=torch.uint8, device="cuda")
     rc = lib.vtkv_decode_append_attention(p, p, p, p, 128, 128, p, p, p, None, host, 600, 8, 1, 128, 1024, 1.0, 16, None,
-                                          _C.BF16, _C.BF16, _C.BF16, C.c_void_p(ws.data_ptr()), ws.numel(), 0, None)
+                                          _C.BF16, _C.BF16, _C.BF16, 1.0, 1.0, C.c_void_p(ws.data_ptr()), ws.numel(), 0,
+                                          None)
     assert rc == _C.EINVAL and "512" in _C.last_error()
     rc = lib.vtkv_decode_append_attention(p, p, p, p, 128, 128, p, p, p, p, None, 1, 8, 1, 128, 1024, 1.0, 16, None,
-                                          _C.BF16, _C.BF16, _C.FP8_E4M3, C.c_void_p(ws.data_ptr()), ws.numel(), 0, None)
-    assert rc == _C.EINVAL and "bf16" in _C.last_error()
+                                          _C.BF16, _C.BF16, _C.F32, 1.0, 1.0, C.c_void_p(ws.data_ptr()), ws.numel(), 0, None)
+    assert rc == _C.EINVAL and "BF16 or FP8_E4M3" in _C.last_error()
+    rc = lib.vtkv_decode_append_attention(p, p, p, p, 128, 128, p, p, p, p, None, 1, 8, 1, 128, 1024, 1.0, 16, None,
+                                          _C.BF16, _C.BF16, _C.FP8_E4M3, 0.0, 1.0, C.c_void_p(ws.data_ptr()), ws.numel(),
+                                          0, None)
+    assert rc == _C.EINVAL and "scales" in _C.last_error()

@@ -12,7 +12,7 @@ from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("kv,fused", [("bf16", True), ("bf16", False), ("fp8", False)])
+@pytest.mark.parametrize("kv,fused", [("bf16", True), ("bf16", False), ("fp8", False), ("fp8", True)])
 def test_plan_matches_ops_and_oracle(gpu_pool, kv, fused):
     import torch
 
