@@ -101,6 +101,13 @@ def lib() -> C.CDLL:
             raise VtkvLibraryMissing(
                 f"{LIB_PATH} is missing: build it with `python -m glake_amd.build` (needs hipcc). "
                 "glake_amd has no fallback implementation.")
+        # PyTorch ships its own copy of the HIP runtime.  Loaded after this library, it comes in as a second
+        # runtime beside the system's one, and a stream or allocation of the one means nothing to the other;
+        # loaded first, the dynamic loader resolves this library's dependency to the copy already there.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         handle = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)

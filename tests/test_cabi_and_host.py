@@ -113,6 +113,17 @@ def test_product_package_never_touches_the_oracle():
                 assert "oracle" not in text.replace("the oracle", ""), f"{f} mentions the oracle"
 
 
+def test_one_hip_runtime_whichever_import_comes_first():
+    """PyTorch ships its own copy of the HIP runtime; the library has to end up on the same copy, or a
+    torch stream handed to it would belong to another runtime."""
+    code = ("from glake_amd import _C; _C.lib(); import torch\n"
+            "libs = sorted({l.split()[-1] for l in open('/proc/self/maps') if 'libamdhip64' in l})\n"
+            "print(len(libs), libs)")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=ROOT)
+    assert r.returncode == 0, r.stderr
+    assert r.stdout.split()[0] == "1", r.stdout
+
+
 def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
