@@ -69,6 +69,12 @@ constexpr int kThreads = kWaves * 64;
 #define VTKV_ATTN_FP8_STAGES 1
 #endif
 constexpr int kStagesFp8 = VTKV_ATTN_FP8_STAGES;  // likewise for the fp8 variant (see the kernel)
+#ifndef VTKV_ATTN_FP8_PAIR
+#define VTKV_ATTN_FP8_PAIR 1  // fp8 rows: a workgroup streams two adjacent kv heads (see the kernel)
+#endif
+#ifndef VTKV_ATTN_FP8_WAVES
+#define VTKV_ATTN_FP8_WAVES 3  // waves per SIMD of the fp8 variants
+#endif
 constexpr int kStagesBf16 = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
 constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
 constexpr int kMinSpan = 4;        // a workgroup takes at least one tile per wave
@@ -90,6 +96,7 @@ struct AttnParams {
   // kernel (fused_merge); zero between launches: the workgroup that arrives last resets its counter
   uint32_t *seg_count;
   int fused_merge;
+  int heads_per_seg;  // kv heads that share a segment of the tile order: 1, or 2 for the PAIR variants
   void *out;           // [B,Hq,D] bf16, or fp32 when out_f32
   int out_f32;
   int64_t q_stride;
@@ -121,13 +128,22 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // bf16 in registers (K) or on the way into the LDS tile (V); the per-tensor scales are folded into the
 // logit scale (K) and into the final normalisation (V), so dequantisation costs no multiply per element.
 //
+// PAIR: an fp8 head row is 128 bytes, and a stream of isolated 128-byte pieces (one per token, the kv heads
+// of a token being 128 bytes apart) reaches about 6.1 TB/s on this part where 256-byte pieces reach 6.9 to
+// 7.1, whichever workgroup fetches the neighbouring piece.  The PAIR variants therefore make a pair of
+// adjacent kv heads the unit of the tile order: a segment is (sequence, head pair), waves 0 and 2 take the
+// even head of the pair and waves 1 and 3 the odd one, over the same rows at about the same time, so the
+// two 128-byte halves of a 256-byte piece are requested together from one CU.  Everything a wave does is
+// unchanged; only two waves instead of four share a head's tiles and its end-of-segment merge.
+//
 // APPEND: seq_lens count the step's new token, whose K/V row is not in the cache yet but in new_k /
 // new_v.  The rows before it are read from the cache as usual; the new row forms one more tile of its
 // own at the end of the sequence's tile list, loaded from new_k / new_v, and the wave that handles it
 // also stores the row into the cache.  One launch then does reshape_and_cache and attention, and each
 // byte of the new rows is read once.
-template <bool ALIBI, bool FP8, bool APPEND>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(FP8 ? 3 : VTKV_ATTN_BF16_WAVES)))
+template <bool ALIBI, bool FP8, bool APPEND, bool PAIR>
+__global__ void __launch_bounds__(kThreads)
+    __attribute__((amdgpu_waves_per_eu(FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES)))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
   // An fp8 tile is half the bytes of a bf16 tile for the same chain of dependent steps, so that variant
   // is bound by latency, not by HBM: it runs three waves per SIMD (it fits 168 registers with one
@@ -140,7 +156,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
   __shared__ int s_wave_tot[kWaves];
   // pieces of shared (sequence, kv head) segments this workgroup has written: segment, first and last
   // workgroup of the segment, and whether this workgroup delivered the last piece
-  __shared__ int s_pend[2][4];
+  __shared__ int s_pend[4][4];
   __shared__ int s_npend;
 
   const int lane = threadIdx.x & 63;
@@ -151,6 +167,11 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
   const int G = p.group;
   const int Hkv = p.num_kv_heads;
   const int B = p.num_seqs;
+  constexpr int kHps = PAIR ? 2 : 1;           // kv heads per segment
+  constexpr int kWph = kWaves / kHps;          // waves that share a head's tiles
+  const int side = PAIR ? (wave & 1) : 0;      // this wave's head inside the segment
+  const int ws = PAIR ? (wave >> 1) : wave;    // its place among the waves of that head
+  const int Hseg = Hkv / kHps;                 // segments per sequence
   auto len_of = [&](int idx) { return p.inline_lens ? il.v[idx] : p.seq_lens[idx]; };
   // tiles of one kv head of a sequence: its cached rows in 16s, plus the new row's own tile
   auto tiles_of = [](int len) {
@@ -190,7 +211,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
     __syncthreads();
   }
   const int seq_tiles_total = uniform(s_cum[B]);
-  const int total_tiles = seq_tiles_total * Hkv;
+  const int total_tiles = seq_tiles_total * Hseg;
   if (blockIdx.x == 0)
     for (int i = threadIdx.x; i <= B; i += kThreads) p.cum_tiles[i] = s_cum[i];
 
@@ -201,19 +222,19 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
   if (g_cur >= total_tiles) return;
   const int g_end = min(total_tiles, g_cur + span);
 
-  // first sequence of the span: the last b with Hkv*cum[b] <= g_cur (sequences without rows own no tile)
+  // first sequence of the span: the last b with Hseg*cum[b] <= g_cur (sequences without rows own no tile)
   int b;
   {
-    int lo = 0, hi = B;  // invariant: Hkv*cum[lo] <= g_cur < Hkv*cum[hi]
+    int lo = 0, hi = B;  // invariant: Hseg*cum[lo] <= g_cur < Hseg*cum[hi]
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
-      if (uniform(s_cum[mid]) * Hkv <= g_cur) lo = mid; else hi = mid;
+      if (uniform(s_cum[mid]) * Hseg <= g_cur) lo = mid; else hi = mid;
     }
     b = lo;
   }
   int nt_b = uniform(s_cum[b + 1]) - uniform(s_cum[b]);
-  int kvh = (g_cur - uniform(s_cum[b]) * Hkv) / nt_b;
-  int tile0 = g_cur - uniform(s_cum[b]) * Hkv - kvh * nt_b;
+  int kvg = (g_cur - uniform(s_cum[b]) * Hseg) / nt_b;  // segment of the sequence: kv head, or pair of kv heads
+  int tile0 = g_cur - uniform(s_cum[b]) * Hseg - kvg * nt_b;
 
   typedef const __attribute__((address_space(1))) char *gptr;
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
@@ -223,8 +244,9 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
   char *v_tile = smem + wave * (kTile * kRowBytes);
   char *k_tile = smem + kWaves * kTile * kRowBytes + 1024 + wave * (kTile * kRowBytes);
 
-  // ---- one segment = the part of the span that lies in one (sequence, kv head)
+  // ---- one segment = the part of the span that lies in one (sequence, kv head or pair of kv heads)
   while (g_cur < g_end) {
+    const int kvh = kvg * kHps + side;  // this wave's kv head
     const int seg_tiles = min(g_end - g_cur, nt_b - tile0);
     const int seq_len = uniform(len_of(b));
     const int ctx_len = APPEND ? seq_len - 1 : seq_len;                // rows read from the cache
@@ -267,11 +289,11 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
     float m_run = -INFINITY;  // running max of scaled logits (log2 units) of head n
     float l_run = 0.f;        // this lane's share of the running sum
 
-    // The segment's tiles are dealt round-robin to the four waves: this wave owns tiles wave, wave+4, ...
+    // The segment's tiles are dealt round-robin to the waves of a head: this wave owns tiles ws, ws+kWph, ...
     // Only the last tile of a sequence can be ragged; its missing rows are redirected to the last valid
     // row (their logits are masked) so no lane reads past the mapped part of a range.
     const int n_tiles = seg_tiles - (has_new ? 1 : 0);  // tiles of cached rows; the new row's tile comes last
-    const int my_tiles = (seg_tiles - wave + kWaves - 1) / kWaves;
+    const int my_tiles = (seg_tiles - ws + kWph - 1) / kWph;
     // rows in the last tile of cached rows, 1..16
     const int valid_last = n_tiles > 0 ? seg_end - (seg_start + (n_tiles - 1) * kTile) : kTile;
     // per-lane byte offsets inside a K or V tile: load j of a lane takes row 4j+g, piece n, i.e. four
@@ -297,7 +319,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
     // bytes instead (one cache line per load, not consumed).
     auto load_tile = [&](gptr base, gptr new_base, int i, u32x4 *regs) {
       const bool live = i < my_tiles;
-      const int tile = wave + kWaves * i;
+      const int tile = ws + kWph * i;
       const bool last = tile == n_tiles - 1;
       const bool is_new = APPEND && has_new && live && tile == seg_tiles - 1;
       // (masks, not selects: selects here end up as branches around separate copies of the loads)
@@ -318,7 +340,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
 
     // one 16-row tile: logits, online softmax update, P.V
     auto consume = [&](int i, u32x4 *kreg, u32x4 *vreg) {
-      const int tile = wave + kWaves * i;
+      const int tile = ws + kWph * i;
       const bool is_new = APPEND && has_new && tile == seg_tiles - 1;
       const int t0 = is_new ? seq_len - 1 : seg_start + tile * kTile;                  // position of the tile's row 0
       const int valid = is_new ? 1 : (tile == n_tiles - 1 ? valid_last : kTile);       // rows that count
@@ -504,7 +526,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
       }
     }
 
-    // ---- merge the four waves.  l_run is still split over the four row groups of a lane column.
+    // ---- merge the waves of each head.  l_run is still split over the four row groups of a lane column.
     l_run = sum_over_row_groups(l_run);
     __syncthreads();  // every wave is done with its V tile: smem is free for the merge
     float *sm_m = reinterpret_cast<float *>(smem + kWaves * kTile * kRowBytes);  // [4][16]
@@ -515,17 +537,24 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
       sm_l[wave * 16 + n] = l_run;
     }
     __syncthreads();
-    const float m_wg = fmaxf(fmaxf(sm_m[n], sm_m[16 + n]), fmaxf(sm_m[32 + n], sm_m[48 + n]));
-    const float f = __builtin_amdgcn_exp2f(m_run - m_wg);  // 0 for a wave that saw no row
-    // slot of this (workgroup, segment): both indices only grow along the tile order, so the sum is unique
-    const int64_t slot_idx = (int64_t)wg + (int64_t)b * Hkv + kvh;
-    // workgroups w0..w1 hold the pieces of this (sequence, kv head): its tiles are [first, first + nt_b)
-    // of the global order
-    const int first_tile = uniform(s_cum[b]) * Hkv + kvh * nt_b;
+    // the waves of head `sd` of the segment are sd, sd + kHps, ...
+    auto head_max = [&](int sd, int head) {
+      float m = sm_m[sd * 16 + head];
+#pragma unroll
+      for (int j = 1; j < kWph; ++j) m = fmaxf(m, sm_m[(sd + kHps * j) * 16 + head]);
+      return m;
+    };
+    const float f = __builtin_amdgcn_exp2f(m_run - head_max(side, n));  // 0 for a wave that saw no row
+    // Slot of this (workgroup, segment, head): kHps * workgroup + (sequence * Hkv + kv head).  Along the tile
+    // order neither the workgroup nor the segment ever decreases, and a later workgroup's kv head is at most
+    // kHps - 1 lower than an earlier one's (inside a shared pair), so the sum is unique.
+    // Workgroups w0..w1 hold the pieces of this segment: its tiles are [first, first + nt_b) of the
+    // global order.
+    const int first_tile = uniform(s_cum[b]) * Hseg + kvg * nt_b;
     const int w0 = first_tile / span, w1 = (first_tile + nt_b - 1) / span;
     const bool whole = p.fused_merge && w0 == w1;  // no other workgroup: the result is final
-    auto store_out = [&](int head, int d, float r) {
-      const int64_t oi = ((int64_t)b * p.num_heads + kvh * G + head) * kD + d;
+    auto store_out = [&](int kv_head, int head, int d, float r) {
+      const int64_t oi = ((int64_t)b * p.num_heads + kv_head * G + head) * kD + d;
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
@@ -543,22 +572,26 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
       }
       __syncthreads();
       const int nh = min(G, h0 + 8) - h0;
-      for (int idx = threadIdx.x; idx < nh * kD; idx += kThreads) {
-        const int hh = idx / kD, d = idx % kD;
+      for (int idx = threadIdx.x; idx < kHps * nh * kD; idx += kThreads) {
+        const int sd = PAIR ? idx / (nh * kD) : 0;
+        const int rem = idx - sd * (nh * kD);
+        const int hh = rem / kD, d = rem % kD;
         const int head = h0 + hh;
-        const float mw = fmaxf(fmaxf(sm_m[head], sm_m[16 + head]), fmaxf(sm_m[32 + head], sm_m[48 + head]));
+        const int kv_head = kvg * kHps + sd;
+        const float mw = head_max(sd, head);
         float lsum = 0.f, o = 0.f;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
+        for (int j = 0; j < kWph; ++j) {
+          const int w = sd + kHps * j;
           lsum += sm_l[w * 16 + head] * __builtin_amdgcn_exp2f(sm_m[w * 16 + head] - mw);
           o += sm_o[(w * 8 + hh) * kD + d];
         }
         const float o_norm = o / lsum;
         if (whole) {
-          store_out(head, d, o_norm * p.v_scale);
+          store_out(kv_head, head, d, o_norm * p.v_scale);
           continue;
         }
-        const int64_t pidx = slot_idx * G + head;
+        const int64_t pidx = ((int64_t)kHps * wg + (int64_t)b * Hkv + kv_head) * G + head;
         if (p.fused_merge) {
           store_device_coherent(&p.part_out[pidx * kD + d], o_norm);
           if (d == 0) {
@@ -575,14 +608,16 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
       }
     }
     if (p.fused_merge && !whole && threadIdx.x == 0) {
-      // A piece of a (sequence, kv head) that other workgroups share.  Its arrival is counted at the end
-      // of this workgroup's span, not here, so that the streaming goes on without waiting for the
+      // Pieces of (sequence, kv head) segments that other workgroups share.  Their arrival is counted at the
+      // end of this workgroup's span, not here, so that the streaming goes on without waiting for the
       // stores.  Only the first and the last segment of a span can be such pieces.
-      const int k = s_npend;
-      s_pend[k][0] = b * Hkv + kvh;
-      s_pend[k][1] = w0;
-      s_pend[k][2] = w1;
-      s_npend = k + 1;
+      int k = s_npend;
+      for (int sd = 0; sd < kHps; ++sd, ++k) {
+        s_pend[k][0] = b * Hkv + kvg * kHps + sd;
+        s_pend[k][1] = w0;
+        s_pend[k][2] = w1;
+      }
+      s_npend = k;
     }
 
     // ---- next segment of the span
@@ -591,8 +626,8 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
     if (g_cur < g_end) {
       if (tile0 == nt_b) {
         tile0 = 0;
-        if (++kvh == Hkv) {
-          kvh = 0;
+        if (++kvg == Hseg) {
+          kvg = 0;
           do {
             ++b;
             nt_b = uniform(s_cum[b + 1]) - uniform(s_cum[b]);
@@ -635,7 +670,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(F
         float pm[4], ps[4], po[4];
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-          const int64_t pidx = (min(wb + jj, w1) + seg) * G + head;
+          const int64_t pidx = ((int64_t)kHps * min(wb + jj, w1) + seg) * G + head;
           pm[jj] = load_device_coherent(&p.part_max[pidx]);
           ps[jj] = load_device_coherent(&p.part_sum[pidx]);
           po[jj] = load_device_coherent(&p.part_out[pidx * kD + d]);
@@ -679,9 +714,10 @@ __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
   const int cum_b = p.cum_tiles[b];
   const int nt = p.cum_tiles[b + 1] - cum_b;
   if (nt <= 0) return;
-  const int total_tiles = p.cum_tiles[p.num_seqs] * Hkv;
+  const int hps = p.heads_per_seg, Hseg = Hkv / hps;
+  const int total_tiles = p.cum_tiles[p.num_seqs] * Hseg;
   const int span = span_of(p, total_tiles);
-  const int first = cum_b * Hkv + kvh * nt;
+  const int first = cum_b * Hseg + (kvh / hps) * nt;
   const int w0 = first / span, w1 = (first + nt - 1) / span;
   const int64_t seg = (int64_t)b * Hkv + kvh;
   for (int h0 = 0; h0 < G; h0 += 4) {
@@ -695,7 +731,7 @@ __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
 #pragma unroll
         for (int hh = 0; hh < 4; ++hh) {
           // (pieces and heads past the end repeat the last one; their weights are set to zero below)
-          const int64_t pidx = (min(wb + jj, w1) + seg) * G + min(h0 + hh, G - 1);
+          const int64_t pidx = ((int64_t)hps * min(wb + jj, w1) + seg) * G + min(h0 + hh, G - 1);
           pm[jj][hh] = p.part_max[pidx];
           ps[jj][hh] = p.part_sum[pidx];
           po[jj][hh] = p.part_out[pidx * kD + d];
@@ -743,7 +779,7 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 8;  // instantiations of the streaming kernel
+constexpr int kVariants = 12;  // instantiations of the streaming kernel
 struct Residency {
   std::mutex mu;
   int device = -1;
@@ -830,23 +866,25 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
 
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   const bool alibi = alibi_slopes != nullptr;
-  // kernel variant: bit 0 fp8, bit 1 alibi, bit 2 fused append
-  const int variant = (append ? 4 : 0) + (alibi ? 2 : 0) + (fp8 ? 1 : 0);
-  void (*kernel)(AttnParams, InlineLens) = nullptr;
-  switch (variant) {
-    case 0: kernel = decode_attn_stream_kernel<false, false, false>; break;
-    case 1: kernel = decode_attn_stream_kernel<false, true, false>; break;
-    case 2: kernel = decode_attn_stream_kernel<true, false, false>; break;
-    case 3: kernel = decode_attn_stream_kernel<true, true, false>; break;
-    case 4: kernel = decode_attn_stream_kernel<false, false, true>; break;
-    case 5: kernel = decode_attn_stream_kernel<false, true, true>; break;
-    case 6: kernel = decode_attn_stream_kernel<true, false, true>; break;
-    default: kernel = decode_attn_stream_kernel<true, true, true>; break;
-  }
+  // Two adjacent kv heads per segment for fp8 rows (see the kernel).  Slots: 2 * grid + num_seqs * num_kv_heads
+  // of `group` heads each, which the workspace (16 heads per workgroup) holds for groups up to 8.
+  const bool pair = VTKV_ATTN_FP8_PAIR && fp8 && num_kv_heads % 2 == 0 && group <= 8;
+  const int seg_heads = pair ? 2 : 1;
+  // kernel variant: bit 0 alibi, bit 1 fused append; 0..3 bf16, 4..7 fp8, 8..11 fp8 with paired kv heads
+  const int variant = (fp8 ? (pair ? 8 : 4) : 0) + (append ? 2 : 0) + (alibi ? 1 : 0);
+  static void (*const kKernels[kVariants])(AttnParams, InlineLens) = {
+      decode_attn_stream_kernel<false, false, false, false>, decode_attn_stream_kernel<true, false, false, false>,
+      decode_attn_stream_kernel<false, false, true, false>,  decode_attn_stream_kernel<true, false, true, false>,
+      decode_attn_stream_kernel<false, true, false, false>,  decode_attn_stream_kernel<true, true, false, false>,
+      decode_attn_stream_kernel<false, true, true, false>,   decode_attn_stream_kernel<true, true, true, false>,
+      decode_attn_stream_kernel<false, true, false, true>,   decode_attn_stream_kernel<true, true, false, true>,
+      decode_attn_stream_kernel<false, true, true, true>,    decode_attn_stream_kernel<true, true, true, true>,
+  };
+  void (*kernel)(AttnParams, InlineLens) = kKernels[variant];
   int64_t grid;
   if (partition_tokens > 0) {
     // (the fused append adds one tile per sequence and kv head)
-    grid = fixed_span_grid(num_seqs, num_kv_heads, max_seq_len + (append ? kTile : 0), partition_tokens);
+    grid = fixed_span_grid(num_seqs, num_kv_heads / seg_heads, max_seq_len + (append ? kTile : 0), partition_tokens);
     VTKV_REQUIRE(grid <= (1ll << 24), "partition_tokens %d gives %lld workgroups", partition_tokens, (long long)grid);
   } else {
     const int g = resident_grid(kernel, variant);
@@ -877,7 +915,9 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   // most (sequence, kv head) segments lie inside one workgroup and need no merge at all (measured: +4.5 %
   // per step at 2048 segments on 512 workgroups, +1.5 % at 1024, -1.6 % at 512), so it is the default
   // from two segments per workgroup on.
-  p.fused_merge = g_fused_merge == 1 || (g_fused_merge < 0 && (int64_t)num_seqs * num_kv_heads >= 2 * grid);
+  p.fused_merge =
+      g_fused_merge == 1 || (g_fused_merge < 0 && (int64_t)num_seqs * (num_kv_heads / seg_heads) >= 2 * grid);
+  p.heads_per_seg = seg_heads;
   p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
   p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);
   p.part_max = p.part_out + n_stat * kD;

@@ -16,7 +16,7 @@ from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from
 pytestmark = pytest.mark.gpu
 
 
-def run_case(vmm, seed, seq_lens, hq, hkv, d=128, alibi=False, spread=1.0):
+def run_case(vmm, seed, seq_lens, hq, hkv, d=128, alibi=False, spread=1.0, partition_tokens=0):
     import torch
 
     from glake_amd import _custom_ops as ops
@@ -54,8 +54,8 @@ def run_case(vmm, seed, seq_lens, hq, hkv, d=128, alibi=False, spread=1.0):
     args = (torch_bf16_from_bits(q), kt, vt, hkv, scale, torch.tensor(seq_lens, dtype=torch.int32, device="cuda"), 1,
             max(seq_lens), None if slopes is None else torch.from_numpy(slopes).cuda(), "fp8", k_scale,
             torch.tensor(slots, dtype=torch.int64, device="cuda"))
-    ops.paged_attention_v1(out32, *args, v_scale=v_scale)
-    ops.paged_attention_v1(out16, *args, v_scale=v_scale)
+    ops.paged_attention_v1(out32, *args, v_scale=v_scale, partition_tokens=partition_tokens)
+    ops.paged_attention_v1(out16, *args, v_scale=v_scale, partition_tokens=partition_tokens)
     torch.cuda.synchronize()
     gpu.close()
     got = out32.cpu().numpy()

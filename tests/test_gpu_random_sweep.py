@@ -8,11 +8,15 @@ import numpy as np
 import pytest
 
 import test_gpu_attention as A
+import test_gpu_attention_fp8 as F
 import test_gpu_prefill_attention as P
 
 pytestmark = pytest.mark.gpu
 
 HEADS = [(32, 8), (64, 8), (8, 8), (16, 1), (12, 4), (8, 2), (16, 16), (48, 8), (128, 8), (7, 7), (10, 2)]
+# fp8 rows: an even number of kv heads with groups up to 8 takes the kernel variants that stream two kv
+# heads per workgroup, everything else (odd counts, one kv head, groups above 8) the one-head variants
+HEADS_FP8 = HEADS + [(6, 3), (40, 8), (32, 2), (18, 2), (2, 2), (24, 6), (64, 4)]
 
 
 @pytest.mark.parametrize("seed", [101, 202, 303])
@@ -49,5 +53,37 @@ def test_random_sweep(gpu_pool, seed):
                 fp8, al = bool(rng.integers(4) == 0), bool(rng.integers(4) == 0)
                 print(f"prompt case {case}: seed {sub} heads {hq}/{hkv} queries {ql} rows {seq} fp8 {fp8} alibi {al}", flush=True)
                 P.run_case(gpu_pool, sub, ql, seq, hq, hkv, alibi=al, fp8=fp8, tol=3e-2 if fp8 else 2e-3)
+    finally:
+        _C.check(lib.vtkv_set_fused_merge(-1))
+
+
+@pytest.mark.parametrize("seed", [404, 505])
+def test_random_sweep_fp8_decode(gpu_pool, seed):
+    from glake_amd import _C
+
+    lib = _C.lib()
+    rng = np.random.default_rng(seed)
+    try:
+        for case in range(40):
+            hq, hkv = HEADS_FP8[rng.integers(len(HEADS_FP8))]
+            b = int(rng.integers(1, 24))
+            kind = rng.integers(4)
+            if kind == 0:
+                lens = rng.integers(1, 40, b)
+            elif kind == 1:
+                lens = rng.integers(1, 700, b)
+            elif kind == 2:
+                lens = rng.integers(1, 3000, max(1, b // 3))
+            else:
+                lens = np.concatenate([rng.integers(1, 20, b), rng.integers(2000, 6000, 1)])
+            lens = [int(x) for x in lens]
+            pt = int(rng.choice([0, 0, 0, 64, 128, 256, 512, 1024]))
+            alibi = bool(rng.integers(4) == 0)
+            merge = int(rng.integers(-1, 2))
+            sub = int(rng.integers(1 << 30))
+            _C.check(lib.vtkv_set_fused_merge(merge))
+            print(f"fp8 decode case {case}: seed {sub} heads {hq}/{hkv} lens {lens} partition {pt} alibi {alibi} "
+                  f"merge {merge}", flush=True)
+            F.run_case(gpu_pool, sub, lens, hq, hkv, alibi=alibi, partition_tokens=pt)
     finally:
         _C.check(lib.vtkv_set_fused_merge(-1))
