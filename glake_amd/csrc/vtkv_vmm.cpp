@@ -67,9 +67,13 @@ struct Pool {
   int64_t retired = 0;  // chunks still mapped at the top of shrunken segments; they count as free
   // chunks that are mapped into more than one segment (shared prefixes): handle -> number of mappings
   std::unordered_map<hipMemGenericAllocationHandle_t, int> shared;
-  // map/unmap cycles a chunk has been through since it was created (see kCyclesPerChunk)
+  // mappings a chunk has been through since it was created, and their sum over all chunks of the pool
+  // (see kRuntimeEntries)
   std::unordered_map<hipMemGenericAllocationHandle_t, int> cycles;
+  int64_t pairs = 0;
   int64_t recreated = 0;
+  // what the pool has asked of the runtime so far (reported when a mapping fails)
+  int64_t maps = 0, ranges_reserved = 0, bytes_reserved = 0;
   // map-ahead worker (started on the first request, joined by vtkv_pool_destroy or at exit)
   struct Request { vtkv_segment *seg; int chunks; };
   std::deque<Request> requests;
@@ -105,6 +109,10 @@ hipError_t take_range_locked(int64_t bytes, char **out) {
   void *p = nullptr;
   const hipError_t e = hipMemAddressReserve(&p, bytes, kChunk, nullptr, 0);
   *out = (char *)p;
+  if (e == hipSuccess) {
+    ++g_pool.ranges_reserved;
+    g_pool.bytes_reserved += bytes;
+  }
   return e;
 }
 void give_range_locked(char *p, int64_t bytes) { g_pool.spare_ranges[bytes].push_back(p); }
@@ -131,6 +139,8 @@ using vtkv::kChunk;
 
 namespace {
 
+void note_mapping_locked(hipMemGenericAllocationHandle_t h);  // below, with the rule it serves
+
 // Map `n` chunks at offset `held` (== `mapped`: the caller has taken back all retired chunks) of
 // every range.  Caller holds the pool mutex and has checked the free list holds 2*layers*n chunks.
 // On a HIP failure everything mapped by this call is rolled back.
@@ -155,11 +165,15 @@ int map_chunks_locked(vtkv_segment *s, int n) {
           break;
         }
         g_pool.free_chunks.pop_back();
+        note_mapping_locked(h);
         auto *list = which ? &s->v_chunks[l] : &s->k_chunks[l];
         list->push_back(h);
         done.push_back({va, h, list});
         // (one call over several chunks costs the same per chunk: measured 28 us each either way)
         err = hipMemSetAccess(va, kChunk, &ad, 1);
+        if (err != hipSuccess)
+          snprintf(where, sizeof(where), " (hipMemSetAccess, %s range of layer %d, offset %lld of %lld)", which ? "V" : "K",
+                   l, (long long)(s->held + (int64_t)j * kChunk), (long long)s->context_max);
       }
     }
   }
@@ -169,20 +183,41 @@ int map_chunks_locked(vtkv_segment *s, int n) {
       it->list->pop_back();
       g_pool.free_chunks.push_back(it->h);
     }
-    return vtkv::fail(VTKV_EHIP, "mapping a chunk failed: %s%s", hipGetErrorString(err), where);
+    return vtkv::fail(VTKV_EHIP, "mapping a chunk failed: %s%s; the pool has mapped %lld chunks (%lld mappings of its live chunks), "
+                      "re-created %lld and reserved %lld ranges (%lld MiB) so far", hipGetErrorString(err), where,
+                      (long long)g_pool.maps, (long long)g_pool.pairs, (long long)g_pool.recreated, (long long)g_pool.ranges_reserved,
+                      (long long)(g_pool.bytes_reserved >> 20));
   }
   s->held += (int64_t)n * kChunk;
   s->mapped = s->held;
   return VTKV_OK;
 }
 
-// A physical chunk is created anew after this many map/unmap cycles.  The runtime keeps something per
-// (chunk, address) pair a chunk has ever been mapped at and gives it up only with the chunk: a pure HIP
-// program that maps 96 chunks at the top of 250 ranges in turn gets "invalid argument" from
-// hipMemSetAccess and "out of memory" from hipMemCreate after 330 000 mappings with 300 GB free, and
-// runs on without limit when it re-creates its chunks now and then.  A server maps a chunk at a new
-// address at every 2 MiB boundary a sequence crosses, so it would get there within hours.
+// This runtime keeps one entry per physical chunk and one per (chunk, virtual address) pair a chunk has
+// ever been mapped at; it gives a pair's entry up only together with the chunk (hipMemRelease), and a
+// process has 65 536 of them.  A pure HIP program with 700 chunks that maps one chunk at one of 1 200
+// ranges per step, (chunk, range) pairs mostly new, gets "invalid argument" from hipMemSetAccess at step
+// 64 810, and at step 63 510 with 2 000 chunks; with every chunk confined to two ranges it runs on without
+// limit, and so it does when it re-creates a chunk every 16 or 64 mappings.  A server maps a chunk at a
+// new address at every 2 MiB boundary a sequence crosses, so it would get there within hours.
+//
+// The pool therefore counts the mappings of every chunk since its creation (an upper bound of its pairs)
+// and their sum, and re-creates a chunk when it comes back to the free list if the chunk has been through
+// kCyclesPerChunk mappings or the sum is above the pool's share of the entries: above it every cycle of a
+// chunk gives back at least the entry it took, so the sum stays below the share plus one entry per
+// mapped chunk.  vtkv_pool_init keeps chunks + one pair per chunk below the limit.
 constexpr int kCyclesPerChunk = 256;
+constexpr int64_t kRuntimeEntries = 64000;   // of the 65 536: some are in use before the pool starts
+constexpr int64_t kMaxPoolChunks = 30000;    // 2 entries per mapped chunk, and room to remap
+
+int64_t pair_share_locked() { return std::max<int64_t>(kRuntimeEntries - 2 * g_pool.total - 1000, 2000); }
+
+// `h` has just been mapped at an address.
+void note_mapping_locked(hipMemGenericAllocationHandle_t h) {
+  ++g_pool.cycles[h];
+  ++g_pool.pairs;
+  ++g_pool.maps;
+}
 
 // One mapping of `h` is gone: the chunk is free again unless another segment still maps it.
 void release_handle_locked(hipMemGenericAllocationHandle_t h) {
@@ -191,7 +226,9 @@ void release_handle_locked(hipMemGenericAllocationHandle_t h) {
     if (--it->second == 1) g_pool.shared.erase(it);
     return;
   }
-  if (++g_pool.cycles[h] >= kCyclesPerChunk) {
+  auto cyc = g_pool.cycles.find(h);
+  const int n = cyc == g_pool.cycles.end() ? 0 : cyc->second;
+  if (n > 0 && (n >= kCyclesPerChunk || g_pool.pairs > pair_share_locked())) {
     hipMemAllocationProp prop = {};
     prop.type = hipMemAllocationTypePinned;
     prop.location.type = hipMemLocationTypeDevice;
@@ -199,7 +236,8 @@ void release_handle_locked(hipMemGenericAllocationHandle_t h) {
     hipMemGenericAllocationHandle_t fresh;
     // (if the new chunk cannot be had now, the old one serves on and is tried again after its next cycle)
     if (hipMemCreate(&fresh, kChunk, &prop, 0) == hipSuccess) {
-      g_pool.cycles.erase(h);
+      g_pool.cycles.erase(cyc);
+      g_pool.pairs -= n;
       (void)hipMemRelease(h);
       h = fresh;
       ++g_pool.recreated;
@@ -352,6 +390,7 @@ void worker_main() {
       if (err != hipSuccess)
         for (size_t i = 0; i < done; ++i) (void)hipMemUnmap(va_of(i), kChunk);
       lk.lock();
+      for (size_t i = 0; i < std::min(done + 1, handles.size()); ++i) note_mapping_locked(handles[i]);
       if (err == hipSuccess) {
         for (int l = 0; l < layers; ++l)
           for (int which = 0; which < 2; ++which)
@@ -420,6 +459,11 @@ int vtkv_pool_init(int device, int64_t num_chunks) {
   VTKV_HIP(hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityMinimum));
   if (gran == 0 || kChunk % (int64_t)gran != 0)
     return vtkv::fail(VTKV_EHIP, "allocation granularity %zu does not divide the 2 MiB chunk", gran);
+  if (g_pool.total + num_chunks > kMaxPoolChunks)
+    return vtkv::fail(VTKV_EINVAL,
+                      "a pool of %lld chunks is more than this HIP runtime can serve: a process has 65536 entries for "
+                      "chunks and (chunk, address) mappings together; at most %lld chunks of 2 MiB",
+                      (long long)(g_pool.total + num_chunks), (long long)kMaxPoolChunks);
   g_pool.device = device;
   g_pool.free_chunks.reserve(g_pool.free_chunks.size() + num_chunks);
   for (int64_t i = 0; i < num_chunks; ++i) {
@@ -485,6 +529,7 @@ int vtkv_pool_destroy(void) {
   for (auto h : g_pool.free_chunks) VTKV_HIP(hipMemRelease(h));
   g_pool.free_chunks.clear();
   g_pool.cycles.clear();
+  g_pool.pairs = 0;
   g_pool.total = 0;
   g_pool.device = -1;
   return VTKV_OK;
@@ -686,6 +731,7 @@ int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, v
         char *va = base + j * kChunk;
         err = hipMemMap(va, kChunk, 0, from[j], 0);
         if (err != hipSuccess) break;
+        note_mapping_locked(from[j]);
         to.push_back(from[j]);
         done.push_back({va, &to, from[j]});
         err = hipMemSetAccess(va, kChunk, &ad, 1);

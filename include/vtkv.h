@@ -53,7 +53,8 @@ int64_t vtkv_chunk_bytes(void);
 
 /* Create `num_chunks` physical chunks on `device` and keep them in the free pool.
  * Replaces init_physical_handle(num_blocks, device_id) (vmm_allocator.cpp:113-151).
- * May be called again to add chunks. */
+ * May be called again to add chunks.  At most 30000 chunks in all (VTKV_EINVAL beyond): the HIP runtime
+ * has 65536 entries per process for physical chunks and their mappings together. */
 int vtkv_pool_init(int device, int64_t num_chunks);
 /* Chunks no sequence owns; replaces showFreeBlocks() (vmm_allocator.cpp:472-474). <0 on error.
  * Unmapping is lazy: a segment that shrinks (preempt, release, swap-out) keeps its chunks mapped at the
@@ -62,9 +63,10 @@ int vtkv_pool_init(int device, int64_t num_chunks);
 int64_t vtkv_pool_free_chunks(void);
 /* How many of the free chunks are retired, i.e. still mapped.  No counterpart in the reference. */
 int64_t vtkv_pool_retired_chunks(void);
-/* Physical chunks the pool has released and created anew so far: a chunk is replaced after 256 map/unmap
- * cycles, because the HIP runtime keeps per-chunk state for every address a chunk was ever mapped at and
- * runs out of it otherwise.  No counterpart in the reference. */
+/* Physical chunks the pool has released and created anew so far: a chunk is replaced after 256 mappings,
+ * or earlier once the live chunks of the pool have been through more mappings than its share of the
+ * runtime's entries, because the HIP runtime keeps an entry for every address a chunk was ever mapped at
+ * until the chunk is released, and runs out of them otherwise.  No counterpart in the reference. */
 int64_t vtkv_pool_recreated_chunks(void);
 /* Unmap retired chunks now, until at least `max_chunks` are unmapped or none is left (< 0: all; whole
  * rows, i.e. one chunk of every range of a segment, at a time), so that later growth finds them on the

@@ -373,3 +373,40 @@ def test_chunks_are_replaced_after_many_map_unmap_cycles(gpu_pool):
     assert vmm.recreatedBlocks() - made0 >= 4     # two chunks per cycle, each replaced at 256 and 512 cycles
     seg.destroy()
     assert vmm.showFreeBlocks() == free0 and vmm.totalBlocks() == total0
+
+
+def test_mappings_at_ever_new_addresses_stay_within_what_the_runtime_can_hold(gpu_pool):
+    """48 slots grow by changing numbers of chunks and give them back, round after round, so that the
+    chunks on top of the free list keep meeting addresses they have not been mapped at before: 75 000
+    mappings, no chunk through more than some 150.  The HIP runtime holds 65 536 entries per process, one
+    per chunk and one per (chunk, address) pair of a live chunk, and fails with "invalid argument" beyond;
+    the pool counts the mappings of its live chunks and re-creates chunks on their way back to the free
+    list once the count is above its share.  The books stay balanced and the memory works."""
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    free0, total0, made0 = vmm.showFreeBlocks(), vmm.totalBlocks(), vmm.recreatedBlocks()
+    nseg, per = 48, 10
+    segs = [vmm.KVcacheSegment(1, per * CHUNK, 0, False) for _ in range(nseg)]
+    payload = np.arange(4096, dtype=np.uint8)
+    back = np.empty_like(payload)
+    maps = rounds = 0
+    while maps < 75000:
+        for i, seg in enumerate(segs):
+            n = 1 + (i * 7 + rounds * 3) % per
+            seg.expandMultiSegment(n)
+            maps += 2 * n
+        if rounds % 20 == 0:
+            for seg in segs[::7]:
+                dst = seg.getValueDevicePtr(0) + seg.actual_size - 4096
+                _C.check(_C.lib().vtkv_memcpy_h2d(dst, payload.ctypes.data_as(C.c_void_p), 4096))
+                _C.check(_C.lib().vtkv_memcpy_d2h(back.ctypes.data_as(C.c_void_p), dst, 4096))
+                assert np.array_equal(back, payload)
+        for seg in segs:
+            seg.preempt_seq(0)
+        vmm.trim()
+        rounds += 1
+    assert vmm.recreatedBlocks() > made0
+    for seg in segs:
+        seg.destroy()
+    assert vmm.showFreeBlocks() == free0 and vmm.totalBlocks() == total0
