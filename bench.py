@@ -31,7 +31,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # calibration copy of known size that this script runs before timing).  Counters cannot be read from
 # inside this process, so the measured ratio is kept here with the summary it comes from.
 MEASURED_TRAFFIC = {
-    "c2": (1.004, "profiles/decode_attn_stream_kernel_c2_llama3_8b_decode.md"),
+    "c2": (1.003, "profiles/decode_attn_stream_kernel_c2_llama3_8b_decode.md"),
 }
 
 CONFIGS = {
