@@ -39,6 +39,7 @@ SIGNATURES = {
     "vtkv_last_error": (C.c_char_p, []),
     "vtkv_version": (_i, []),
     "vtkv_chunk_bytes": (_i64, []),
+    "vtkv_pool_set_chunk_bytes": (_i, [_i64]),
     "vtkv_pool_init": (_i, [_i, _i64]),
     "vtkv_pool_free_chunks": (_i64, []),
     "vtkv_pool_total_chunks": (_i64, []),

@@ -18,7 +18,7 @@ from __future__ import annotations
 import enum
 from typing import Dict, List, Optional
 
-PHY_GRAN = 2 * 1024 * 1024  # bytes of one chunk (sequence.py:345)
+PHY_GRAN = 2 * 1024 * 1024  # bytes of one chunk (sequence.py:345); pools with larger chunks pass their size
 PREFILL_SLACK_TOKENS = 100  # a prompt reserves room for 100 more tokens (sequence.py:343)
 
 
@@ -33,12 +33,15 @@ class SequenceChunks:
     """Bytes and chunks one sequence needs in each of its ranges (sequence.py:342-360).
 
     ``token_size`` is the bytes of one token row of one range (num_kv_heads * head_size * element
-    bytes).  ``logical_block_num`` counts K and V chunks together, i.e. two per 2 MiB of rows."""
+    bytes).  ``logical_block_num`` counts K and V chunks together, i.e. two per chunk of rows."""
 
-    def __init__(self, token_size: int):
+    def __init__(self, token_size: int, chunk_bytes: int = PHY_GRAN):
         if token_size <= 0:
             raise ValueError("token_size must be positive")
+        if chunk_bytes <= 0 or chunk_bytes % PHY_GRAN:
+            raise ValueError("chunk_bytes must be a positive multiple of 2 MiB")
         self.token_size = int(token_size)
+        self.chunk_bytes = int(chunk_bytes)
         self.reserve_size = 0       # bytes the sequence has claimed per range, a multiple of the chunk
         self.free_size = 0          # claimed bytes not yet written
         self.logical_block_num = 0  # chunks claimed (K + V)
@@ -48,20 +51,21 @@ class SequenceChunks:
     def append_tokens(self, num_tokens: int) -> None:
         """One call per scheduling step: the prompt (any number of tokens, plus slack) or one new token."""
         plus = 0 if num_tokens == 1 else PREFILL_SLACK_TOKENS
+        gran = self.chunk_bytes
         need = self.token_size * (num_tokens + plus)
         if self.reserve_size == 0:
-            rounded = PHY_GRAN * ((need + PHY_GRAN - 1) // PHY_GRAN)
+            rounded = gran * ((need + gran - 1) // gran)
             self.reserve_size = rounded
             self.free_size = rounded - need
-            self.logical_block_num = 2 * (rounded // PHY_GRAN)
+            self.logical_block_num = 2 * (rounded // gran)
         elif self.free_size >= need:
             self.free_size -= need
         else:
             gap = need - self.free_size
-            rounded = PHY_GRAN * ((gap + PHY_GRAN - 1) // PHY_GRAN)
+            rounded = gran * ((gap + gran - 1) // gran)
             self.reserve_size += rounded
             self.free_size = rounded - gap
-            self.logical_block_num += 2 * (rounded // PHY_GRAN)
+            self.logical_block_num += 2 * (rounded // gran)
 
     # the reference's accessor names (sequence.py:331-340)
     def get_slot(self) -> int:

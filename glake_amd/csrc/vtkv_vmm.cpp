@@ -51,7 +51,9 @@ int fail(int code, const char *fmt, ...) {
 
 namespace {
 
-constexpr int64_t kChunk = 2ll << 20;  // vmm_allocator.h:45 granularitySize
+constexpr int64_t kMinChunk = 2ll << 20;  // vmm_allocator.h:45 granularitySize
+// bytes of one physical chunk: the reference's 2 MiB unless vtkv_pool_set_chunk_bytes has asked for more
+int64_t g_chunk = kMinChunk;
 
 }  // namespace
 }  // namespace vtkv
@@ -107,7 +109,7 @@ hipError_t take_range_locked(int64_t bytes, char **out) {
     return hipSuccess;
   }
   void *p = nullptr;
-  const hipError_t e = hipMemAddressReserve(&p, bytes, kChunk, nullptr, 0);
+  const hipError_t e = hipMemAddressReserve(&p, bytes, g_chunk, nullptr, 0);
   *out = (char *)p;
   if (e == hipSuccess) {
     ++g_pool.ranges_reserved;
@@ -135,7 +137,7 @@ struct vtkv_segment {
 };
 
 using vtkv::g_pool;
-using vtkv::kChunk;
+using vtkv::g_chunk;
 
 namespace {
 
@@ -156,12 +158,12 @@ int map_chunks_locked(vtkv_segment *s, int n) {
   for (int l = 0; l < s->layer_num && err == hipSuccess; ++l) {
     for (int j = 0; j < n && err == hipSuccess; ++j) {
       for (int which = 0; which < 2 && err == hipSuccess; ++which) {
-        char *va = (which ? s->v_base[l] : s->k_base[l]) + s->held + (int64_t)j * kChunk;
+        char *va = (which ? s->v_base[l] : s->k_base[l]) + s->held + (int64_t)j * g_chunk;
         hipMemGenericAllocationHandle_t h = g_pool.free_chunks.back();
-        err = hipMemMap(va, kChunk, 0, h, 0);
+        err = hipMemMap(va, g_chunk, 0, h, 0);
         if (err != hipSuccess) {
           snprintf(where, sizeof(where), " (hipMemMap, %s range of layer %d, offset %lld of %lld)", which ? "V" : "K", l,
-                   (long long)(s->held + (int64_t)j * kChunk), (long long)s->context_max);
+                   (long long)(s->held + (int64_t)j * g_chunk), (long long)s->context_max);
           break;
         }
         g_pool.free_chunks.pop_back();
@@ -170,16 +172,16 @@ int map_chunks_locked(vtkv_segment *s, int n) {
         list->push_back(h);
         done.push_back({va, h, list});
         // (one call over several chunks costs the same per chunk: measured 28 us each either way)
-        err = hipMemSetAccess(va, kChunk, &ad, 1);
+        err = hipMemSetAccess(va, g_chunk, &ad, 1);
         if (err != hipSuccess)
           snprintf(where, sizeof(where), " (hipMemSetAccess, %s range of layer %d, offset %lld of %lld)", which ? "V" : "K",
-                   l, (long long)(s->held + (int64_t)j * kChunk), (long long)s->context_max);
+                   l, (long long)(s->held + (int64_t)j * g_chunk), (long long)s->context_max);
       }
     }
   }
   if (err != hipSuccess) {
     for (auto it = done.rbegin(); it != done.rend(); ++it) {
-      (void)hipMemUnmap(it->va, kChunk);
+      (void)hipMemUnmap(it->va, g_chunk);
       it->list->pop_back();
       g_pool.free_chunks.push_back(it->h);
     }
@@ -188,7 +190,7 @@ int map_chunks_locked(vtkv_segment *s, int n) {
                       (long long)g_pool.maps, (long long)g_pool.pairs, (long long)g_pool.recreated, (long long)g_pool.ranges_reserved,
                       (long long)(g_pool.bytes_reserved >> 20));
   }
-  s->held += (int64_t)n * kChunk;
+  s->held += (int64_t)n * g_chunk;
   s->mapped = s->held;
   return VTKV_OK;
 }
@@ -235,7 +237,7 @@ void release_handle_locked(hipMemGenericAllocationHandle_t h) {
     prop.location.id = g_pool.device;
     hipMemGenericAllocationHandle_t fresh;
     // (if the new chunk cannot be had now, the old one serves on and is tried again after its next cycle)
-    if (hipMemCreate(&fresh, kChunk, &prop, 0) == hipSuccess) {
+    if (hipMemCreate(&fresh, g_chunk, &prop, 0) == hipSuccess) {
       g_pool.cycles.erase(cyc);
       g_pool.pairs -= n;
       (void)hipMemRelease(h);
@@ -249,21 +251,21 @@ void release_handle_locked(hipMemGenericAllocationHandle_t h) {
 // Physically unmap the retired chunks of `s` at offsets >= max(keep_held, mapped), top down, at most
 // `max_rows` chunk rows (one row = one chunk of every range; < 0: all).  Returns rows unmapped or < 0.
 int64_t trim_segment_locked(vtkv_segment *s, int64_t keep_held, int64_t max_rows) {
-  const int64_t floor_n = std::max(keep_held, s->mapped) / kChunk;
+  const int64_t floor_n = std::max(keep_held, s->mapped) / g_chunk;
   int64_t rows = 0;
-  while (s->held / kChunk > floor_n && (max_rows < 0 || rows < max_rows)) {
-    const int64_t top = s->held / kChunk - 1;
+  while (s->held / g_chunk > floor_n && (max_rows < 0 || rows < max_rows)) {
+    const int64_t top = s->held / g_chunk - 1;
     for (int l = 0; l < s->layer_num; ++l) {
       for (int which = 0; which < 2; ++which) {
         auto &list = which ? s->v_chunks[l] : s->k_chunks[l];
         char *base = which ? s->v_base[l] : s->k_base[l];
         // one call per mapping: each chunk was mapped on its own
-        VTKV_HIP(hipMemUnmap(base + top * kChunk, kChunk));
+        VTKV_HIP(hipMemUnmap(base + top * g_chunk, g_chunk));
         release_handle_locked(list.back());
         list.pop_back();
       }
     }
-    s->held -= kChunk;
+    s->held -= g_chunk;
     g_pool.retired -= 2ll * s->layer_num;
     ++rows;
   }
@@ -286,24 +288,24 @@ int reclaim_locked(int64_t need) {
 
 int expand_locked(vtkv_segment *s, int n) {
   if (n <= 0) return VTKV_OK;
-  if (s->mapped + (int64_t)n * kChunk > s->context_max)
+  if (s->mapped + (int64_t)n * g_chunk > s->context_max)
     return vtkv::fail(VTKV_EINVAL, "segment would grow to %lld bytes, beyond its reserved %lld",
-                      (long long)(s->mapped + (int64_t)n * kChunk), (long long)s->context_max);
+                      (long long)(s->mapped + (int64_t)n * g_chunk), (long long)s->context_max);
   // the segment's own retired chunks are still mapped right where it grows: take them back first
-  const int revive = (int)std::min<int64_t>(n, (s->held - s->mapped) / kChunk);
+  const int revive = (int)std::min<int64_t>(n, (s->held - s->mapped) / g_chunk);
   const int fresh = n - revive;
   const int64_t need = 2ll * s->layer_num * fresh;
   // (its retired chunks beyond `revive` are none when fresh > 0, so reclaiming never touches `s`)
   if (fresh > 0 && (int64_t)g_pool.free_chunks.size() + g_pool.retired - 2ll * s->layer_num * revive < need)
     return vtkv::fail(VTKV_ENOMEM, "chunk pool exhausted: need %lld, free %lld", (long long)need,
                       (long long)((int64_t)g_pool.free_chunks.size() + g_pool.retired - 2ll * s->layer_num * revive));
-  s->mapped += (int64_t)revive * kChunk;
+  s->mapped += (int64_t)revive * g_chunk;
   g_pool.retired -= 2ll * s->layer_num * revive;
   if (fresh == 0) return VTKV_OK;
   int rc = reclaim_locked(need);
   if (rc >= 0) rc = map_chunks_locked(s, fresh);
   if (rc < 0) {  // leave the segment as it was
-    s->mapped -= (int64_t)revive * kChunk;
+    s->mapped -= (int64_t)revive * g_chunk;
     g_pool.retired += 2ll * s->layer_num * revive;
   }
   return rc;
@@ -313,7 +315,7 @@ int expand_locked(vtkv_segment *s, int n) {
 // until the pool needs them; see the note at the top of the file.
 int shrink_locked(vtkv_segment *s, int64_t keep_bytes) {
   if (keep_bytes >= s->mapped) return VTKV_OK;
-  const int64_t keep_n = keep_bytes / kChunk;
+  const int64_t keep_n = keep_bytes / g_chunk;
   // Chunks that another segment maps as well cannot be counted as free while they sit here retired:
   // if any of the chunks given up is shared, everything above `keep` is unmapped right away.
   bool any_shared = false;
@@ -321,10 +323,10 @@ int shrink_locked(vtkv_segment *s, int64_t keep_bytes) {
     for (int l = 0; l < s->layer_num && !any_shared; ++l)
       for (int which = 0; which < 2 && !any_shared; ++which) {
         const auto &list = which ? s->v_chunks[l] : s->k_chunks[l];
-        for (int64_t j = keep_n; j < s->mapped / kChunk && !any_shared; ++j) any_shared = g_pool.shared.count(list[j]) != 0;
+        for (int64_t j = keep_n; j < s->mapped / g_chunk && !any_shared; ++j) any_shared = g_pool.shared.count(list[j]) != 0;
       }
-  g_pool.retired += 2ll * s->layer_num * (s->mapped / kChunk - keep_n);
-  s->mapped = keep_n * kChunk;
+  g_pool.retired += 2ll * s->layer_num * (s->mapped / g_chunk - keep_n);
+  s->mapped = keep_n * g_chunk;
   if (any_shared && trim_segment_locked(s, keep_bytes, -1) < 0) return VTKV_EHIP;
   return VTKV_OK;
 }
@@ -352,9 +354,9 @@ void worker_main() {
       g_pool.done_cv.notify_all();
       continue;
     }
-    int n = (int)std::min<int64_t>(rq.chunks, (s->context_max - s->mapped) / kChunk);
-    const int revive = (int)std::min<int64_t>(n, (s->held - s->mapped) / kChunk);
-    s->mapped += (int64_t)revive * kChunk;
+    int n = (int)std::min<int64_t>(rq.chunks, (s->context_max - s->mapped) / g_chunk);
+    const int revive = (int)std::min<int64_t>(n, (s->held - s->mapped) / g_chunk);
+    s->mapped += (int64_t)revive * g_chunk;
     g_pool.retired -= 2ll * s->layer_num * revive;
     n -= revive;
     const int64_t need = 2ll * s->layer_num * n;
@@ -376,19 +378,19 @@ void worker_main() {
       size_t done = 0;  // handle index i maps range (layer, which) = (i / (2n), (i / n) % 2), chunk i % n
       auto va_of = [&](size_t i) {
         const int l = (int)(i / (2 * (size_t)n)), which = (int)((i / n) % 2), j = (int)(i % n);
-        return (which ? s->v_base[l] : s->k_base[l]) + at + (int64_t)j * kChunk;
+        return (which ? s->v_base[l] : s->k_base[l]) + at + (int64_t)j * g_chunk;
       };
       for (; done < handles.size() && err == hipSuccess; ++done) {
-        err = hipMemMap(va_of(done), kChunk, 0, handles[done], 0);
+        err = hipMemMap(va_of(done), g_chunk, 0, handles[done], 0);
         if (err != hipSuccess) break;
-        err = hipMemSetAccess(va_of(done), kChunk, &ad, 1);
+        err = hipMemSetAccess(va_of(done), g_chunk, &ad, 1);
         if (err != hipSuccess) {
-          (void)hipMemUnmap(va_of(done), kChunk);
+          (void)hipMemUnmap(va_of(done), g_chunk);
           break;
         }
       }
       if (err != hipSuccess)
-        for (size_t i = 0; i < done; ++i) (void)hipMemUnmap(va_of(i), kChunk);
+        for (size_t i = 0; i < done; ++i) (void)hipMemUnmap(va_of(i), g_chunk);
       lk.lock();
       for (size_t i = 0; i < std::min(done + 1, handles.size()); ++i) note_mapping_locked(handles[i]);
       if (err == hipSuccess) {
@@ -396,7 +398,7 @@ void worker_main() {
           for (int which = 0; which < 2; ++which)
             for (int j = 0; j < n; ++j)
               (which ? s->v_chunks[l] : s->k_chunks[l]).push_back(handles[((size_t)l * 2 + which) * n + j]);
-        s->held += (int64_t)n * kChunk;
+        s->held += (int64_t)n * g_chunk;
         s->mapped = s->held;
       } else {
         for (auto h : handles) g_pool.free_chunks.push_back(h);
@@ -411,7 +413,7 @@ void worker_main() {
 int ensure_locked(vtkv_segment *s, int64_t token_bytes) {
   if (s->used + token_bytes <= s->mapped) return 0;
   const int64_t gap = s->used + token_bytes - s->mapped;
-  const int n = (int)((gap + kChunk - 1) / kChunk);
+  const int n = (int)((gap + g_chunk - 1) / g_chunk);
   int rc = expand_locked(s, n);
   return rc < 0 ? rc : 1;
 }
@@ -420,11 +422,11 @@ int reserve_locked(vtkv_segment *s, int64_t token_bytes, int64_t kv_size) {
   // vmm_allocator.cpp:322-337: room for the new rows plus a 100-row slack, rounded up to chunks
   const int64_t want = s->used + token_bytes + 100 * kv_size;
   if (want > s->mapped) {
-    int64_t n = (want - s->mapped + kChunk - 1) / kChunk;
+    int64_t n = (want - s->mapped + g_chunk - 1) / g_chunk;
     // the slack must not push a sequence past its reserved range
-    const int64_t room = (s->context_max - s->mapped) / kChunk;
+    const int64_t room = (s->context_max - s->mapped) / g_chunk;
     if (n > room) n = room;
-    if (s->used + token_bytes > s->mapped + n * kChunk)
+    if (s->used + token_bytes > s->mapped + n * g_chunk)
       return vtkv::fail(VTKV_EINVAL, "sequence of %lld bytes does not fit its reserved %lld",
                         (long long)(s->used + token_bytes), (long long)s->context_max);
     int rc = expand_locked(s, (int)n);
@@ -440,7 +442,20 @@ extern "C" {
 
 const char *vtkv_last_error(void) { return vtkv::error_buffer(); }
 int vtkv_version(void) { return 100; }
-int64_t vtkv_chunk_bytes(void) { return kChunk; }
+int64_t vtkv_chunk_bytes(void) { return g_chunk; }
+
+int vtkv_pool_set_chunk_bytes(int64_t bytes) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  VTKV_REQUIRE(bytes >= vtkv::kMinChunk && bytes <= (1ll << 30) && (bytes & (bytes - 1)) == 0,
+               "chunk size %lld is not a power of two between 2 MiB and 1 GiB", (long long)bytes);
+  if (bytes == g_chunk) return VTKV_OK;
+  // chunks, segments and the kept address ranges are all laid out in units of the current size
+  if (g_pool.total != 0 || !g_pool.segments.empty() || !g_pool.spare_ranges.empty())
+    return vtkv::fail(VTKV_ESTATE, "the chunk size can only change while the pool is empty (before vtkv_pool_init "
+                                   "or after vtkv_pool_destroy)");
+  g_chunk = bytes;
+  return VTKV_OK;
+}
 
 int vtkv_pool_init(int device, int64_t num_chunks) {
   std::unique_lock<std::mutex> lk(g_pool.mu);
@@ -457,18 +472,19 @@ int vtkv_pool_init(int device, int64_t num_chunks) {
   prop.location.id = device;
   size_t gran = 0;
   VTKV_HIP(hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityMinimum));
-  if (gran == 0 || kChunk % (int64_t)gran != 0)
-    return vtkv::fail(VTKV_EHIP, "allocation granularity %zu does not divide the 2 MiB chunk", gran);
+  if (gran == 0 || g_chunk % (int64_t)gran != 0)
+    return vtkv::fail(VTKV_EHIP, "allocation granularity %zu does not divide the chunk size", gran);
   if (g_pool.total + num_chunks > kMaxPoolChunks)
     return vtkv::fail(VTKV_EINVAL,
                       "a pool of %lld chunks is more than this HIP runtime can serve: a process has 65536 entries for "
-                      "chunks and (chunk, address) mappings together; at most %lld chunks of 2 MiB",
-                      (long long)(g_pool.total + num_chunks), (long long)kMaxPoolChunks);
+                      "chunks and (chunk, address) mappings together; at most %lld chunks (of %lld MiB; "
+                      "vtkv_pool_set_chunk_bytes makes them larger)",
+                      (long long)(g_pool.total + num_chunks), (long long)kMaxPoolChunks, (long long)(g_chunk >> 20));
   g_pool.device = device;
   g_pool.free_chunks.reserve(g_pool.free_chunks.size() + num_chunks);
   for (int64_t i = 0; i < num_chunks; ++i) {
     hipMemGenericAllocationHandle_t h;
-    hipError_t e = hipMemCreate(&h, kChunk, &prop, 0);
+    hipError_t e = hipMemCreate(&h, g_chunk, &prop, 0);
     if (e != hipSuccess)
       return vtkv::fail(VTKV_ENOMEM, "hipMemCreate failed after %lld of %lld chunks: %s", (long long)i,
                         (long long)num_chunks, hipGetErrorString(e));
@@ -541,9 +557,9 @@ vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t 
     vtkv::fail(VTKV_ESTATE, "vtkv_pool_init has not been called");
     return nullptr;
   }
-  if (layer_num <= 0 || context_max_bytes <= 0 || context_max_bytes % kChunk != 0 || expand_bytes < 0 ||
-      expand_bytes % kChunk != 0 || expand_bytes > context_max_bytes) {
-    vtkv::fail(VTKV_EINVAL, "layer_num must be > 0 and sizes multiples of the 2 MiB chunk (max %lld, expand %lld)",
+  if (layer_num <= 0 || context_max_bytes <= 0 || context_max_bytes % g_chunk != 0 || expand_bytes < 0 ||
+      expand_bytes % g_chunk != 0 || expand_bytes > context_max_bytes) {
+    vtkv::fail(VTKV_EINVAL, "layer_num must be > 0 and sizes multiples of the chunk size (max %lld, expand %lld)",
                (long long)context_max_bytes, (long long)expand_bytes);
     return nullptr;
   }
@@ -570,7 +586,7 @@ vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t 
     s->v_base.push_back(v);
   }
   if (expand && expand_bytes > 0) {
-    if (expand_locked(s, (int)(expand_bytes / kChunk)) < 0) {
+    if (expand_locked(s, (int)(expand_bytes / g_chunk)) < 0) {
       for (char *p : s->k_base) vtkv::give_range_locked(p, context_max_bytes);
       for (char *p : s->v_base) vtkv::give_range_locked(p, context_max_bytes);
       delete s;
@@ -708,8 +724,8 @@ int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, v
   VTKV_REQUIRE(bytes >= 0 && bytes <= src->used && src->used <= src->mapped, "prefix of %lld bytes exceeds the source's %lld",
                (long long)bytes, (long long)src->used);
   VTKV_REQUIRE(dst->mapped == 0 && dst->used == 0, "the destination segment must be empty");
-  const int64_t whole = bytes / kChunk, tail = bytes % kChunk;
-  VTKV_REQUIRE((whole + (tail ? 1 : 0)) * kChunk <= dst->context_max, "prefix does not fit the destination's range");
+  const int64_t whole = bytes / g_chunk, tail = bytes % g_chunk;
+  VTKV_REQUIRE((whole + (tail ? 1 : 0)) * g_chunk <= dst->context_max, "prefix does not fit the destination's range");
   if (trim_segment_locked(dst, 0, -1) < 0) return VTKV_EHIP;  // its retired chunks would be in the way
   if (tail && (int64_t)g_pool.free_chunks.size() + g_pool.retired < 2ll * dst->layer_num)
     return vtkv::fail(VTKV_ENOMEM, "chunk pool exhausted: need %lld, free %lld", 2ll * dst->layer_num,
@@ -728,18 +744,18 @@ int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, v
       auto &to = which ? dst->v_chunks[l] : dst->k_chunks[l];
       char *base = which ? dst->v_base[l] : dst->k_base[l];
       for (int64_t j = 0; j < whole && err == hipSuccess; ++j) {
-        char *va = base + j * kChunk;
-        err = hipMemMap(va, kChunk, 0, from[j], 0);
+        char *va = base + j * g_chunk;
+        err = hipMemMap(va, g_chunk, 0, from[j], 0);
         if (err != hipSuccess) break;
         note_mapping_locked(from[j]);
         to.push_back(from[j]);
         done.push_back({va, &to, from[j]});
-        err = hipMemSetAccess(va, kChunk, &ad, 1);
+        err = hipMemSetAccess(va, g_chunk, &ad, 1);
       }
     }
   if (err != hipSuccess) {
     for (auto it = done.rbegin(); it != done.rend(); ++it) {
-      (void)hipMemUnmap(it->va, kChunk);
+      (void)hipMemUnmap(it->va, g_chunk);
       it->list->pop_back();
     }
     return vtkv::fail(VTKV_EHIP, "mapping a shared chunk failed: %s", hipGetErrorString(err));
@@ -748,7 +764,7 @@ int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, v
     auto it = g_pool.shared.find(d.h);
     if (it == g_pool.shared.end()) g_pool.shared[d.h] = 2; else ++it->second;
   }
-  dst->held = dst->mapped = whole * kChunk;
+  dst->held = dst->mapped = whole * g_chunk;
   if (tail) {
     // the partly filled chunk is the destination's own: both sequences go on writing behind the prefix
     int rc = expand_locked(dst, 1);
@@ -758,8 +774,8 @@ int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, v
     }
     for (int l = 0; l < dst->layer_num; ++l)
       for (int which = 0; which < 2; ++which) {
-        char *to = (which ? dst->v_base[l] : dst->k_base[l]) + whole * kChunk;
-        const char *from = (which ? src->v_base[l] : src->k_base[l]) + whole * kChunk;
+        char *to = (which ? dst->v_base[l] : dst->k_base[l]) + whole * g_chunk;
+        const char *from = (which ? src->v_base[l] : src->k_base[l]) + whole * g_chunk;
         VTKV_HIP(hipMemcpyAsync(to, from, (size_t)tail, hipMemcpyDeviceToDevice, (hipStream_t)stream));
       }
   }

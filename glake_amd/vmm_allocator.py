@@ -26,8 +26,20 @@ from . import _C
 granularitySize = 2 * 1024 * 1024  # vmm_allocator.h:45
 
 
+def chunkBytes() -> int:
+    """Bytes of one physical chunk: ``granularitySize`` unless ``set_chunk_bytes`` asked for more."""
+    return int(_C.lib().vtkv_chunk_bytes())
+
+
+def set_chunk_bytes(nbytes: int) -> None:
+    """Chunks of ``nbytes`` (a power of two from 2 MiB to 1 GiB) from the next ``init_physical_handle`` on; only
+    while the pool is empty.  The reference's granularity is fixed; with this HIP runtime a pool holds at most
+    30000 chunks, so a cache above 58 GiB needs larger ones.  No counterpart in the reference."""
+    _C.check(_C.lib().vtkv_pool_set_chunk_bytes(int(nbytes)))
+
+
 def init_physical_handle(num_blocks: int, device_id: int) -> bool:
-    """Create ``num_blocks`` 2 MiB physical chunks on ``device_id`` (vmm_allocator.cpp:113-151)."""
+    """Create ``num_blocks`` physical chunks (2 MiB each by default) on ``device_id`` (vmm_allocator.cpp:113-151)."""
     _C.check(_C.lib().vtkv_pool_init(int(device_id), int(num_blocks)))
     return True
 

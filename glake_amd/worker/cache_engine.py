@@ -16,7 +16,6 @@ import torch
 
 from .. import _C, _custom_ops as ops, vmm_allocator as vmm
 
-PHY_GRAN = 2 * 1024 * 1024  # cache_engine.py:54
 
 
 def _dtype_size(dtype: torch.dtype) -> int:
@@ -72,10 +71,11 @@ class CacheEngine:
         self.token_size = num_kv_heads * head_size * _dtype_size(dtype)  # bytes of one K (or V) row
         # cache_engine.py:53-57: every slot reserves room for max_num_batched_tokens rows
         ctx = max_num_batched_tokens * self.token_size
-        self.max_context_size = PHY_GRAN * ((ctx + PHY_GRAN - 1) // PHY_GRAN)
+        gran = self.chunk_bytes = vmm.chunkBytes()  # 2 MiB (cache_engine.py:54) unless the pool was given larger chunks
+        self.max_context_size = gran * ((ctx + gran - 1) // gran)
         self.kv_batch_stride = self.max_context_size
         # cache_engine.py:58-71: the first cache_seqs slots keep cache_tokens chunks mapped
-        keep = PHY_GRAN * cache_tokens if cache_seqs > 0 else 0
+        keep = gran * cache_tokens if cache_seqs > 0 else 0
         self.vmm_kvcache_segment = [
             vmm.KVcacheSegment(num_layers, self.max_context_size, keep, cache_seqs > 0 and i < cache_seqs)
             for i in range(max_num_seqs)
@@ -144,7 +144,7 @@ class CacheEngine:
                 raise _C.VtkvError(_C.ESTATE, f"slot {slot} is not swapped out")
             off, used = self._swapped[slot]
             seg = self.vmm_kvcache_segment[slot]
-            need = (used + PHY_GRAN - 1) // PHY_GRAN - seg.actual_size // PHY_GRAN
+            need = (used + self.chunk_bytes - 1) // self.chunk_bytes - seg.actual_size // self.chunk_bytes
             if need > 0:
                 seg.expandMultiSegment(need)
             seg.set_used_size(used)

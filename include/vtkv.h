@@ -48,13 +48,21 @@ int vtkv_version(void);
  * Replaces the pybind module `vmmAllocator` (vmm_allocator/vmm_allocator.h:190-219).
  * ---------------------------------------------------------------------------------------- */
 
-/* Size of one physical chunk in bytes (2 MiB; vmm_allocator/vmm_allocator.h:45 granularitySize). */
+/* Size of one physical chunk in bytes (2 MiB unless changed; vmm_allocator/vmm_allocator.h:45
+ * granularitySize). */
 int64_t vtkv_chunk_bytes(void);
+/* Use chunks of `bytes` (a power of two from 2 MiB to 1 GiB) from the next vtkv_pool_init on.  Only while the
+ * pool is empty: before the first vtkv_pool_init or after vtkv_pool_destroy (VTKV_ESTATE otherwise).  The
+ * reference's granularity is fixed at 2 MiB; a pool holds at most 30000 chunks with this HIP runtime (see
+ * vtkv_pool_init), so a cache above 58 GiB needs larger ones: 16 MiB chunks serve up to 468 GiB.  Every size
+ * and offset the other calls take in chunks or require to be chunk multiples then refers to this size. */
+int vtkv_pool_set_chunk_bytes(int64_t bytes);
 
 /* Create `num_chunks` physical chunks on `device` and keep them in the free pool.
  * Replaces init_physical_handle(num_blocks, device_id) (vmm_allocator.cpp:113-151).
  * May be called again to add chunks.  At most 30000 chunks in all (VTKV_EINVAL beyond): the HIP runtime
- * has 65536 entries per process for physical chunks and their mappings together. */
+ * has 65536 entries per process for physical chunks and their mappings together; larger caches take larger
+ * chunks (vtkv_pool_set_chunk_bytes). */
 int vtkv_pool_init(int device, int64_t num_chunks);
 /* Chunks no sequence owns; replaces showFreeBlocks() (vmm_allocator.cpp:472-474). <0 on error.
  * Unmapping is lazy: a segment that shrinks (preempt, release, swap-out) keeps its chunks mapped at the

@@ -24,8 +24,9 @@ class GpuSeqs:
 
     def __init__(self, vmm, num_slots, num_kv_heads, head_size, elem_bytes, max_tokens, layers=1):
         self.vmm = vmm
+        self.chunk = vmm.chunkBytes()  # CHUNK unless the pool was set up with larger chunks
         self.row_bytes = num_kv_heads * head_size * elem_bytes
-        self.max_bytes = round_up(max_tokens * self.row_bytes, CHUNK)
+        self.max_bytes = round_up(max_tokens * self.row_bytes, self.chunk)
         self.segs = [vmm.KVcacheSegment(layers, self.max_bytes, 0, False) for _ in range(num_slots)]
         self.layers = layers
         self.k_tables = [vmm.KVCache(num_slots) for _ in range(layers)]
@@ -38,9 +39,9 @@ class GpuSeqs:
 
         seg = self.segs[slot]
         nbytes = k_rows.nbytes
-        need = round_up(nbytes, CHUNK) - seg.actual_size
+        need = round_up(nbytes, self.chunk) - seg.actual_size
         if need > 0:
-            seg.expandMultiSegment(need // CHUNK)
+            seg.expandMultiSegment(need // self.chunk)
         k_rows = np.ascontiguousarray(k_rows)
         v_rows = np.ascontiguousarray(v_rows)
         _C.check(_C.lib().vtkv_memcpy_h2d(seg.getKeyDevicePtr(layer), k_rows.ctypes.data_as(C.c_void_p), nbytes))
@@ -53,9 +54,9 @@ class GpuSeqs:
 
         zeros = np.zeros(nbytes, np.uint8)
         for seg in self.segs:
-            need = round_up(nbytes, CHUNK) - seg.actual_size
+            need = round_up(nbytes, self.chunk) - seg.actual_size
             if need > 0:
-                seg.expandMultiSegment(need // CHUNK)
+                seg.expandMultiSegment(need // self.chunk)
             for dst in (seg.getKeyDevicePtr(layer), seg.getValueDevicePtr(layer)):
                 _C.check(_C.lib().vtkv_memcpy_h2d(dst, zeros.ctypes.data_as(C.c_void_p), nbytes))
 
