@@ -919,12 +919,15 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   // the counters come first, at a place that does not depend on the sizes of a call
   p.seg_count = (uint32_t *)workspace;
   // Merging inside the streaming kernel saves the second launch, but the workgroup that arrives last
-  // does it at the very end of the kernel with device-coherent round trips (about 6 us).  That pays when
-  // most (sequence, kv head) segments lie inside one workgroup and need no merge at all (measured: +4.5 %
-  // per step at 2048 segments on 512 workgroups, +1.5 % at 1024, -1.6 % at 512), so it is the default
-  // from two segments per workgroup on.
-  p.fused_merge =
-      g_fused_merge == 1 || (g_fused_merge < 0 && (int64_t)num_seqs * (num_kv_heads / seg_heads) >= 2 * grid);
+  // does it at the very end of the kernel with device-coherent round trips (about 6 us), and every shared
+  // segment costs its workgroups coherent stores and an arrival.  That pays when most (sequence, kv head)
+  // segments lie inside one workgroup and need no merge at all.  Measured on 512 workgroups with ragged
+  // lengths, stream kernel + merge, inside against separate (the separate form also lets every XCD take a
+  // contiguous part of the tile order): 1024 segments 188 against 180 us (group 4) and 196 against 192 us
+  // (group 8); 1280 segments 212 / 209 and 219 / 221; 1536 segments 206 / 205 and 217 / 222; 2048 segments
+  // 201.5 / 212 and 216 / 231.  Hence inside from two and a half segments per workgroup on.
+  p.fused_merge = g_fused_merge == 1 ||
+                  (g_fused_merge < 0 && 2 * (int64_t)num_seqs * (num_kv_heads / seg_heads) >= 5 * grid);
   p.heads_per_seg = seg_heads;
   p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
   p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);

@@ -312,7 +312,8 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
 
 /* Where the partial results of the workgroups that share a (sequence, kv head) are merged: 1 = inside the
  * attention kernel, by whichever of them finishes last; 0 = by a second kernel; -1 (the default) = inside
- * when the batch has at least two (sequence, kv head) pairs per workgroup, so that most need no merge.
+ * when the batch has at least two and a half (sequence, kv head) pairs per workgroup, so that most need no
+ * merge.
  * For A/B measurements; results agree up to fp32 summation order.  No counterpart in the reference. */
 int vtkv_set_fused_merge(int on);
 
