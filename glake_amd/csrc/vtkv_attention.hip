@@ -129,20 +129,22 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // bf16 in registers (K) or on the way into the LDS tile (V); the per-tensor scales are folded into the
 // logit scale (K) and into the final normalisation (V), so dequantisation costs no multiply per element.
 //
-// PAIR: an fp8 head row is 128 bytes, and a stream of isolated 128-byte pieces (one per token, the kv heads
-// of a token being 128 bytes apart) reaches about 6.1 TB/s on this part where 256-byte pieces reach 6.9 to
-// 7.1, whichever workgroup fetches the neighbouring piece.  The PAIR variants therefore make a pair of
-// adjacent kv heads the unit of the tile order: a segment is (sequence, head pair), waves 0 and 2 take the
-// even head of the pair and waves 1 and 3 the odd one, over the same rows at about the same time, so the
-// two 128-byte halves of a 256-byte piece are requested together from one CU.  Everything a wave does is
-// unchanged; only two waves instead of four share a head's tiles and its end-of-segment merge.
+// HPS (kv heads per segment) = 2: a pair of adjacent kv heads is the unit of the tile order: a segment is
+// (sequence, head pair), waves 0 and 2 take the even head of the pair and waves 1 and 3 the odd one, over the
+// same rows at about the same time.  Everything a wave does is unchanged; only two waves instead of four
+// share a head's tiles and its end-of-segment merge.  Two uses.  An fp8 head row is 128 bytes, and a stream
+// of isolated 128-byte pieces (one per token, the kv heads of a token being 128 bytes apart) reaches about
+// 6.1 TB/s on this part where 256-byte pieces reach 6.9 to 7.1, whichever workgroup fetches the
+// neighbouring piece: with pairs the two 128-byte halves of a 256-byte piece are requested together from
+// one CU.  And a batch of very many short sequences pays the start and the merge of a segment half as
+// often.
 //
 // APPEND: seq_lens count the step's new token, whose K/V row is not in the cache yet but in new_k /
 // new_v.  The rows before it are read from the cache as usual; the new row forms one more tile of its
 // own at the end of the sequence's tile list, loaded from new_k / new_v, and the wave that handles it
 // also stores the row into the cache.  One launch then does reshape_and_cache and attention, and each
 // byte of the new rows is read once.
-template <bool ALIBI, bool FP8, bool APPEND, bool PAIR>
+template <bool ALIBI, bool FP8, bool APPEND, int HPS>
 __global__ void __launch_bounds__(kThreads)
     __attribute__((amdgpu_waves_per_eu(FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES)))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
@@ -157,7 +159,7 @@ __global__ void __launch_bounds__(kThreads)
   __shared__ int s_wave_tot[kWaves];
   // pieces of shared (sequence, kv head) segments this workgroup has written: segment, first and last
   // workgroup of the segment, and whether this workgroup delivered the last piece
-  __shared__ int s_pend[4][4];
+  __shared__ int s_pend[8][4];
   __shared__ int s_npend;
 
   const int lane = threadIdx.x & 63;
@@ -168,10 +170,12 @@ __global__ void __launch_bounds__(kThreads)
   const int G = p.group;
   const int Hkv = p.num_kv_heads;
   const int B = p.num_seqs;
-  constexpr int kHps = PAIR ? 2 : 1;           // kv heads per segment
+  static_assert(HPS == 1 || HPS == 2 || HPS == 4, "1, 2 or 4 kv heads per segment");  // (4 measured: no better than 2)
+  constexpr int kHps = HPS;                    // kv heads per segment
+  constexpr bool PAIR = HPS > 1;
   constexpr int kWph = kWaves / kHps;          // waves that share a head's tiles
-  const int side = PAIR ? (wave & 1) : 0;      // this wave's head inside the segment
-  const int ws = PAIR ? (wave >> 1) : wave;    // its place among the waves of that head
+  const int side = wave % kHps;                // this wave's head inside the segment
+  const int ws = wave / kHps;                  // its place among the waves of that head
   const int Hseg = Hkv / kHps;                 // segments per sequence
   auto len_of = [&](int idx) { return p.inline_lens ? il.v[idx] : p.seq_lens[idx]; };
   // tiles of one kv head of a sequence: its cached rows in 16s, plus the new row's own tile
@@ -656,13 +660,13 @@ __global__ void __launch_bounds__(kThreads)
     __syncthreads();
     const int np = uniform(s_npend);
     if (np == 0) return;
-    if (lane == 0 && wave < np) {
-      const int seg = s_pend[wave][0];
-      const unsigned pieces = (unsigned)(s_pend[wave][2] - s_pend[wave][1] + 1);
+    for (int k = wave; k < np && lane == 0; k += kWaves) {
+      const int seg = s_pend[k][0];
+      const unsigned pieces = (unsigned)(s_pend[k][2] - s_pend[k][1] + 1);
       const unsigned old = __hip_atomic_fetch_add(&p.seg_count[seg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last_piece = old + 1 == pieces;
       if (last_piece) __hip_atomic_store(&p.seg_count[seg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_pend[wave][3] = last_piece;
+      s_pend[k][3] = last_piece;
     }
     __syncthreads();
     const int per_seg = G * kD;
@@ -787,7 +791,7 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 12;  // instantiations of the streaming kernel
+constexpr int kVariants = 16;  // instantiations of the streaming kernel
 struct Residency {
   std::mutex mu;
   int device = -1;
@@ -874,20 +878,25 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
 
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   const bool alibi = alibi_slopes != nullptr;
-  // Two adjacent kv heads per segment for fp8 rows (see the kernel).  Slots: 2 * grid + num_seqs * num_kv_heads
-  // of `group` heads each, which the workspace (16 heads per workgroup) holds for groups up to 8.
-  const bool pair = VTKV_ATTN_FP8_PAIR && fp8 && num_kv_heads % 2 == 0 && group <= 8;
+  // kv heads per segment (see the kernel): two for fp8 rows, and for bf16 rows when the batch is made of very
+  // many short segments (16 or more per CU of this part), where halving the number of segment starts and
+  // merges per workgroup is worth 3 to 7 % (1 024 sequences of 64..512 rows: 250 -> 235 us; 512 sequences
+  // of 128..1 024 rows: 219 -> 211 us) while batches of fewer, longer sequences gain nothing or lose (the
+  // merge kernel sees twice the pieces per head: config 3 152 -> 158 us).  Slots: seg_heads * grid +
+  // num_seqs * num_kv_heads of `group` heads each, which the workspace (16 heads per workgroup) holds for
+  // groups up to 8.
+  const bool many_short = (int64_t)num_seqs * num_kv_heads >= 4096;
+  const bool pair = (fp8 ? VTKV_ATTN_FP8_PAIR != 0 : many_short) && num_kv_heads % 2 == 0 && group <= 8;
   const int seg_heads = pair ? 2 : 1;
-  // kernel variant: bit 0 alibi, bit 1 fused append; 0..3 bf16, 4..7 fp8, 8..11 fp8 with paired kv heads
-  const int variant = (fp8 ? (pair ? 8 : 4) : 0) + (append ? 2 : 0) + (alibi ? 1 : 0);
+  // kernel variant: bit 0 alibi, bit 1 fused append, bit 2 paired kv heads, bit 3 fp8
+  const int variant = (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0);
+#define VTKV_ROW(F8, H)                                                                                      \
+  decode_attn_stream_kernel<false, F8, false, H>, decode_attn_stream_kernel<true, F8, false, H>,             \
+      decode_attn_stream_kernel<false, F8, true, H>, decode_attn_stream_kernel<true, F8, true, H>
   static void (*const kKernels[kVariants])(AttnParams, InlineLens) = {
-      decode_attn_stream_kernel<false, false, false, false>, decode_attn_stream_kernel<true, false, false, false>,
-      decode_attn_stream_kernel<false, false, true, false>,  decode_attn_stream_kernel<true, false, true, false>,
-      decode_attn_stream_kernel<false, true, false, false>,  decode_attn_stream_kernel<true, true, false, false>,
-      decode_attn_stream_kernel<false, true, true, false>,   decode_attn_stream_kernel<true, true, true, false>,
-      decode_attn_stream_kernel<false, true, false, true>,   decode_attn_stream_kernel<true, true, false, true>,
-      decode_attn_stream_kernel<false, true, true, true>,    decode_attn_stream_kernel<true, true, true, true>,
+      VTKV_ROW(false, 1), VTKV_ROW(false, 2), VTKV_ROW(true, 1), VTKV_ROW(true, 2),
   };
+#undef VTKV_ROW
   void (*kernel)(AttnParams, InlineLens) = kKernels[variant];
   int64_t grid;
   if (partition_tokens > 0) {

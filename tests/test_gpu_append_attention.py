@@ -125,6 +125,15 @@ def test_fixed_partitions_agree(gpu_pool, pt):
     assert np.abs(got - base).max() <= 2e-3
 
 
+@pytest.mark.parametrize("lens_from", ["host", "device"])
+def test_very_many_short_sequences(gpu_pool, lens_from):
+    # 512 sequences x 8 kv heads = 4096 segments: the variants that stream a pair of kv heads per workgroup
+    rng = np.random.default_rng(5)
+    lens = [int(x) for x in rng.integers(1, 50, 509)] + [900, 1, 17]
+    run_case(gpu_pool, 21, lens, 32, 8, lens_from=lens_from)
+    run_case(gpu_pool, 22, lens, 16, 8, lens_from=lens_from, alibi=True)
+
+
 def test_long_sequence_many_workgroups_per_segment(gpu_pool):
     # one sequence spread over many workgroups plus short ones: the new row's tile is a segment of its own for some
     run_case(gpu_pool, 9, [40000, 1, 2, 5000], 32, 8, lens_from="device")

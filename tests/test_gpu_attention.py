@@ -148,6 +148,25 @@ def test_merge_inside_and_outside_the_kernel(gpu_pool, mode):
         _C.check(lib.vtkv_set_fused_merge(-1))
 
 
+@pytest.mark.parametrize("mode", [-1, 0, 1])
+def test_very_many_short_sequences_pair_their_kv_heads(gpu_pool, mode):
+    """From 4096 (sequence, kv head) segments on the library runs the variants in which a workgroup streams a
+    pair of adjacent kv heads (two waves per head); 540 sequences of 8 kv heads, most of a few rows, a few
+    long enough to be shared by several workgroups, with and without ALiBi, every merge mode."""
+    from glake_amd import _C
+
+    rng = np.random.default_rng(77)
+    lens = [int(x) for x in rng.integers(1, 40, 536)] + [700, 1, 1500, 16]
+    lib = _C.lib()
+    _C.check(lib.vtkv_set_fused_merge(mode))
+    try:
+        run_case(gpu_pool, 41, lens, 32, 8)
+        run_case(gpu_pool, 42, lens[200:], 16, 16, alibi=True, bf16_step_check=False)
+        run_case(gpu_pool, 43, lens, 24, 8, partition_tokens=64)
+    finally:
+        _C.check(lib.vtkv_set_fused_merge(-1))
+
+
 def test_calls_on_two_streams_do_not_share_scratch(gpu_pool):
     """Two batches attend at the same time on two streams, twenty times over; each result equals the one
     the same call gives when it runs alone (the wrapper keeps one scratch buffer per device and stream)."""
