@@ -146,6 +146,8 @@ def main() -> int:
                     help="plan path: separate reshape_and_cache and attention launches instead of the fused one")
     ap.add_argument("--merge", default="auto", choices=["auto", "fused", "separate"],
                     help="where the attention's partial results are merged (auto: the library decides per call)")
+    ap.add_argument("--value-skew", type=int, default=256,
+                    help="bytes between the base of a V range and its first row (0 = the reference's placement)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -177,11 +179,11 @@ def main() -> int:
     kv_dtype = "fp8" if fp8 else "auto"
     row = Hkv * D * eb
     max_tokens = max(ctx0) + total_steps + 1
-    chunks_per_range = (max_tokens * row + (2 << 20) - 1) // (2 << 20)
+    chunks_per_range = (max_tokens * row + args.value_skew + (2 << 20) - 1) // (2 << 20)
     vmm.init_physical_handle(2 * B * chunks_per_range + 16, 0)
     engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.uint8 if fp8 else torch.bfloat16,
                          max_num_seqs=B,
-                         max_num_batched_tokens=max_tokens, swap_space_bytes=1 << 30)
+                         max_num_batched_tokens=max_tokens, swap_space_bytes=1 << 30, value_skew=args.value_skew)
     segs = engine.vmm_kvcache_segment
 
     # ---- resident synthetic KV: N(0,1) -> bf16, written straight into the mapped ranges
@@ -190,7 +192,7 @@ def main() -> int:
     k_scale = v_scale = 6.0 / 448.0 if fp8 else 1.0
     for b in range(B):
         nbytes = ctx0[b] * row
-        segs[b].expandMultiSegment((nbytes + (2 << 20) - 1) // (2 << 20))
+        segs[b].ensure_mapped(nbytes)  # counts the V offset
         for base in (segs[b].getKeyDevicePtr(0), segs[b].getValueDevicePtr(0)):
             t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
             if fp8:

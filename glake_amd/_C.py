@@ -51,6 +51,8 @@ SIGNATURES = {
     "vtkv_seg_destroy": (_i, [_p]),
     "vtkv_seg_key_ptr": (_u64, [_p, _i]),
     "vtkv_seg_value_ptr": (_u64, [_p, _i]),
+    "vtkv_seg_value_skew": (_i64, [_p]),
+    "vtkv_seg_set_value_skew": (_i, [_p, _i64]),
     "vtkv_seg_get_used": (_i64, [_p]),
     "vtkv_seg_set_used": (_i, [_p, _i64]),
     "vtkv_seg_mapped_bytes": (_i64, [_p]),

@@ -35,13 +35,18 @@ class SequenceChunks:
     ``token_size`` is the bytes of one token row of one range (num_kv_heads * head_size * element
     bytes).  ``logical_block_num`` counts K and V chunks together, i.e. two per chunk of rows."""
 
-    def __init__(self, token_size: int, chunk_bytes: int = PHY_GRAN):
+    def __init__(self, token_size: int, chunk_bytes: int = PHY_GRAN, value_skew: int = 0):
         if token_size <= 0:
             raise ValueError("token_size must be positive")
+        if value_skew < 0 or value_skew >= chunk_bytes:
+            raise ValueError("value_skew must lie in [0, chunk_bytes)")
         if chunk_bytes <= 0 or chunk_bytes % PHY_GRAN:
             raise ValueError("chunk_bytes must be a positive multiple of 2 MiB")
         self.token_size = int(token_size)
         self.chunk_bytes = int(chunk_bytes)
+        # bytes by which the engine sets the V rows off from the base of their range (CacheEngine's
+        # value_skew): claimed once, with the first rows, so that the claim bounds what the ranges map
+        self.value_skew = int(value_skew)
         self.reserve_size = 0       # bytes the sequence has claimed per range, a multiple of the chunk
         self.free_size = 0          # claimed bytes not yet written
         self.logical_block_num = 0  # chunks claimed (K + V)
@@ -54,6 +59,7 @@ class SequenceChunks:
         gran = self.chunk_bytes
         need = self.token_size * (num_tokens + plus)
         if self.reserve_size == 0:
+            need += self.value_skew
             rounded = gran * ((need + gran - 1) // gran)
             self.reserve_size = rounded
             self.free_size = rounded - need

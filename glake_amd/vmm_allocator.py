@@ -94,6 +94,23 @@ class KVcacheSegment:
     def getValueDevicePtr(self, layer_index: int) -> int:
         return int(_C.check_ptr(_C.lib().vtkv_seg_value_ptr(self._h, int(layer_index)), "getValueDevicePtr"))
 
+    @property
+    def value_skew(self) -> int:
+        """Bytes between the base of a V range and its first row (0 unless set); ``getValueDevicePtr`` includes
+        them and the segment keeps ``used_size + value_skew <= actual_size``.  With 256 the K and the V row
+        of a token lie in different memory channels.  No counterpart in the reference."""
+        return int(_C.check(_C.lib().vtkv_seg_value_skew(self._h)))
+
+    def set_value_skew(self, nbytes: int) -> None:
+        """Set that offset (a multiple of 256 up to 4096); only while the segment holds no rows.  Pointers
+        fetched before are stale afterwards."""
+        _C.check(_C.lib().vtkv_seg_set_value_skew(self._h, int(nbytes)))
+
+    def ensure_mapped(self, nbytes: int) -> None:
+        """Map what ``nbytes`` more bytes per range behind ``used_size`` need, the V offset included
+        (``vtkv_seg_ensure``); for callers that write rows through the pointers themselves."""
+        _C.check(_C.lib().vtkv_seg_ensure(self._h, int(nbytes)))
+
     # --- accounting
     def get_used_slot(self) -> int:
         return int(_C.check(_C.lib().vtkv_seg_get_used(self._h)))

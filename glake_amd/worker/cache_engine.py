@@ -62,7 +62,7 @@ class _HostArena:
 class CacheEngine:
     def __init__(self, num_layers: int, num_kv_heads: int, head_size: int, dtype: torch.dtype, max_num_seqs: int,
                  max_num_batched_tokens: int, cache_seqs: int = 0, cache_tokens: int = 0,
-                 swap_space_bytes: int = 0, device: int = 0) -> None:
+                 swap_space_bytes: int = 0, device: int = 0, value_skew: int = 256) -> None:
         self.num_layers = num_layers
         self.num_kv_heads = num_kv_heads
         self.head_size = head_size
@@ -70,7 +70,9 @@ class CacheEngine:
         self.device = device
         self.token_size = num_kv_heads * head_size * _dtype_size(dtype)  # bytes of one K (or V) row
         # cache_engine.py:53-57: every slot reserves room for max_num_batched_tokens rows
-        ctx = max_num_batched_tokens * self.token_size
+        # (plus the bytes by which the V rows are set off from the base of their range)
+        self.value_skew = int(value_skew)
+        ctx = max_num_batched_tokens * self.token_size + self.value_skew
         gran = self.chunk_bytes = vmm.chunkBytes()  # 2 MiB (cache_engine.py:54) unless the pool was given larger chunks
         self.max_context_size = gran * ((ctx + gran - 1) // gran)
         self.kv_batch_stride = self.max_context_size
@@ -80,6 +82,9 @@ class CacheEngine:
             vmm.KVcacheSegment(num_layers, self.max_context_size, keep, cache_seqs > 0 and i < cache_seqs)
             for i in range(max_num_seqs)
         ]
+        if self.value_skew:  # before any pointer is fetched
+            for seg in self.vmm_kvcache_segment:
+                seg.set_value_skew(self.value_skew)
         # cache_engine.py:111-129: per layer one pointer table for K and one for V
         self.gpu_cache = [(vmm.KV_cache(max_num_seqs, l), vmm.KV_cache(max_num_seqs, l)) for l in range(num_layers)]
         vmm.copy_kv_cache([k.kv_cache for k, _ in self.gpu_cache], [v.kv_cache for _, v in self.gpu_cache],
@@ -144,7 +149,9 @@ class CacheEngine:
                 raise _C.VtkvError(_C.ESTATE, f"slot {slot} is not swapped out")
             off, used = self._swapped[slot]
             seg = self.vmm_kvcache_segment[slot]
-            need = (used + self.chunk_bytes - 1) // self.chunk_bytes - seg.actual_size // self.chunk_bytes
+            # the V rows start value_skew bytes into their range, so that much more must be mapped
+            span = used + self.value_skew if used else 0
+            need = (span + self.chunk_bytes - 1) // self.chunk_bytes - seg.actual_size // self.chunk_bytes
             if need > 0:
                 seg.expandMultiSegment(need)
             seg.set_used_size(used)

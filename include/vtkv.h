@@ -100,6 +100,19 @@ int vtkv_seg_destroy(vtkv_segment *seg);
  * (vmm_allocator.cpp:299-305).  0 on error. */
 uint64_t vtkv_seg_key_ptr(const vtkv_segment *seg, int layer);
 uint64_t vtkv_seg_value_ptr(const vtkv_segment *seg, int layer);
+/* Offset in bytes of the segment's V rows inside their V ranges (0 unless set): vtkv_seg_value_ptr and the V
+ * pointer tables hand out range base + offset, the K rows start at the base.  The K and the V row of one
+ * token and kv head are read together; in two chunk-aligned ranges they share every address bit below the
+ * chunk size and meet in one memory channel, which costs 5 to 6 % of the streaming rate; 256 bytes apart they
+ * do not.  Mapping counts the offset: the segment keeps used + offset <= mapped, so a range holds
+ * (max bytes - offset) / row bytes rows and reaches a chunk boundary one row early; a caller that maps by
+ * hand (vtkv_seg_expand) and writes through the pointers must count it too.  No counterpart in the reference,
+ * which places both ranges at their base (vmm_allocator.cpp:177-212). */
+int64_t vtkv_seg_value_skew(const vtkv_segment *seg);
+/* Set that offset (a multiple of 256 up to 4096).  Only while the segment holds no rows (VTKV_ESTATE
+ * otherwise); pointers and pointer-table entries fetched before the call are stale after it.  Both segments
+ * of a vtkv_seg_share_prefix must use the same offset. */
+int vtkv_seg_set_value_skew(vtkv_segment *seg, int64_t bytes);
 /* used_size (bytes written per range) get/set; replaces get_used_slot / set_used_size (vmm_allocator.cpp:339-345). */
 int64_t vtkv_seg_get_used(const vtkv_segment *seg);
 int vtkv_seg_set_used(vtkv_segment *seg, int64_t used_bytes);

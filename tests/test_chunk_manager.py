@@ -40,6 +40,23 @@ def test_decode_claims_a_chunk_pair_exactly_when_the_rows_run_out():
     assert grown_at == [25, 25 + 1024]
 
 
+@pytest.mark.parametrize("prompt", [2, 923, 924, 925, 5000])
+def test_value_skew_is_claimed_once_with_the_first_rows(prompt):
+    """With the engine's 256-byte V offset a range needs rows * ROW + 256 bytes: the claim grows one row
+    early at every chunk boundary and always bounds that need."""
+    s = SequenceChunks(ROW, value_skew=256)
+    s.append_tokens(prompt)
+    rows = prompt + PREFILL_SLACK_TOKENS
+    for t in range(2200):
+        need = rows * ROW + 256
+        assert s.reserve_size == -(-need // PHY_GRAN) * PHY_GRAN and s.logical_block_num == 2 * (s.reserve_size // PHY_GRAN)
+        assert s.free_size == s.reserve_size - need
+        s.append_tokens(1)
+        rows += 1
+    with pytest.raises(ValueError):
+        SequenceChunks(ROW, value_skew=PHY_GRAN)
+
+
 def test_conservation_and_watermark_under_random_traffic():
     rng = random.Random(5)
     total = 400

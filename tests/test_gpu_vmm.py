@@ -315,6 +315,92 @@ def test_shared_prefix_maps_whole_chunks_twice_and_copies_the_tail(gpu_pool):
     assert vmm.showFreeBlocks() == free0 and vmm.retiredBlocks() == 0
 
 
+def test_value_rows_set_off_from_the_base_of_their_range(gpu_pool):
+    """A segment whose V rows start 256 bytes into their ranges (so that the K and the V row of a token lie in
+    different memory channels): the V pointer moves, the K pointer does not, mapping counts the offset (a chunk
+    boundary is reached one row early, a range filled to the last byte of a chunk owns the next one), and a
+    shared prefix that ends on a chunk boundary gets a chunk of its own for the V rows' last 256 bytes."""
+    import torch
+
+    from glake_amd import _C
+
+    def read(ptr, n):
+        out = np.empty(n, np.uint8)
+        _C.check(_C.lib().vtkv_memcpy_d2h(out.ctypes.data_as(C.c_void_p), ptr, n))
+        return out
+
+    def write(ptr, data):
+        _C.check(_C.lib().vtkv_memcpy_h2d(ptr, data.ctypes.data_as(C.c_void_p), data.nbytes))
+
+    vmm = gpu_pool
+    vmm.trim()
+    free0 = vmm.showFreeBlocks()
+    row = 8 * 128 * 2
+    rng = np.random.default_rng(11)
+    seg = vmm.KVcacheSegment(1, 4 * CHUNK, 0, False)
+    k0, v0 = seg.getKeyDevicePtr(0), seg.getValueDevicePtr(0)
+    assert seg.value_skew == 0
+    with pytest.raises(_C.VtkvError):
+        seg.set_value_skew(100)                            # not a multiple of 256
+    with pytest.raises(_C.VtkvError):
+        seg.set_value_skew(8192)
+    seg.set_value_skew(256)
+    assert seg.value_skew == 256 and seg.getKeyDevicePtr(0) == k0 and seg.getValueDevicePtr(0) == v0 + 256
+    kt, vt = vmm.KV_cache(1, 0), vmm.KV_cache(1, 0)
+    vmm.copy_kv_cache([kt.kv_cache], [vt.kv_cache], [seg])                # the pointer tables carry the offset too
+    assert int(read(kt.vmm_ptr, 8).view(np.int64)[0]) == k0 and int(read(vt.vmm_ptr, 8).view(np.int64)[0]) == v0 + 256
+    # rows 0..1022 fit the first chunk with the offset, row 1023 does not
+    seg.ensure_mapped(1022 * row)
+    assert seg.actual_size == CHUNK
+    seg.set_used_size(1022 * row)
+    assert vmm.extend_kv_cache_batch(None, None, [0], [row], [seg], [0], row, True) == [1022 * row]
+    assert seg.actual_size == CHUNK
+    assert vmm.extend_kv_cache_batch(None, None, [0], [row], [seg], [0], row, True) == [1023 * row]
+    assert seg.actual_size == 2 * CHUNK and seg.used_size == CHUNK
+    blobs = {}
+    for which, ptr in (("k", seg.getKeyDevicePtr(0)), ("v", seg.getValueDevicePtr(0))):
+        blobs[which] = rng.integers(0, 256, CHUNK, dtype=np.uint8)   # the V rows end 256 bytes into the second chunk
+        write(ptr, blobs[which])
+        assert np.array_equal(read(ptr, CHUNK), blobs[which])
+    with pytest.raises(_C.VtkvError):
+        seg.set_value_skew(0)                              # it holds rows
+    with pytest.raises(_C.VtkvError):
+        seg.set_used_size(4 * CHUNK)                       # the V rows would end beyond the range
+    # a prefix of exactly one chunk: that chunk is shared, the V rows' last 256 bytes are copied
+    dst = vmm.KVcacheSegment(1, 4 * CHUNK, 0, False)
+    with pytest.raises(_C.VtkvError):
+        dst.share_prefix(seg, CHUNK)                       # the two place their V rows differently
+    dst.set_value_skew(256)
+    dst.share_prefix(seg, CHUNK, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert dst.used_size == CHUNK and dst.actual_size == 2 * CHUNK and vmm.sharedBlocks() == 2
+    assert vmm.showFreeBlocks() == free0 - 2 * 2 - 1 * 2
+    for which, ptr in (("k", dst.getKeyDevicePtr(0)), ("v", dst.getValueDevicePtr(0))):
+        assert np.array_equal(read(ptr, CHUNK), blobs[which])
+    # the copied tail is the destination's own
+    mine = rng.integers(0, 256, 256, dtype=np.uint8)
+    write(dst.getValueDevicePtr(0) + CHUNK - 256, mine)
+    assert np.array_equal(read(seg.getValueDevicePtr(0) + CHUNK - 256, 256), blobs["v"][CHUNK - 256:])
+    # a prefix whose V rows end in the chunk behind the one its K rows end in: two chunks of its own
+    seg.ensure_mapped(CHUNK - 128)
+    assert seg.actual_size == 3 * CHUNK
+    more = {}
+    for which, ptr in (("k", seg.getKeyDevicePtr(0)), ("v", seg.getValueDevicePtr(0))):
+        more[which] = rng.integers(0, 256, CHUNK - 128, dtype=np.uint8)
+        write(ptr + CHUNK, more[which])
+    seg.set_used_size(2 * CHUNK - 128)
+    third = vmm.KVcacheSegment(1, 4 * CHUNK, 0, False)
+    third.set_value_skew(256)
+    third.share_prefix(seg, 2 * CHUNK - 128)
+    torch.cuda.synchronize()
+    assert third.actual_size == 3 * CHUNK and third.used_size == 2 * CHUNK - 128
+    for which, ptr in (("k", third.getKeyDevicePtr(0)), ("v", third.getValueDevicePtr(0))):
+        assert np.array_equal(read(ptr, 2 * CHUNK - 128), np.concatenate([blobs[which], more[which]]))
+    for s in (dst, third, seg):
+        s.destroy()
+    assert vmm.showFreeBlocks() == free0 and vmm.sharedBlocks() == 0
+
+
 def test_slots_are_created_and_destroyed_over_and_over(gpu_pool):
     """Churn: sets of slots of one size are created, some of them written and read, and all destroyed,
     hundreds of times.  The address ranges of destroyed slots are handed to the next slots of that size,
