@@ -347,7 +347,7 @@ def main() -> int:
         "dtype": "bf16 (fp8-e4m3 KV)" if fp8 else "bf16", "data": "synthetic",
         "config": {"workload": cfg["name"], "layers": 1, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
                    "mean_ctx": round(float(np.mean(final_lens)), 1), "host_path": args.host_path,
-                   "fused_append": bool(plan.fused) and step is step_plan},
+                   "fused_append": bool(plan.fused) and step is step_plan, "value_skew_bytes": engine.value_skew},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "host_issue_ms_per_step": round(host_dt / K * 1e3, 4),
