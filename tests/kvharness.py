@@ -22,12 +22,16 @@ def bf16_randn(rng, shape):
 class GpuSeqs:
     """`num_slots` sequence slots of one layer, each with a K and a V range."""
 
-    def __init__(self, vmm, num_slots, num_kv_heads, head_size, elem_bytes, max_tokens, layers=1):
+    def __init__(self, vmm, num_slots, num_kv_heads, head_size, elem_bytes, max_tokens, layers=1, value_skew=0):
         self.vmm = vmm
         self.chunk = vmm.chunkBytes()  # CHUNK unless the pool was set up with larger chunks
         self.row_bytes = num_kv_heads * head_size * elem_bytes
-        self.max_bytes = round_up(max_tokens * self.row_bytes, self.chunk)
+        self.value_skew = value_skew  # bytes between the base of a V range and its first row (the engine uses 256)
+        self.max_bytes = round_up(max_tokens * self.row_bytes + value_skew, self.chunk)
         self.segs = [vmm.KVcacheSegment(layers, self.max_bytes, 0, False) for _ in range(num_slots)]
+        if value_skew:
+            for seg in self.segs:
+                seg.set_value_skew(value_skew)
         self.layers = layers
         self.k_tables = [vmm.KVCache(num_slots) for _ in range(layers)]
         self.v_tables = [vmm.KVCache(num_slots) for _ in range(layers)]
@@ -39,7 +43,7 @@ class GpuSeqs:
 
         seg = self.segs[slot]
         nbytes = k_rows.nbytes
-        need = round_up(nbytes, self.chunk) - seg.actual_size
+        need = round_up(nbytes + self.value_skew, self.chunk) - seg.actual_size
         if need > 0:
             seg.expandMultiSegment(need // self.chunk)
         k_rows = np.ascontiguousarray(k_rows)
@@ -54,7 +58,7 @@ class GpuSeqs:
 
         zeros = np.zeros(nbytes, np.uint8)
         for seg in self.segs:
-            need = round_up(nbytes, self.chunk) - seg.actual_size
+            need = round_up(nbytes + self.value_skew, self.chunk) - seg.actual_size
             if need > 0:
                 seg.expandMultiSegment(need // self.chunk)
             for dst in (seg.getKeyDevicePtr(layer), seg.getValueDevicePtr(layer)):

@@ -16,8 +16,9 @@ pytestmark = pytest.mark.gpu
 TOL = 2e-3
 
 
-def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partition_tokens=0, d=128, fp8=False):
-    """seq_lens count the new token."""
+def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partition_tokens=0, d=128, fp8=False,
+             value_skew=0):
+    """seq_lens count the new token; value_skew: bytes between the base of a V range and its first row."""
     import torch
 
     from glake_amd import _custom_ops as ops
@@ -34,7 +35,7 @@ def run_case(vmm, seed, seq_lens, hq, hkv, lens_from="host", alibi=False, partit
     def stored(bits, sc):  # what the cache holds for bf16 source rows
         return O.fp8_encode(O.bf16_to_f32(bits), sc) if fp8 else bits
 
-    gpu = GpuSeqs(vmm, num_slots, hkv, d, eb, max(seq_lens) + 1)
+    gpu = GpuSeqs(vmm, num_slots, hkv, d, eb, max(seq_lens) + 1, value_skew=value_skew)
     k_host, v_host = {}, {}
     for i, t in enumerate(seq_lens):
         s = int(slots[i])
@@ -132,6 +133,17 @@ def test_very_many_short_sequences(gpu_pool, lens_from):
     lens = [int(x) for x in rng.integers(1, 50, 509)] + [900, 1, 17]
     run_case(gpu_pool, 21, lens, 32, 8, lens_from=lens_from)
     run_case(gpu_pool, 22, lens, 16, 8, lens_from=lens_from, alibi=True)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_value_rows_offset_from_their_range_base_around_chunk_ends(gpu_pool, fp8):
+    """The engine's placement (V rows 256 bytes into their range): sequences whose new row is the last one that
+    fits the first chunk with the offset, the first one that does not, and rows on either side of the 2 MiB and
+    4 MiB marks; cache bytes exact, attention within tolerance."""
+    per = (2 << 20) // (8 * 128 * (1 if fp8 else 2))       # rows per chunk
+    lens = [per - 1, per, per + 1, per + 2, 2 * per - 1, 2 * per, 2 * per + 1, 5, 700, 1]
+    run_case(gpu_pool, 31, lens, 32, 8, fp8=fp8, value_skew=256)
+    run_case(gpu_pool, 32, lens, 64, 8, lens_from="device", fp8=fp8, value_skew=256, alibi=True)
 
 
 def test_long_sequence_many_workgroups_per_segment(gpu_pool):

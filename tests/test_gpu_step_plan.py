@@ -12,8 +12,11 @@ from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("kv,fused", [("bf16", True), ("bf16", False), ("fp8", False), ("fp8", True)])
-def test_plan_matches_ops_and_oracle(gpu_pool, kv, fused):
+@pytest.mark.parametrize("kv,fused,skew", [("bf16", True, 0), ("bf16", False, 0), ("fp8", False, 0), ("fp8", True, 0),
+                                           ("bf16", True, 256), ("bf16", False, 256), ("fp8", True, 256)])
+def test_plan_matches_ops_and_oracle(gpu_pool, kv, fused, skew):
+    """skew: bytes between the base of a V range and its first row (0 = the reference's placement, 256 = what
+    the cache engine sets up)."""
     import torch
 
     from glake_amd import _custom_ops as ops, vmm_allocator as vmm
@@ -31,7 +34,7 @@ def test_plan_matches_ops_and_oracle(gpu_pool, kv, fused):
     kv_dtype = "fp8" if fp8 else "auto"
     scale = d ** -0.5
     # two identical sets of sequences: one driven by the plan, one by the separate ops
-    sets = [GpuSeqs(vmm, B, hkv, d, eb, rows_per_chunk + 64) for _ in range(2)]
+    sets = [GpuSeqs(vmm, B, hkv, d, eb, rows_per_chunk + 64, value_skew=skew) for _ in range(2)]
     host_k, host_v = [], []
     for b in range(B):
         kb, vb = bf16_randn(rng, (ctx[b], hkv, d)), bf16_randn(rng, (ctx[b], hkv, d))
