@@ -148,6 +148,8 @@ def main() -> int:
                     help="where the attention's partial results are merged (auto: the library decides per call)")
     ap.add_argument("--value-skew", type=int, default=256,
                     help="bytes between the base of a V range and its first row (0 = the reference's placement)")
+    ap.add_argument("--head-major", default="auto", choices=["auto", "on", "off"],
+                    help="tile order of the decode kernel: (kv head, sequence, rows) or (sequence, kv head, rows)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -167,6 +169,7 @@ def main() -> int:
             args.steps, args.warmup = 20, 3
         return prompt_run(args, cfg)
     _C.check(_C.lib().vtkv_set_fused_merge({"auto": -1, "fused": 1, "separate": 0}[args.merge]))
+    _C.check(_C.lib().vtkv_set_head_major({"auto": -1, "on": 1, "off": 0}[args.head_major]))
     B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
     K, W = args.steps, args.warmup
     torch.cuda.set_device(0)

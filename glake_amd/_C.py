@@ -90,6 +90,7 @@ SIGNATURES = {
     "vtkv_prefill_unit_tokens": (_i, [_i, _i, _i]),
     "vtkv_prefill_attention": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f, _i, _p, _i, _i, _i, _f, _f, _p]),
     "vtkv_set_fused_merge": (_i, [_i]),
+    "vtkv_set_head_major": (_i, [_i]),
     "vtkv_set_kernel_timing": (_i, [_i]),
     "vtkv_attention_kernel_times": (_i, [_p, _p, _i]),
 }

@@ -148,6 +148,34 @@ def test_merge_inside_and_outside_the_kernel(gpu_pool, mode):
         _C.check(lib.vtkv_set_fused_merge(-1))
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+def test_head_major_and_sequence_major_tile_orders(gpu_pool, mode):
+    """The workgroups walk over the batch in (sequence, kv head, rows) or in (kv head, sequence, rows) order;
+    the library picks the second where it lines the kv heads up with the XCDs.  Both forced here (separate
+    merge kernel, which the head-major order needs): short sequences, several per workgroup; long ones over
+    many workgroups; 8, 3, 1 and 16 kv heads; ALiBi; the fused append."""
+    from glake_amd import _C
+
+    import test_gpu_append_attention as A
+
+    lib = _C.lib()
+    _C.check(lib.vtkv_set_head_major(mode))
+    _C.check(lib.vtkv_set_fused_merge(0))
+    try:
+        run_case(gpu_pool, 51, [1, 15, 16, 17, 64, 65, 257, 1025], 32, 8)
+        run_case(gpu_pool, 52, [30000, 3, 9000, 700], 32, 8)
+        run_case(gpu_pool, 53, [700, 64, 1500, 2049, 1, 33], 12, 3, alibi=True)
+        run_case(gpu_pool, 54, [5000, 17, 900], 8, 1)
+        run_case(gpu_pool, 55, [333, 4000, 16, 2], 32, 16)
+        rng = np.random.default_rng(1001)
+        run_case(gpu_pool, 1001, rng.integers(512, 4097, 64).tolist(), 32, 8)
+        A.run_case(gpu_pool, 56, [1, 2, 17, 1025, 1026, 40000, 300], 32, 8, lens_from="device")
+        A.run_case(gpu_pool, 57, rng.integers(1, 3000, 48).tolist(), 64, 8)
+    finally:
+        _C.check(lib.vtkv_set_head_major(-1))
+        _C.check(lib.vtkv_set_fused_merge(-1))
+
+
 @pytest.mark.parametrize("mode", [-1, 0, 1])
 def test_very_many_short_sequences_pair_their_kv_heads(gpu_pool, mode):
     """From 4096 (sequence, kv head) segments on the library runs the variants in which a workgroup streams a
