@@ -615,8 +615,8 @@ __global__ void __launch_bounds__(kThreads)
           store_out(kv_head, head, d, o_norm * p.v_scale);
           continue;
         }
-        // (head-major order, one kv head per segment only: kv head * B + sequence is what grows along it)
-        const int64_t seg_rank = head_major ? (int64_t)kv_head * B + b : (int64_t)b * Hkv + kv_head;
+        // (head-major order: (segment's kv heads, sequence, head inside the segment) is what grows along it)
+        const int64_t seg_rank = head_major ? ((int64_t)kvg * B + b) * kHps + sd : (int64_t)b * Hkv + kv_head;
         const int64_t pidx = ((int64_t)kHps * wg + seg_rank) * G + head;
         if (p.fused_merge) {
           store_device_coherent(&p.part_out[pidx * kD + d], o_norm);
@@ -751,9 +751,9 @@ __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
   const int hps = p.heads_per_seg, Hseg = Hkv / hps;
   const int total_tiles = p.cum_tiles[p.num_seqs] * Hseg;
   const int span = span_of(p, total_tiles);
-  const int first = p.head_major ? kvh * p.cum_tiles[p.num_seqs] + cum_b : cum_b * Hseg + (kvh / hps) * nt;
+  const int first = p.head_major ? (kvh / hps) * p.cum_tiles[p.num_seqs] + cum_b : cum_b * Hseg + (kvh / hps) * nt;
   const int w0 = first / span, w1 = (first + nt - 1) / span;
-  const int64_t seg = p.head_major ? (int64_t)kvh * p.num_seqs + b : (int64_t)b * Hkv + kvh;
+  const int64_t seg = p.head_major ? ((int64_t)(kvh / hps) * p.num_seqs + b) * hps + kvh % hps : (int64_t)b * Hkv + kvh;
   for (int h0 = 0; h0 < G; h0 += 4) {
     float m[4], wsum[4], o[4];
 #pragma unroll
@@ -975,10 +975,13 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.span_tiles = partition_tokens > 0 ? partition_tokens / kTile : 0;
   p.grid = (int)grid;
   p.xcd_spans = !p.fused_merge && partition_tokens == 0 && grid % 8 == 0 ? (int)(grid / 8) : 0;
-  // Head-major tile order (see the kernel) where it lines the kv heads up with the XCDs: one kv head per
-  // segment, the separate merge kernel, a contiguous eighth of the order per XCD and kv heads in eights.
-  p.head_major = seg_heads == 1 && !p.fused_merge && partition_tokens == 0 &&
-                 (g_head_major == 1 || (g_head_major < 0 && p.xcd_spans > 0 && num_kv_heads % 8 == 0));
+  // Head-major tile order (see the kernel) where it lines the kv heads up with the XCDs: the separate merge
+  // kernel, a contiguous eighth of the order per XCD, and eight XCDs per whole number of segments of a
+  // sequence or the other way round (8 kv heads: one per XCD; 4 pairs of fp8 heads: a pair per two XCDs).
+  const int segs_per_seq = num_kv_heads / seg_heads;
+  p.head_major = !p.fused_merge && partition_tokens == 0 &&
+                 (g_head_major == 1 ||
+                  (g_head_major < 0 && p.xcd_spans > 0 && (segs_per_seq % 8 == 0 || 8 % segs_per_seq == 0)));
   // x = code * scale: the K scale multiplies every logit, the V scale the whole output
   p.scale_log2 = scale * kLog2e * (fp8 ? k_scale : 1.f);
   p.v_scale = fp8 ? v_scale : 1.f;

@@ -330,9 +330,9 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
  * For A/B measurements; results agree up to fp32 summation order.  No counterpart in the reference. */
 int vtkv_set_fused_merge(int on);
 /* Order in which the decode kernel's workgroups walk over the batch: 1 = (kv head, sequence, rows) wherever
- * the kernel supports it (one kv head per segment, separate merge kernel, no fixed partitions), 0 =
- * (sequence, kv head, rows) always, -1 (the default) = head-major where it lines the kv heads up with the
- * eight XCDs (kv heads in multiples of eight and one contiguous eighth of the order per XCD).
+ * the kernel supports it (separate merge kernel, no fixed partitions), 0 = (sequence, kv head, rows) always,
+ * -1 (the default) = head-major where it lines the kv heads up with the eight XCDs (one contiguous eighth of
+ * the order per XCD, and eight a multiple or a divisor of the kv heads, or pairs of fp8 kv heads, per sequence).
  * For A/B measurements; results agree up to fp32 summation order.  No counterpart in the reference. */
 int vtkv_set_head_major(int on);
 

@@ -153,7 +153,7 @@ def test_head_major_and_sequence_major_tile_orders(gpu_pool, mode):
     """The workgroups walk over the batch in (sequence, kv head, rows) or in (kv head, sequence, rows) order;
     the library picks the second where it lines the kv heads up with the XCDs.  Both forced here (separate
     merge kernel, which the head-major order needs): short sequences, several per workgroup; long ones over
-    many workgroups; 8, 3, 1 and 16 kv heads; ALiBi; the fused append."""
+    many workgroups; 8, 3, 1 and 16 kv heads; ALiBi; the fused append; fp8 rows (pairs of kv heads)."""
     from glake_amd import _C
 
     import test_gpu_append_attention as A
@@ -171,6 +171,9 @@ def test_head_major_and_sequence_major_tile_orders(gpu_pool, mode):
         run_case(gpu_pool, 1001, rng.integers(512, 4097, 64).tolist(), 32, 8)
         A.run_case(gpu_pool, 56, [1, 2, 17, 1025, 1026, 40000, 300], 32, 8, lens_from="device")
         A.run_case(gpu_pool, 57, rng.integers(1, 3000, 48).tolist(), 64, 8)
+        # fp8 rows: a segment is a pair of kv heads
+        A.run_case(gpu_pool, 58, [1, 2, 17, 2049, 2050, 30000, 300], 64, 8, fp8=True)
+        A.run_case(gpu_pool, 59, rng.integers(1, 5000, 40).tolist(), 32, 4, lens_from="device", fp8=True, alibi=True)
     finally:
         _C.check(lib.vtkv_set_head_major(-1))
         _C.check(lib.vtkv_set_fused_merge(-1))
