@@ -1,7 +1,7 @@
 """A seeded random sweep of decode and prompt attention against the oracle: head counts (GQA groups 1 to
 16, odd head counts), batch sizes, length mixes (all short, mixed, one very long sequence among short
-ones), fixed partitions and stream-K spans, ALiBi, fp8, and the three merge modes.  Every case builds its
-own sequence slots and destroys them again.  Same tolerances as the dedicated tests; with ALiBi the check
+ones), fixed partitions and stream-K spans, ALiBi, fp8, and the three merge modes and tile orders.  Every case
+builds its own sequence slots and destroys them again.  Same tolerances as the dedicated tests; with ALiBi the check
 on bf16 steps is left out (slopes drawn from N(0,1) times positions in the thousands give biases whose
 fp32 rounding alone exceeds a bf16 step of a small output, inside the tolerance on the fp32 values)."""
 import numpy as np
@@ -43,9 +43,11 @@ def test_random_sweep(gpu_pool, seed):
             alibi = bool(rng.integers(4) == 0)
             merge = int(rng.integers(-1, 2))
             sub = int(rng.integers(1 << 30))
+            order = (sub >> 3) % 3 - 1  # tile order: -1 the library's choice, 0 sequence-major, 1 head-major where possible
             _C.check(lib.vtkv_set_fused_merge(merge))
-            print(f"decode case {case}: seed {sub} heads {hq}/{hkv} lens {lens} partition {pt} alibi {alibi} merge {merge}",
-                  flush=True)
+            _C.check(lib.vtkv_set_head_major(order))
+            print(f"decode case {case}: seed {sub} heads {hq}/{hkv} lens {lens} partition {pt} alibi {alibi} merge {merge} "
+                  f"order {order}", flush=True)
             A.run_case(gpu_pool, sub, lens, hq, hkv, partition_tokens=pt, alibi=alibi, bf16_step_check=not alibi)
             if rng.integers(3) == 0:
                 seq = [int(x) for x in rng.integers(1, 600, int(rng.integers(1, 6)))]
@@ -55,6 +57,7 @@ def test_random_sweep(gpu_pool, seed):
                 P.run_case(gpu_pool, sub, ql, seq, hq, hkv, alibi=al, fp8=fp8, tol=3e-2 if fp8 else 2e-3)
     finally:
         _C.check(lib.vtkv_set_fused_merge(-1))
+        _C.check(lib.vtkv_set_head_major(-1))
 
 
 @pytest.mark.parametrize("seed", [404, 505])
@@ -81,9 +84,12 @@ def test_random_sweep_fp8_decode(gpu_pool, seed):
             alibi = bool(rng.integers(4) == 0)
             merge = int(rng.integers(-1, 2))
             sub = int(rng.integers(1 << 30))
+            order = (sub >> 3) % 3 - 1
             _C.check(lib.vtkv_set_fused_merge(merge))
+            _C.check(lib.vtkv_set_head_major(order))
             print(f"fp8 decode case {case}: seed {sub} heads {hq}/{hkv} lens {lens} partition {pt} alibi {alibi} "
-                  f"merge {merge}", flush=True)
+                  f"merge {merge} order {order}", flush=True)
             F.run_case(gpu_pool, sub, lens, hq, hkv, alibi=alibi, partition_tokens=pt)
     finally:
         _C.check(lib.vtkv_set_fused_merge(-1))
+        _C.check(lib.vtkv_set_head_major(-1))
