@@ -160,7 +160,7 @@ __global__ void __launch_bounds__(kThreads)
   __shared__ int s_wave_tot[kWaves];
   // pieces of shared (sequence, kv head) segments this workgroup has written: segment, first and last
   // workgroup of the segment, and whether this workgroup delivered the last piece
-  __shared__ int s_pend[8][4];
+  __shared__ int s_pend[8][5];
   __shared__ int s_npend;
 
   const int lane = threadIdx.x & 63;
@@ -229,7 +229,8 @@ __global__ void __launch_bounds__(kThreads)
   // the gain grows with the run of consecutive spans per XCD: 16, 32, 64 spans give 150, 146, 144 us;
   // config 2: 111.4 -> 110.1 us; each XCD has its own L2 and address translation, which of the two it is
   // has not been established); many short sequences with the merge inside this kernel lose 1.7 %
-  // (config 5), so the host asks for it only together with the separate merge kernel.
+  // (config 5) unless the tile order is head-major as well (below), so the host asks for it together with the
+  // separate merge kernel or with that order.
   const int wg = p.xcd_spans > 0 ? (int)(blockIdx.x % 8) * p.xcd_spans + (int)(blockIdx.x / 8) : (int)blockIdx.x;
   int g_cur = wg * span;
   if (g_cur >= total_tiles) return;
@@ -640,6 +641,7 @@ __global__ void __launch_bounds__(kThreads)
       int k = s_npend;
       for (int sd = 0; sd < kHps; ++sd, ++k) {
         s_pend[k][0] = b * Hkv + kvg * kHps + sd;
+        s_pend[k][4] = head_major ? (kvg * B + b) * kHps + sd : s_pend[k][0];  // its place among the partial slots
         s_pend[k][1] = w0;
         s_pend[k][2] = w1;
       }
@@ -696,7 +698,7 @@ __global__ void __launch_bounds__(kThreads)
       const int j = idx / per_seg;
       if (!s_pend[j][3]) continue;
       const int head = (idx - j * per_seg) / kD, d = idx % kD;
-      const int64_t seg = s_pend[j][0];
+      const int64_t seg = s_pend[j][0], seg_rank = s_pend[j][4];
       const int w0 = s_pend[j][1], w1 = s_pend[j][2];
       // four pieces at a time, all their loads in flight together; running (max, sum, out) across batches
       float m = -INFINITY, wsum = 0.f, o = 0.f;
@@ -704,7 +706,7 @@ __global__ void __launch_bounds__(kThreads)
         float pm[4], ps[4], po[4];
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-          const int64_t pidx = ((int64_t)kHps * min(wb + jj, w1) + seg) * G + head;
+          const int64_t pidx = ((int64_t)kHps * min(wb + jj, w1) + seg_rank) * G + head;
           pm[jj] = load_device_coherent(&p.part_max[pidx]);
           ps[jj] = load_device_coherent(&p.part_sum[pidx]);
           po[jj] = load_device_coherent(&p.part_out[pidx * kD + d]);
@@ -958,8 +960,16 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   // contiguous part of the tile order): 1024 segments 188 against 180 us (group 4) and 196 against 192 us
   // (group 8); 1280 segments 212 / 209 and 219 / 221; 1536 segments 206 / 205 and 217 / 222; 2048 segments
   // 201.5 / 212 and 216 / 231.  Hence inside from two and a half segments per workgroup on.
-  p.fused_merge = g_fused_merge == 1 ||
-                  (g_fused_merge < 0 && 2 * (int64_t)num_seqs * (num_kv_heads / seg_heads) >= 5 * grid);
+  // Where the head-major tile order applies (below) the merge inside gains more from it than the separate
+  // form (torch allocations, 300 000 rows over 64..1024 ragged sequences, group 4 / group 8, inside against
+  // separate, both head-major: 1 segment per workgroup 173 / 174 and 179 / 178 us; 2 segments 190 / 194 and
+  // 201 / 203; 4 segments 197 / 205 and 210 / 219; 16 segments 223 / 243 and 247 / 271): inside from two
+  // segments per workgroup on.
+  const int segs_per_seq = num_kv_heads / seg_heads;
+  const int64_t segs = (int64_t)num_seqs * segs_per_seq;
+  const bool hm_fits = partition_tokens == 0 && grid % 8 == 0 && (segs_per_seq % 8 == 0 || 8 % segs_per_seq == 0);
+  const bool hm_auto = g_head_major != 0 && hm_fits;  // the head-major order is open to this call
+  p.fused_merge = g_fused_merge == 1 || (g_fused_merge < 0 && (hm_auto ? segs >= 2 * grid : 2 * segs >= 5 * grid));
   p.heads_per_seg = seg_heads;
   p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
   p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);
@@ -974,14 +984,14 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.group = group;
   p.span_tiles = partition_tokens > 0 ? partition_tokens / kTile : 0;
   p.grid = (int)grid;
-  p.xcd_spans = !p.fused_merge && partition_tokens == 0 && grid % 8 == 0 ? (int)(grid / 8) : 0;
-  // Head-major tile order (see the kernel) where it lines the kv heads up with the XCDs: the separate merge
-  // kernel, a contiguous eighth of the order per XCD, and eight XCDs per whole number of segments of a
-  // sequence or the other way round (8 kv heads: one per XCD; 4 pairs of fp8 heads: a pair per two XCDs).
-  const int segs_per_seq = num_kv_heads / seg_heads;
-  p.head_major = !p.fused_merge && partition_tokens == 0 &&
-                 (g_head_major == 1 ||
-                  (g_head_major < 0 && p.xcd_spans > 0 && (segs_per_seq % 8 == 0 || 8 % segs_per_seq == 0)));
+  // Head-major tile order (see the kernel) where it lines the kv heads up with the XCDs: a contiguous eighth
+  // of the order per XCD, and eight XCDs per whole number of segments of a sequence or the other way round
+  // (8 kv heads: one per XCD; 4 pairs of kv heads: a pair per two XCDs).  Without it the per-XCD span order
+  // only pays with the separate merge kernel (config 5 with the merge inside lost 1.7 %).
+  p.xcd_spans = partition_tokens == 0 && grid % 8 == 0 && (!p.fused_merge || hm_auto || g_head_major == 1)
+                    ? (int)(grid / 8) : 0;
+  p.head_major = partition_tokens == 0 && (g_head_major == 1 ? (!p.fused_merge || p.xcd_spans > 0)
+                                                              : (hm_auto && p.xcd_spans > 0));
   // x = code * scale: the K scale multiplies every logit, the V scale the whole output
   p.scale_log2 = scale * kLog2e * (fp8 ? k_scale : 1.f);
   p.v_scale = fp8 ? v_scale : 1.f;

@@ -325,12 +325,12 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
 
 /* Where the partial results of the workgroups that share a (sequence, kv head) are merged: 1 = inside the
  * attention kernel, by whichever of them finishes last; 0 = by a second kernel; -1 (the default) = inside
- * when the batch has at least two and a half (sequence, kv head) pairs per workgroup, so that most need no
- * merge.
+ * when the batch has at least two (sequence, kv head) pairs per workgroup (two and a half where the
+ * head-major tile order does not apply), so that most need no merge.
  * For A/B measurements; results agree up to fp32 summation order.  No counterpart in the reference. */
 int vtkv_set_fused_merge(int on);
 /* Order in which the decode kernel's workgroups walk over the batch: 1 = (kv head, sequence, rows) wherever
- * the kernel supports it (separate merge kernel, no fixed partitions), 0 = (sequence, kv head, rows) always,
+ * the kernel supports it (no fixed partitions), 0 = (sequence, kv head, rows) always,
  * -1 (the default) = head-major where it lines the kv heads up with the eight XCDs (one contiguous eighth of
  * the order per XCD, and eight a multiple or a divisor of the kv heads, or pairs of fp8 kv heads, per sequence).
  * For A/B measurements; results agree up to fp32 summation order.  No counterpart in the reference. */

@@ -148,11 +148,11 @@ def test_merge_inside_and_outside_the_kernel(gpu_pool, mode):
         _C.check(lib.vtkv_set_fused_merge(-1))
 
 
-@pytest.mark.parametrize("mode", [0, 1])
-def test_head_major_and_sequence_major_tile_orders(gpu_pool, mode):
+@pytest.mark.parametrize("mode,merge", [(0, 0), (1, 0), (1, 1)])
+def test_head_major_and_sequence_major_tile_orders(gpu_pool, mode, merge):
     """The workgroups walk over the batch in (sequence, kv head, rows) or in (kv head, sequence, rows) order;
-    the library picks the second where it lines the kv heads up with the XCDs.  Both forced here (separate
-    merge kernel, which the head-major order needs): short sequences, several per workgroup; long ones over
+    the library picks the second where it lines the kv heads up with the XCDs.  Both forced here, the head-major
+    one with the separate merge kernel and with the merge inside the kernel: short sequences, several per workgroup; long ones over
     many workgroups; 8, 3, 1 and 16 kv heads; ALiBi; the fused append; fp8 rows (pairs of kv heads)."""
     from glake_amd import _C
 
@@ -160,7 +160,7 @@ def test_head_major_and_sequence_major_tile_orders(gpu_pool, mode):
 
     lib = _C.lib()
     _C.check(lib.vtkv_set_head_major(mode))
-    _C.check(lib.vtkv_set_fused_merge(0))
+    _C.check(lib.vtkv_set_fused_merge(merge))
     try:
         run_case(gpu_pool, 51, [1, 15, 16, 17, 64, 65, 257, 1025], 32, 8)
         run_case(gpu_pool, 52, [30000, 3, 9000, 700], 32, 8)
