@@ -49,7 +49,11 @@
 
 #include "vtkv_common.h"
 #ifndef VTKV_ATTN_STAGES
-#define VTKV_ATTN_STAGES 2
+// Register tiles per wave of the bf16 variants.  One (the next tile's K loads are issued as soon as the K
+// registers are free, its V loads likewise) against two: config 2 and 3 the same within 0.3 %, config 5
+// 1 to 1.5 % faster per step (0.2083 against 0.2115 ms); three are 0.5 % slower than two.  More loads in
+// flight do not help a kernel that already saturates the memory system.
+#define VTKV_ATTN_STAGES 1
 #endif
 #ifndef VTKV_ATTN_BF16_WAVES
 #define VTKV_ATTN_BF16_WAVES 2  // waves per SIMD of the bf16 variants (3 spills)
