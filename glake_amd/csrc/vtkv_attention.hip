@@ -748,8 +748,13 @@ __global__ void __launch_bounds__(kThreads)
 // pieces four at a time, so that up to 48 loads of a thread are in flight together: the kernel is a chain
 // of three or four memory round trips (tile counts, then statistics and partial outputs of a batch), and
 // with one small workgroup per query head it was that chain times many more workgroups.
-__global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
-  const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+// GROUPS > 1 (segments of many pieces: a few long sequences): GROUPS sets of kD threads take every GROUPS-th
+// batch of four pieces and their running (max, sum, out) are combined through LDS at the end, so the chain
+// of dependent round trips is GROUPS times shorter (config 3: 37 pieces per segment).
+template <int GROUPS>
+__global__ void __launch_bounds__(kD * GROUPS) decode_attn_reduce_kernel(AttnParams p) {
+  const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x % kD, grp = threadIdx.x / kD;
+  __shared__ float sm_red[GROUPS > 1 ? 3 * GROUPS * 4 * kD : 1];
   const int G = p.group, Hkv = p.num_kv_heads;
   const int cum_b = p.cum_tiles[b];
   const int nt = p.cum_tiles[b + 1] - cum_b;
@@ -764,7 +769,7 @@ __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
     float m[4], wsum[4], o[4];
 #pragma unroll
     for (int hh = 0; hh < 4; ++hh) m[hh] = -INFINITY, wsum[hh] = 0.f, o[hh] = 0.f;
-    for (int wb = w0; wb <= w1; wb += 4) {
+    for (int wb = w0 + 4 * grp; wb <= w1; wb += 4 * GROUPS) {
       float pm[4][4], ps[4][4], po[4][4];
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj)
@@ -794,6 +799,31 @@ __global__ void __launch_bounds__(kD) decode_attn_reduce_kernel(AttnParams p) {
         m[hh] = m_new;
       }
     }
+    if constexpr (GROUPS > 1) {
+      if (h0 > 0) __syncthreads();  // the previous heads' values have been read
+#pragma unroll
+      for (int hh = 0; hh < 4; ++hh) {
+        float *at = sm_red + ((grp * 4 + hh) * kD + d) * 3;
+        at[0] = m[hh], at[1] = wsum[hh], at[2] = o[hh];
+      }
+      __syncthreads();
+      if (grp == 0) {
+#pragma unroll
+        for (int hh = 0; hh < 4; ++hh) {
+          float mm = m[hh];  // finite: group 0 always has the segment's first piece
+          for (int gg = 1; gg < GROUPS; ++gg) mm = fmaxf(mm, sm_red[((gg * 4 + hh) * kD + d) * 3]);
+          float ws = 0.f, oo = 0.f;
+          for (int gg = 0; gg < GROUPS; ++gg) {
+            const float *at = sm_red + ((gg * 4 + hh) * kD + d) * 3;
+            const float f = __builtin_amdgcn_exp2f(at[0] - mm);  // 0 for a group that saw no piece
+            ws += at[1] * f;
+            oo += at[2] * f;
+          }
+          wsum[hh] = ws, o[hh] = oo;
+        }
+      }
+    }
+    if (grp != 0) continue;
 #pragma unroll
     for (int hh = 0; hh < 4; ++hh) {
       if (h0 + hh >= G) break;
@@ -1023,8 +1053,13 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, p, il);
   if (timed) VTKV_HIP(hipEventRecord(ev[1], st));
-  if (!p.fused_merge)
-    hipLaunchKernelGGL(decode_attn_reduce_kernel, dim3(num_kv_heads, num_seqs), dim3(kD), 0, st, p);
+  if (!p.fused_merge) {
+    // segments of at least four pieces on average: four sets of threads share a segment's pieces
+    if (4 * segs <= grid)
+      hipLaunchKernelGGL(decode_attn_reduce_kernel<4>, dim3(num_kv_heads, num_seqs), dim3(4 * kD), 0, st, p);
+    else
+      hipLaunchKernelGGL(decode_attn_reduce_kernel<1>, dim3(num_kv_heads, num_seqs), dim3(kD), 0, st, p);
+  }
   if (timed) {
     VTKV_HIP(hipEventRecord(ev[2], st));
     ++g_timer.calls;
