@@ -751,9 +751,13 @@ __global__ void __launch_bounds__(kThreads)
 // GROUPS > 1 (segments of many pieces: a few long sequences): GROUPS sets of kD threads take every GROUPS-th
 // batch of four pieces and their running (max, sum, out) are combined through LDS at the end, so the chain
 // of dependent round trips is GROUPS times shorter (config 3: 37 pieces per segment).
-template <int GROUPS>
-__global__ void __launch_bounds__(kD * GROUPS) decode_attn_reduce_kernel(AttnParams p) {
-  const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x % kD, grp = threadIdx.x / kD;
+// HSETS > 1 (only with GROUPS == 1, which has no barrier): HSETS sets of kD threads take the group's heads
+// four at a time in turn, so a group of eight heads is merged in one pass instead of two.
+template <int GROUPS, int HSETS>
+__global__ void __launch_bounds__(kD * GROUPS * HSETS) decode_attn_reduce_kernel(AttnParams p) {
+  static_assert(GROUPS == 1 || HSETS == 1, "head sets only without piece groups");
+  const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x % kD;
+  const int grp = GROUPS > 1 ? threadIdx.x / kD : 0, hset = HSETS > 1 ? threadIdx.x / kD : 0;
   __shared__ float sm_red[GROUPS > 1 ? 3 * GROUPS * 4 * kD : 1];
   const int G = p.group, Hkv = p.num_kv_heads;
   const int cum_b = p.cum_tiles[b];
@@ -765,7 +769,7 @@ __global__ void __launch_bounds__(kD * GROUPS) decode_attn_reduce_kernel(AttnPar
   const int first = p.head_major ? (kvh / hps) * p.cum_tiles[p.num_seqs] + cum_b : cum_b * Hseg + (kvh / hps) * nt;
   const int w0 = first / span, w1 = (first + nt - 1) / span;
   const int64_t seg = p.head_major ? ((int64_t)(kvh / hps) * p.num_seqs + b) * hps + kvh % hps : (int64_t)b * Hkv + kvh;
-  for (int h0 = 0; h0 < G; h0 += 4) {
+  for (int h0 = 4 * hset; h0 < G; h0 += 4 * HSETS) {
     float m[4], wsum[4], o[4];
 #pragma unroll
     for (int hh = 0; hh < 4; ++hh) m[hh] = -INFINITY, wsum[hh] = 0.f, o[hh] = 0.f;
@@ -1056,9 +1060,11 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   if (!p.fused_merge) {
     // segments of at least four pieces on average: four sets of threads share a segment's pieces
     if (4 * segs <= grid)
-      hipLaunchKernelGGL(decode_attn_reduce_kernel<4>, dim3(num_kv_heads, num_seqs), dim3(4 * kD), 0, st, p);
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<4, 1>), dim3(num_kv_heads, num_seqs), dim3(4 * kD), 0, st, p);
+    else if (group > 4)
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 2>), dim3(num_kv_heads, num_seqs), dim3(2 * kD), 0, st, p);
     else
-      hipLaunchKernelGGL(decode_attn_reduce_kernel<1>, dim3(num_kv_heads, num_seqs), dim3(kD), 0, st, p);
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 1>), dim3(num_kv_heads, num_seqs), dim3(kD), 0, st, p);
   }
   if (timed) {
     VTKV_HIP(hipEventRecord(ev[2], st));
