@@ -7,7 +7,8 @@
 // and spend as little time as possible outside the streaming loop:
 //
 //  * work is counted in tiles of 16 rows of one kv head.  All tiles of the batch form one sequence
-//    ordered (sequence, kv head, tile); it is cut into gridDim.x equal contiguous spans, one per
+//    ordered (sequence, kv head, tile), or (kv head, sequence, tile) where that lines the kv heads up with
+//    the XCDs; it is cut into gridDim.x equal contiguous spans, one per
 //    workgroup, whatever the sequence lengths are ("stream-K" split).  Every CU therefore gets the
 //    same number of bytes, a workgroup streams a long contiguous run of rows, and the fixed cost of
 //    starting and finishing a (sequence, kv head) segment is paid once or twice per workgroup instead
