@@ -29,10 +29,24 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes moved per launch of the dominant kernel relative to its algorithmic bytes, measured with
 # rocprofv3 (FETCH_SIZE and WRITE_SIZE in separate runs, each scaled by what the counter reads for the
 # calibration copy of known size that this script runs before timing).  Counters cannot be read from
-# inside this process, so the measured ratio is kept here with the summary it comes from.
-MEASURED_TRAFFIC = {
-    "c2": (1.003, "profiles/decode_attn_stream_kernel_c2_llama3_8b_decode.md"),
-}
+# inside this process, so the measured ratios are kept in a small table beside the profile summaries.
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_decode_attn_stream_kernel.txt")
+
+
+def measured_traffic(config: str):
+    """(traffic / algorithmic bytes, MFMA-busy fraction or None, source) for `config`, or (None, None, None)."""
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            for line in f:
+                cols = line.split()
+                if len(cols) >= 6 and cols[0] == config:
+                    fetch, write, algo = float(cols[1]), float(cols[2]), float(cols[3])
+                    mfma = None if cols[4] == "-" else float(cols[4])
+                    return (fetch + write) / algo, mfma, cols[5]
+    except OSError:
+        pass
+    return None, None, None
+
 
 CONFIGS = {
     # BASELINE.json configs[1]: Llama-3-8B-shaped single-layer decode, bf16
@@ -140,8 +154,14 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--partition-tokens", type=int, default=0)
-    ap.add_argument("--host-path", default="plan", choices=["plan", "ops"],
-                    help="plan: DecodeStepPlan (arguments prepared once); ops: the separate reference-style op calls")
+    ap.add_argument("--host-path", default="plan", choices=["plan", "ops", "backend"],
+                    help="plan: DecodeStepPlan (arguments prepared once); ops: the separate reference-style op calls; "
+                         "backend: the reference's own call sequence, one prepare_step then --layers x "
+                         "VTensorImpl.forward per step")
+    ap.add_argument("--layers", type=int, default=32, help="layers of a step with --host-path backend")
+    ap.add_argument("--repeats", type=int, default=0,
+                    help="timed regions of exactly --steps steps each, synchronised on both sides; the median one is "
+                         "reported (0 = 11 for regions of up to 50 steps, else 3)")
     ap.add_argument("--unfused", action="store_true",
                     help="plan path: separate reshape_and_cache and attention launches instead of the fused one")
     ap.add_argument("--merge", default="auto", choices=["auto", "fused", "separate"],
@@ -172,21 +192,25 @@ def main() -> int:
     _C.check(_C.lib().vtkv_set_head_major({"auto": -1, "on": 1, "off": 0}[args.head_major]))
     B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
     K, W = args.steps, args.warmup
+    R = args.repeats if args.repeats > 0 else (11 if K <= 50 else 3)
+    backend_path = args.host_path == "backend"
+    L = args.layers if backend_path else 1
     torch.cuda.set_device(0)
     dev = torch.device("cuda", 0)
     gen = torch.Generator().manual_seed(cfg["seed"])
     ctx0 = torch.randint(cfg["lo"], cfg["hi"] + 1, (B,), generator=gen).tolist()
-    total_steps = 2 * (K + W) + 4  # timed pass + kernel-timing pass, each with warm-up
+    event_steps = max(1, min(K, 1024 // L))          # the library keeps the events of 1024 attention calls
+    total_steps = (W + R * K) + (W + event_steps) + 4  # timed regions + kernel-timing pass, each with warm-up
     fp8 = cfg["kv"] == "fp8"
     eb = 1 if fp8 else 2            # bytes per KV element
     kv_dtype = "fp8" if fp8 else "auto"
     row = Hkv * D * eb
     max_tokens = max(ctx0) + total_steps + 1
     chunks_per_range = (max_tokens * row + args.value_skew + (2 << 20) - 1) // (2 << 20)
-    vmm.init_physical_handle(2 * B * chunks_per_range + 16, 0)
-    engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.uint8 if fp8 else torch.bfloat16,
-                         max_num_seqs=B,
-                         max_num_batched_tokens=max_tokens, swap_space_bytes=1 << 30, value_skew=args.value_skew)
+    vmm.init_physical_handle(2 * L * B * chunks_per_range + 16, 0)
+    engine = CacheEngine(num_layers=L, num_kv_heads=Hkv, head_size=D, dtype=torch.uint8 if fp8 else torch.bfloat16,
+                         max_num_seqs=B, max_num_batched_tokens=max_tokens,
+                         swap_space_bytes=0 if backend_path else 1 << 30, value_skew=args.value_skew)
     segs = engine.vmm_kvcache_segment
 
     # ---- resident synthetic KV: N(0,1) -> bf16, written straight into the mapped ranges
@@ -196,14 +220,15 @@ def main() -> int:
     for b in range(B):
         nbytes = ctx0[b] * row
         segs[b].ensure_mapped(nbytes)  # counts the V offset
-        for base in (segs[b].getKeyDevicePtr(0), segs[b].getValueDevicePtr(0)):
-            t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
-            if fp8:
-                codes = torch.empty(t.shape, dtype=torch.uint8, device=dev)
-                ops.convert_fp8(codes, t, k_scale)
-                t = codes
-            ops.swap_ranges([t.data_ptr()], [base], [nbytes], "d2d")
-            torch.cuda.synchronize()
+        for l in range(L):
+            for base in (segs[b].getKeyDevicePtr(l), segs[b].getValueDevicePtr(l)):
+                t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+                if fp8:
+                    codes = torch.empty(t.shape, dtype=torch.uint8, device=dev)
+                    ops.convert_fp8(codes, t, k_scale)
+                    t = codes
+                ops.swap_ranges([t.data_ptr()], [base], [nbytes], "d2d")
+                torch.cuda.synchronize()
         segs[b].set_used_size(nbytes)
     q = torch.randn(B, Hq * D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
     new_k = torch.randn(B, Hkv * D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -234,7 +259,7 @@ def main() -> int:
     zeros = [0] * B
     tok_bytes = [kv_size] * B
 
-    from glake_amd.worker.step import DecodeStepPlan
+    from glake_amd.worker.step import DecodeStepPlan, prepare_step
     plan = DecodeStepPlan(segs, slot_ids, engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hq, Hkv, D, scale,
                           kv_cache_dtype=kv_dtype, k_scale=k_scale, v_scale=v_scale, device=dev,
                           fused=not args.unfused)
@@ -263,7 +288,34 @@ def main() -> int:
         state["step"] = i + 1
         return sum(lens)
 
-    if args.host_path == "plan" and args.partition_tokens == 0:
+    # The reference's own call sequence (llama.py:307-351): per step the metadata the model runner builds
+    # (model_runner.py:595-622, with its host-to-device uploads), one prologue, then every layer's forward.
+    from glake_amd.attention.backends.vtensor import VTensorBackend
+    impl = VTensorBackend.get_impl_cls()(Hq, D, scale, Hkv, None, None, kv_dtype)
+    impl.fuse_decode_append = not args.unfused
+    no_extend = [-1] * B
+
+    def step_backend() -> int:
+        lens = state["lens"] = [n + 1 for n in state["lens"]]
+        max_len = max(lens)
+        meta = VTensorBackend.make_metadata(
+            num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B, slot_mapping=slot_t, seq_lens=None,
+            seq_lens_tensor=torch.tensor(lens, dtype=torch.int32, device=dev), max_query_len=None,
+            max_prefill_seq_len=0, max_decode_seq_len=max_len, query_start_loc=None, seq_start_loc=None,
+            context_lens_tensor=None, block_tables=None, is_extend=0, kv_batch_stride=engine.kv_batch_stride,
+            kv_num_heads=Hkv, kv_head_size=D, max_seq_len=max_len, slot_mapping_list=slot_ids, set_used_size=zeros,
+            extend_seq_list=no_extend, use_cuda_graph=False)
+        meta.k_cache_segment_ptr_list = engine.k_cache_ptr          # model_runner.py:749-755
+        meta.v_cache_segment_ptr_list = engine.v_cache_ptr
+        meta.kvcache_segment = segs
+        prepare_step(meta, engine.gpu_cache)
+        for kc, vc in engine.gpu_cache:
+            impl.forward(q, new_k, new_v, kc, vc, meta, k_scale, v_scale)
+        return sum(lens)
+
+    if backend_path:
+        step = step_backend
+    elif args.host_path == "plan" and args.partition_tokens == 0:
         step = step_plan
     else:
         step = step_ops
@@ -272,25 +324,33 @@ def main() -> int:
         # K+V rows of every context token, plus q in and out out
         return sum_ctx * 2 * Hkv * D * eb + B * Hq * D * 2 + B * Hq * D * 2
 
+    append_bytes = B * 2 * Hkv * D * (2 + eb)  # reshape_and_cache in/out
+
     # Everything below runs on a non-blocking stream of default priority, not on the null stream:
     # hipMemMap and hipMemUnmap wait for all work queued on the null stream, so a chunk mapped while
     # decode steps are queued there would drain the pipeline every time a sequence crosses 2 MiB.
     torch.cuda.synchronize()
     torch.cuda.set_stream(torch.cuda.Stream(device=dev))
 
-    # ---- timed region: exactly K steps, synchronised on both sides
+    # ---- timed regions: each exactly K steps, synchronised on both sides.  A region of few steps carries the
+    # fixed cost of its two ends (the host work before the first launch reaches the GPU, the wake-up after
+    # the last kernel) and whatever state the clocks are in; R regions are timed and the median one is
+    # reported, all of them listed.
     for _ in range(W):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    bytes_total = 0
-    for _ in range(K):
-        bytes_total += attn_bytes(step()) + B * 2 * Hkv * D * (2 + eb)  # + reshape_and_cache in/out
-    host_dt = time.perf_counter() - t0  # all K steps issued; the GPU may still be running
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    regions = []
+    for _ in range(R):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        nbytes = 0
+        for _ in range(K):
+            nbytes += L * (attn_bytes(step()) + append_bytes)
+        host_dt = time.perf_counter() - t0  # all K steps issued; the GPU may still be running
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        regions.append((nbytes / dt / 1e9, dt, host_dt))
+    gbps, dt, host_dt = sorted(regions)[len(regions) // 2]
     ms_per_step = dt / K * 1e3
-    gbps = bytes_total / dt / 1e9
     tokens_per_s = B * K / dt
 
     # ---- per-kernel pass: HIP events around each kernel on the stream it runs on, steps queued back to
@@ -299,7 +359,9 @@ def main() -> int:
     for _ in range(W):
         step()
     _C.check(lib.vtkv_set_kernel_timing(1))
-    kbytes = [attn_bytes(step()) for _ in range(min(K, 1024))]
+    kbytes = []
+    for _ in range(event_steps):
+        kbytes += [attn_bytes(step())] * L
     _C.check(lib.vtkv_set_kernel_timing(0))
     t_stream = (C.c_float * len(kbytes))()
     t_reduce = (C.c_float * len(kbytes))()
@@ -308,7 +370,7 @@ def main() -> int:
     part_ms, red_ms = list(t_stream), list(t_reduce)
     avg_part_ms = float(np.mean(part_ms))
     achieved = float(np.mean(kbytes)) / (avg_part_ms * 1e-3) / 1e9
-    ratio, source = MEASURED_TRAFFIC.get(args.config, (None, None))
+    ratio, mfma_busy, source = measured_traffic(args.config)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "traffic": None if ratio is None else int(ratio * float(np.mean(kbytes))),
@@ -322,60 +384,152 @@ def main() -> int:
     # ---- swap: 25 % of the sequences out to pinned host memory and back.  Unmapping is lazy, so a
     # sequence swapped back in before its chunks were needed elsewhere finds them still mapped ("warm");
     # the second round trip forces the unmapping in between ("cold": swap-in has to map every chunk).
-    nswap = max(1, B // 4)
-    swap_slots = list(range(nswap))
-    engine.swap_out(swap_slots)  # untimed: first use of the pinned arena and of the copy streams
-    engine.swap_in(swap_slots)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    moved = engine.swap_out(swap_slots)
-    t1 = time.perf_counter()
-    engine.swap_in(swap_slots)
-    t2 = time.perf_counter()
-    engine.swap_out(swap_slots)
-    t3 = time.perf_counter()
-    trimmed = vmm.trim()
-    t4 = time.perf_counter()
-    engine.swap_in(swap_slots)
-    t5 = time.perf_counter()
-    swap = {"bytes_per_direction": moved, "out_gbps": round(moved / (t1 - t0) / 1e9, 2),
-            "in_gbps": round(moved / (t2 - t1) / 1e9, 2), "in_cold_gbps": round(moved / (t5 - t4) / 1e9, 2),
-            "unmap_us_per_chunk": round((t4 - t3) / max(trimmed, 1) * 1e6, 1), "chunks": trimmed,
-            "sequences": nswap}
+    swap = None
+    if not backend_path:
+        nswap = max(1, B // 4)
+        swap_slots = list(range(nswap))
+        engine.swap_out(swap_slots)  # untimed: first use of the pinned arena and of the copy streams
+        engine.swap_in(swap_slots)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        moved = engine.swap_out(swap_slots)
+        t1 = time.perf_counter()
+        engine.swap_in(swap_slots)
+        t2 = time.perf_counter()
+        engine.swap_out(swap_slots)
+        t3 = time.perf_counter()
+        trimmed = vmm.trim()
+        t4 = time.perf_counter()
+        engine.swap_in(swap_slots)
+        t5 = time.perf_counter()
+        swap = {"bytes_per_direction": moved, "out_gbps": round(moved / (t1 - t0) / 1e9, 2),
+                "in_gbps": round(moved / (t2 - t1) / 1e9, 2), "in_cold_gbps": round(moved / (t5 - t4) / 1e9, 2),
+                "unmap_us_per_chunk": round((t4 - t3) / max(trimmed, 1) * 1e6, 1), "chunks": trimmed,
+                "sequences": nswap}
 
+    G = Hq // Hkv
     result = {
         "metric": "decode-attn HBM GB/s (% peak) + tokens/s @ Llama-3-8B shape B=64; swap GB/s",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 (fp8-e4m3 KV)" if fp8 else "bf16", "data": "synthetic",
-        "config": {"workload": cfg["name"], "layers": 1, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
+        "config": {"workload": cfg["name"], "layers": L, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
                    "mean_ctx": round(float(np.mean(final_lens)), 1), "host_path": args.host_path,
-                   "fused_append": bool(plan.fused) and step is step_plan, "value_skew_bytes": engine.value_skew},
+                   "fused_append": (bool(plan.fused) and step is step_plan) or (backend_path and not args.unfused),
+                   "value_skew_bytes": engine.value_skew},
+        "repeats": R,
+        "regions_gbps": [round(r[0], 1) for r in regions],
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
+        "ms_per_layer": round(ms_per_step / L, 4),
         "host_issue_ms_per_step": round(host_dt / K * 1e3, 4),
         "swap": swap,
         "roofline": roofline,
+        # matrix pipe of the dominant kernel, from the same counter runs as `traffic`: the share of SIMD
+        # cycles with an MFMA executing, and the part of it that is real work (G of the 16 head columns)
+        "mfma_util": None if mfma_busy is None else {"busy_frac": mfma_busy, "useful_frac": round(mfma_busy * G / 16, 4),
+                                                      "source": source},
     }
 
-    if not args.no_cpu_baseline and not fp8:
-        result["cpu_baseline"] = cpu_baseline(cfg, engine, final_lens, q, scale, args.cpu_seconds)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg, engine, final_lens, q, scale, args.cpu_seconds, k_scale, v_scale)
+        result["cpu_baseline_c1"] = cpu_baseline_c1(max(2.0, args.cpu_seconds / 3))
 
     print(json.dumps(result))
     engine.close()
     return 0
 
 
-def cpu_baseline(cfg, engine, lens, q, scale, budget_s: float):
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _time_calls(run, budget_s: float):
+    run()  # warm-up (thread pool, page faults)
+    t0 = time.perf_counter()
+    iters = 0
+    while True:
+        run()
+        iters += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s or iters >= 20000:
+            return el / iters, iters, el
+
+
+def cpu_baseline_c1(budget_s: float):
+    """BASELINE config 1 exactly, on this host's cores: fp32, B=8, Hq=32, Hkv=8, D=128, ctx U[128,1024]
+    (seed 1000; draws in the order ctx, q, K, V), the reference's CPU paged_attention_v1 on the paged
+    block-16 layout behind a random block table, and the C restatement on the contiguous [T,Hkv,D] layout."""
+    import torch
+
+    from oracle import oracle as O
+
+    gen = torch.Generator().manual_seed(1000)
+    B, Hq, Hkv, D, bs, x = 8, 32, 8, 128, 16, 4
+    lens = torch.randint(128, 1025, (B,), generator=gen).tolist()
+    q = torch.randn(B, Hq, D, generator=gen).numpy()
+    ks = [torch.randn(n, Hkv, D, generator=gen).numpy() for n in lens]
+    vs = [torch.randn(n, Hkv, D, generator=gen).numpy() for n in lens]
+    nblk = [(n + bs - 1) // bs for n in lens]
+    perm = torch.randperm(sum(nblk), generator=gen).numpy()
+    k_cache = np.zeros((sum(nblk), Hkv, D // x, bs, x), np.float32)
+    v_cache = np.zeros((sum(nblk), Hkv, D, bs), np.float32)
+    block_tables = np.zeros((B, max(nblk)), np.int32)
+    at = 0
+    for b in range(B):
+        ids = perm[at:at + nblk[b]]
+        at += nblk[b]
+        block_tables[b, :nblk[b]] = ids
+        for rows, dst in ((ks[b], k_cache), (vs[b], v_cache)):
+            pad = np.zeros((nblk[b] * bs, Hkv, D), np.float32)
+            pad[:lens[b]] = rows
+            blk = pad.reshape(nblk[b], bs, Hkv, D)
+            if dst is k_cache:
+                dst[ids] = blk.reshape(nblk[b], bs, Hkv, D // x, x).transpose(0, 2, 3, 1, 4)
+            else:
+                dst[ids] = blk.transpose(0, 2, 3, 1)
+    sl = np.array(lens, np.int32)
+    scale = float(D) ** -0.5
+    nbytes = sum(lens) * 2 * Hkv * D * 4 + 2 * B * Hq * D * 4
+    out = {"workload": f"fp32 B={B} Hq={Hq} Hkv={Hkv} D={D} ctx~U[128,1024] seed 1000 ({sum(lens)} context tokens)",
+           "cpu_model": cpu_model(), "unit": "GB/s", "algorithmic_bytes_per_call": nbytes}
+    if O.ref_available():
+        per, iters, el = _time_calls(lambda: O.ref_paged_attention(1, q, k_cache, v_cache, block_tables, sl, scale),
+                                     budget_s)
+        out["paged_block16"] = {"value": round(nbytes / per / 1e9, 3), "kind": "reference", "ms_per_call": round(per * 1e3, 3),
+                                "cores": int(O.ref().ref_num_threads()), "calls": iters}
+    else:
+        pc = O.PagedCache(k_cache, v_cache, block_tables)
+        per, iters, el = _time_calls(lambda: O.paged_attention_v1(q, pc, scale, sl), budget_s)
+        out["paged_block16"] = {"value": round(nbytes / per / 1e9, 3), "kind": "port", "ms_per_call": round(per * 1e3, 3),
+                                "cores": O.num_threads(), "calls": iters}
+    vc = O.VTensorCache(ks, vs, np.arange(B), Hkv, D)
+    per, iters, el = _time_calls(lambda: O.paged_attention_v1(q, vc, scale, sl), budget_s)
+    out["contiguous"] = {"value": round(nbytes / per / 1e9, 3), "kind": "port", "ms_per_call": round(per * 1e3, 3),
+                         "cores": O.num_threads(), "calls": iters}
+    out["omp_max_threads"] = O.num_threads()
+    return out
+
+
+def cpu_baseline(cfg, engine, lens, q, scale, budget_s: float, k_scale: float = 1.0, v_scale: float = 1.0):
     """The reference's CPU paged attention v1 (compiled from the reference sources when that
     build is present, otherwise the C restatement) on the first sequences of the same batch, in the
-    paged block-16 layout it requires."""
+    paged block-16 layout it requires.  An fp8 cache is first converted back to bf16 with its scale, the
+    reference's own protocol for fp8 (tests/kernels/test_attention.py:233-252): its CPU kernels have no fp8."""
     import torch
 
     from glake_amd import _C
     from oracle import oracle as O
 
     B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
+    fp8 = cfg["kv"] == "fp8"
     nsample = min(B, 16)
     bs, x = 16, 8
     lens = lens[:nsample]
@@ -390,7 +544,12 @@ def cpu_baseline(cfg, engine, lens, q, scale, budget_s: float):
         rows = np.zeros((nblk[b] * bs, Hkv, D), np.uint16)
         for which, dst in ((0, k_cache), (1, v_cache)):
             src = seg.getKeyDevicePtr(0) if which == 0 else seg.getValueDevicePtr(0)
-            _C.check(_C.lib().vtkv_memcpy_d2h(rows.ctypes.data_as(C.c_void_p), src, n * Hkv * D * 2))
+            if fp8:
+                codes = np.zeros((n, Hkv, D), np.uint8)
+                _C.check(_C.lib().vtkv_memcpy_d2h(codes.ctypes.data_as(C.c_void_p), src, n * Hkv * D))
+                rows[:n] = O.fp8_decode(codes, k_scale if which == 0 else v_scale, to_bf16=True)
+            else:
+                _C.check(_C.lib().vtkv_memcpy_d2h(rows.ctypes.data_as(C.c_void_p), src, n * Hkv * D * 2))
             blk = rows.reshape(nblk[b], bs, Hkv, D)
             if which == 0:  # [blk, bs, H, D/x, x] -> [blk, H, D/x, bs, x]
                 dst[blk0:blk0 + nblk[b]] = blk.reshape(nblk[b], bs, Hkv, D // x, x).transpose(0, 2, 3, 1, 4)
@@ -409,21 +568,14 @@ def cpu_baseline(cfg, engine, lens, q, scale, budget_s: float):
         pc = O.PagedCache(k_cache, v_cache, block_tables)
         run = lambda: O.paged_attention_v1(q_np, pc, scale, sl)
         cores = O.num_threads()
-    run()  # warm-up (thread pool, page faults)
-    t0 = time.perf_counter()
-    iters = 0
-    while True:
-        run()
-        iters += 1
-        el = time.perf_counter() - t0
-        if el >= budget_s or iters >= 20000:
-            break
-    per_call = el / iters
+    per_call, iters, el = _time_calls(run, budget_s)
+    # the bytes the CPU kernel reads: bf16 rows (also for an fp8 cache, which it sees dequantised)
     nbytes = sum(lens) * 2 * Hkv * D * 2 + 2 * nsample * Hq * D * 2
     return {"value": round(nbytes / per_call / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind,
+            "cpu_model": cpu_model(),
             "tokens_per_s": round(nsample / per_call, 1), "ms_per_call": round(per_call * 1e3, 3),
-            "sample": f"paged_attention_v1 (block 16, bf16) on the first {nsample} of {B} sequences "
-                      f"({sum(lens)} context tokens), {iters} calls in {el:.1f} s"}
+            "sample": f"paged_attention_v1 (block 16, bf16{' from the fp8 cache' if fp8 else ''}) on the first "
+                      f"{nsample} of {B} sequences ({sum(lens)} context tokens), {iters} calls in {el:.1f} s"}
 
 
 if __name__ == "__main__":

@@ -274,11 +274,43 @@ def paged_attention_v2(
     v_scale: Optional[float] = None,
 ) -> None:
     """Split-K entry with the reference's 512-row partitions (csrc/attention/attention_kernels.cu:
-    739-914, vllm/attention/ops/paged_attn.py:139-166).  The kernel is the same split-K kernel as
-    v1; the caller's exp_sum / max_logits / tmp_out buffers are accepted for signature
-    compatibility and not written (partials live in the library's own fp32 scratch)."""
-    paged_attention_v1(out, query, key_cache, value_cache, num_kv_heads, scale, seq_lens, block_size, max_seq_len,
-                       alibi_slopes, kv_cache_dtype, kv_scale, slot_mapping, v_scale, partition_tokens=_PARTITION_SIZE)
+    451-583,739-914, vllm/attention/ops/paged_attn.py:139-166).  With the caller's per-partition buffers
+    (``exp_sum`` / ``max_logits`` float32 [num_seqs, num_heads, P], ``tmp_out`` [num_seqs, num_heads, P,
+    head_size] of the query's dtype, P >= ceil(max_seq_len / 512)) every (sequence, kv head, partition)
+    is one workgroup and the buffers are filled as the reference fills them; ``out`` is merged from fp32
+    partials.  Without them (all three None) the same rows are cut into 512-row spans of the library's own
+    scratch."""
+    given = [t is not None for t in (exp_sum, max_logits, tmp_out)]
+    if not any(given):
+        return paged_attention_v1(out, query, key_cache, value_cache, num_kv_heads, scale, seq_lens, block_size,
+                                  max_seq_len, alibi_slopes, kv_cache_dtype, kv_scale, slot_mapping, v_scale,
+                                  partition_tokens=_PARTITION_SIZE)
+    if not all(given):
+        raise _C.VtkvError(_C.EINVAL, "exp_sum, max_logits and tmp_out come together or not at all")
+    if block_size != 1:
+        raise _C.VtkvError(_C.EINVAL, f"Unsupported block size: {block_size} (contiguous ranges use 1)")
+    _require_cuda(out, exp_sum, max_logits, tmp_out, query, seq_lens, slot_mapping)
+    num_seqs, num_heads, head_size = query.shape
+    if seq_lens.dtype != torch.int32 or slot_mapping.dtype != torch.int64:
+        raise _C.VtkvError(_C.EINVAL, "seq_lens must be int32 and slot_mapping int64")
+    parts = exp_sum.shape[-1] if exp_sum.dim() == 3 else -1
+    if (exp_sum.dtype != torch.float32 or max_logits.dtype != torch.float32 or tmp_out.dtype != query.dtype
+            or tuple(exp_sum.shape) != (num_seqs, num_heads, parts) or max_logits.shape != exp_sum.shape
+            or tuple(tmp_out.shape) != (num_seqs, num_heads, parts, head_size)
+            or not (out.is_contiguous() and exp_sum.is_contiguous() and max_logits.is_contiguous()
+                    and tmp_out.is_contiguous())):
+        raise _C.VtkvError(_C.EINVAL, "exp_sum / max_logits must be contiguous float32 [num_seqs, num_heads, P] and "
+                                      "tmp_out [num_seqs, num_heads, P, head_size] of the query's dtype")
+    qd = _dt(query)
+    lib = _C.lib()
+    ws = _workspace(lib.vtkv_decode_attention_v2_workspace_bytes(num_seqs, num_heads, head_size, parts), query.device)
+    if alibi_slopes is not None:
+        alibi_slopes = alibi_slopes.to(device=query.device, dtype=torch.float32)
+    _C.check(lib.vtkv_decode_attention_v2(
+        _ptr(out), _ptr(exp_sum), _ptr(max_logits), _ptr(tmp_out), _ptr(query), _ptr(key_cache), _ptr(value_cache),
+        _ptr(slot_mapping), _ptr(seq_lens), num_seqs, num_heads, num_kv_heads, head_size, query.stride(0),
+        float(scale), int(max_seq_len), int(parts), _ptr(alibi_slopes), qd, _dt(out), _kv_dtype(kv_cache_dtype, qd),
+        float(kv_scale), float(kv_scale if v_scale is None else v_scale), _ptr(ws), ws.numel(), _stream()))
 
 
 # --------------------------------------------------------------------------------------- cache ops

@@ -3,8 +3,11 @@ one working backend (``vllm/attention/backends/xformers.py``: ``XFormersBackend`
 ``XFormersMetadata`` :65-211, ``XFormersImpl`` :214-433), with the cache write and the decode
 attention served by the HIP kernels of ``libvtkv.so``.
 
-Decode and prompt runs are served (a batch holds one kind, as the fork schedules them); a prompt
-run writes its rows into the cache and then attends over the ranges causally.
+Decode steps, prompt runs and batches that mix the two are served (prompt tokens first, then one token
+per decode sequence, as upstream lays a batch out; the fork schedules the two kinds apart).  A prompt run
+writes its rows into the cache and then attends over the ranges causally; without a cache (the engine's
+profiling run) it attends over the key/value tensors themselves.  The sequence-wise metadata of the fork
+(``slot_mapping`` = one slot id per sequence, ``slot_m``, ``seq_lens_tensor``) is ordered like the batch.
 """
 from __future__ import annotations
 
@@ -72,6 +75,7 @@ class VTensorMetadata(AttentionMetadata, PagedAttentionMetadata):
     # query tokens per prompt when a prompt continues behind rows that are already cached (a reused
     # prefix, a later chunk of a long prompt); None: every prompt is attended in full (query = all rows)
     query_lens: Optional[List[int]] = None
+    query_lens_tensor: Optional[torch.Tensor] = None  # the same on the GPU (int32), made by prepare_step
     _cached_prefill_metadata: Optional["VTensorMetadata"] = None
     _cached_decode_metadata: Optional["VTensorMetadata"] = None
 
@@ -91,7 +95,7 @@ class VTensorMetadata(AttentionMetadata, PagedAttentionMetadata):
         if self._cached_prefill_metadata is None:
             self._cached_prefill_metadata = VTensorMetadata(
                 num_prefills=self.num_prefills, num_prefill_tokens=self.num_prefill_tokens, num_decode_tokens=0,
-                slot_mapping=self.slot_mapping[:self.num_prefill_tokens], seq_lens=self.seq_lens[:self.num_prefills],
+                slot_mapping=self.slot_mapping[:self.num_prefills], seq_lens=self.seq_lens[:self.num_prefills],
                 seq_lens_tensor=self.seq_lens_tensor[:self.num_prefills], max_query_len=self.max_query_len,
                 max_prefill_seq_len=self.max_prefill_seq_len, max_decode_seq_len=0,
                 query_start_loc=None if self.query_start_loc is None else self.query_start_loc[:self.num_prefills + 1],
@@ -109,7 +113,8 @@ class VTensorMetadata(AttentionMetadata, PagedAttentionMetadata):
         if self._cached_decode_metadata is None:
             self._cached_decode_metadata = VTensorMetadata(
                 num_prefills=0, num_prefill_tokens=0, num_decode_tokens=self.num_decode_tokens,
-                slot_mapping=self.slot_mapping, seq_lens=None, seq_lens_tensor=self.seq_lens_tensor,
+                slot_mapping=self.slot_mapping[self.num_prefills:], seq_lens=None,
+                seq_lens_tensor=self.seq_lens_tensor[self.num_prefills:],
                 max_query_len=None, max_prefill_seq_len=0, max_decode_seq_len=self.max_decode_seq_len,
                 query_start_loc=None, seq_start_loc=None, context_lens_tensor=None,
                 block_tables=None if self.block_tables is None else self.block_tables[self.num_prefills:],
@@ -146,68 +151,97 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, key_cache, value_cache,
                 attn_metadata: VTensorMetadata, kv_scale: float = 1.0, v_scale: Optional[float] = None) -> torch.Tensor:
         """query [N, Hq*D], key/value [N, Hkv*D]; key_cache / value_cache are the per-layer
-        ``KV_cache`` handles (xformers.py:269-278); returns [N, Hq*D]."""
+        ``KV_cache`` handles (xformers.py:269-278), or None in the engine's profiling run; returns
+        [N, Hq*D].  The token batch holds the prompt tokens of ``num_prefills`` sequences first, then one
+        token of each decode sequence (xformers.py:314-329); per-sequence metadata (``slot_mapping``,
+        ``slot_m``, ``seq_lens_tensor``) is ordered the same way."""
+        from ... import _custom_ops as ops
+
         query = query.view(-1, self.num_heads, self.head_size)
         key = key.view(-1, self.num_kv_heads, self.head_size)
         value = value.view(-1, self.num_kv_heads, self.head_size)
         vs = kv_scale if v_scale is None else v_scale
+        meta = attn_metadata
+        num_prefill_tokens = meta.num_prefill_tokens
+        num_decode_tokens = meta.num_decode_tokens
+        n_pre = meta.num_prefills
+        assert key.shape[0] == num_prefill_tokens + num_decode_tokens
+        assert value.shape[0] == num_prefill_tokens + num_decode_tokens
 
-        if (self.fuse_decode_append and key_cache is not None and attn_metadata.num_prefill_tokens == 0
-                and attn_metadata.decode_metadata is not None and query.dtype == torch.bfloat16):
-            # A pure decode step: the cache write (xformers.py:310-312) and the decode
-            # attention (:357-371) are one launch.  The row goes to position seq_len - 1 of each range,
-            # which is where slot_m points in the reference's flow (llama.py:340: the bytes used before
-            # this step).
-            from ... import _custom_ops as ops
+        if key_cache is None:
+            # xformers.py:336-343 with kv_caches = [None] * layers (worker.py:157, model_runner.py:846): the
+            # engine's profiling run.  Nothing is cached; the prompts attend over their own key/value rows.
+            if num_decode_tokens:
+                raise ValueError("decode tokens need a KV cache")
             output = torch.empty_like(query)
-            ops.decode_append_attention(
-                output, query, key, value, attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
-                attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], self.num_kv_heads, self.scale,
-                attn_metadata.seq_lens_tensor, attn_metadata.max_seq_len, self.alibi_slopes,
-                attn_metadata.slot_mapping, kv_cache_dtype=self.kv_cache_dtype, kv_scale=kv_scale, v_scale=vs)
+            if num_prefill_tokens:
+                self._attend_packed(output, query, key, value, list(meta.seq_lens[:n_pre]))
             return output.view(-1, self.num_heads * self.head_size)
 
-        if key_cache is not None:
-            # xformers.py:290-312: one row per sequence in decode, max_query_len rows in prefill
-            max_seq_len = 1 if attn_metadata.num_prefill_tokens == 0 else attn_metadata.max_query_len
+        k_table = meta.k_cache_segment_ptr_list[key_cache.layer_index]
+        v_table = meta.v_cache_segment_ptr_list[value_cache.layer_index]
+        output = torch.empty_like(query)
+
+        if n_pre > 0:
+            # xformers.py:290-312, prompt form: every prompt writes its new rows (all of its rows, or the
+            # query_lens rows that follow what is cached already) behind the bytes its range holds ...
+            rows_t = meta.query_lens_tensor if meta.query_lens is not None else meta.seq_lens_tensor[:n_pre]
             PagedAttention.write_to_paged_cache(
-                key, value, attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
-                attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], attn_metadata.slot_m,
-                attn_metadata.slot_mapping, attn_metadata.seq_lens_tensor, attn_metadata.cache_seq_lens, max_seq_len,
+                key[:num_prefill_tokens], value[:num_prefill_tokens], k_table, v_table, meta.slot_m[:n_pre],
+                meta.slot_mapping[:n_pre], rows_t, meta.cache_seq_lens[:n_pre], meta.max_query_len,
                 self.num_kv_heads, self.head_size, self.kv_cache_dtype, kv_scale, vs)
-
-        num_prefill_tokens = attn_metadata.num_prefill_tokens
-        num_decode_tokens = attn_metadata.num_decode_tokens
-        assert key.shape[0] == num_prefill_tokens + num_decode_tokens
-        output = None
-        if attn_metadata.prefill_metadata is not None:
-            # xformers.py:331-386: the prompt run.  The reference attends over the key/value tensors
-            # (plain prompt) or over the cache through an external kernel (cached prefix); the rows were
-            # written to the cache above, so both are one causal attention over the ranges here.
-            if key_cache is None:
-                raise NotImplementedError("prompt attention without a KV cache (the reference's profiling run)")
-            from ... import _custom_ops as ops
-            n = attn_metadata.num_prefills
-            seq_lens = list(attn_metadata.seq_lens[:n])
-            query_lens = list(attn_metadata.query_lens[:n]) if attn_metadata.query_lens is not None else seq_lens
-            output = torch.empty_like(query)
+            # ... and xformers.py:331-386: the reference attends over the key/value tensors (plain prompt)
+            # or over the cache through an external kernel (cached prefix); with the rows in the cache both
+            # are one causal attention over the ranges.
+            seq_lens = list(meta.seq_lens[:n_pre])
+            query_lens = list(meta.query_lens[:n_pre]) if meta.query_lens is not None else seq_lens
             ops.prefill_attention(
-                output[:num_prefill_tokens], query[:num_prefill_tokens],
-                attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
-                attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], self.num_kv_heads, self.scale,
-                query_lens, seq_lens, attn_metadata.slot_mapping[:n], self.alibi_slopes, self.kv_cache_dtype,
+                output[:num_prefill_tokens], query[:num_prefill_tokens], k_table, v_table, self.num_kv_heads,
+                self.scale, query_lens, seq_lens, meta.slot_mapping[:n_pre], self.alibi_slopes, self.kv_cache_dtype,
                 kv_scale, vs)
-            if attn_metadata.decode_metadata is None:
-                return output.view(-1, self.num_heads * self.head_size)
-            raise NotImplementedError("a batch that mixes prompt and decode tokens (the fork schedules them apart)")
 
-        if attn_metadata.decode_metadata is not None:
-            assert key_cache is not None, "decode needs a KV cache"
-            output = PagedAttention.forward_decode(
-                query[num_prefill_tokens:], attn_metadata.k_cache_segment_ptr_list[key_cache.layer_index],
-                attn_metadata.v_cache_segment_ptr_list[value_cache.layer_index], attn_metadata.seq_lens_tensor,
-                attn_metadata.max_seq_len, self.kv_cache_dtype, self.num_kv_heads, self.scale, self.alibi_slopes,
-                kv_scale, attn_metadata.slot_mapping, vs)
-        if output is None:
-            output = torch.empty_like(query)
+        if num_decode_tokens > 0:
+            # xformers.py:388-431: one query token per decode sequence over its whole range.
+            d_query = query[num_prefill_tokens:]
+            d_key, d_value = key[num_prefill_tokens:], value[num_prefill_tokens:]
+            d_slots = meta.slot_mapping[n_pre:]
+            d_lens = meta.seq_lens_tensor[n_pre:]
+            d_out = output[num_prefill_tokens:]
+            max_len = meta.max_decode_seq_len if n_pre > 0 and meta.max_decode_seq_len else meta.max_seq_len
+            if self.fuse_decode_append and query.dtype == torch.bfloat16:
+                # the cache write (xformers.py:310-312) and the decode attention (:357-371) in one launch.
+                # The row goes to position seq_len - 1 of each range, which is where slot_m points in the
+                # reference's flow (llama.py:340: the bytes used before this step).
+                ops.decode_append_attention(
+                    d_out, d_query, d_key, d_value, k_table, v_table, self.num_kv_heads, self.scale, d_lens, max_len,
+                    self.alibi_slopes, d_slots, kv_cache_dtype=self.kv_cache_dtype, kv_scale=kv_scale, v_scale=vs)
+            else:
+                PagedAttention.write_to_paged_cache(
+                    d_key, d_value, k_table, v_table, meta.slot_m[n_pre:], d_slots, None, None, 1,
+                    self.num_kv_heads, self.head_size, self.kv_cache_dtype, kv_scale, vs)
+                ops.paged_attention_v1(d_out, d_query, k_table, v_table, self.num_kv_heads, self.scale, d_lens, 1,
+                                       max_len, self.alibi_slopes, self.kv_cache_dtype, kv_scale, d_slots, vs)
         return output.view(-1, self.num_heads * self.head_size)
+
+    def _attend_packed(self, output: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                       seq_lens: List[int]) -> None:
+        """Causal self-attention of packed prompts over their own key/value rows, without a cache: sequence
+        b's rows [start_b, start_b + len_b) of ``key`` / ``value`` already are a token-major [T, Hkv, D]
+        range, so the prompt kernel runs on them through a pointer table made for the call."""
+        from ... import _custom_ops as ops
+
+        key, value = key.contiguous(), value.contiguous()
+        row = self.num_kv_heads * self.head_size * key.element_size()
+        starts, at = [], 0
+        for n in seq_lens:
+            starts.append(at)
+            at += n
+        if at != query.shape[0]:
+            raise ValueError(f"seq_lens add up to {at} tokens, the batch holds {query.shape[0]}")
+        dev = query.device
+        k_table = torch.tensor([key.data_ptr() + s * row for s in starts], dtype=torch.int64, device=dev)
+        v_table = torch.tensor([value.data_ptr() + s * row for s in starts], dtype=torch.int64, device=dev)
+        slots = torch.arange(len(seq_lens), dtype=torch.int64, device=dev)
+        # the rows are in the model's dtype whatever the cache would hold
+        ops.prefill_attention(output, query, k_table, v_table, self.num_kv_heads, self.scale, seq_lens, seq_lens,
+                              slots, self.alibi_slopes, "auto", 1.0, 1.0)

@@ -44,6 +44,7 @@
 // force.  fp32 accumulation, output rounded to bf16 once.  No epsilon is added to the softmax
 // denominator (the CPU twin has none, csrc/cpu/attention.cpp:43-67).
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -117,6 +118,14 @@ struct AttnParams {
   int64_t new_k_stride, new_v_stride;
   float k_quant, v_quant;  // fp8 cache: the new rows are stored as e4m3fn(x / k_quant), e4m3fn(x / v_quant)
   int inline_lens;  // sequence lengths come with the kernel arguments instead of from seq_lens
+  // Partitions aligned with the sequences, the reference's split (csrc/attention/attention_kernels.cu:451-482):
+  // > 0: workgroup ((sequence * segments per sequence + segment) * aligned_parts + j) takes rows
+  // [j * 16 * span_tiles, (j + 1) * 16 * span_tiles) of that sequence, and besides its partial result in the
+  // scratch it writes the caller's exp_sums / max_logits [B, Hq, aligned_parts] and tmp_out
+  // [B, Hq, aligned_parts, D] (bf16), which the reference's interface hands in.
+  int aligned_parts;
+  float *v2_exp_sums, *v2_max_logits;
+  uint16_t *v2_tmp_out;
 };
 
 // Sequence lengths passed by value (no upload, no dependent global load at the start of the kernel).
@@ -237,9 +246,10 @@ __global__ void __launch_bounds__(kThreads)
   // (config 5) unless the tile order is head-major as well (below), so the host asks for it together with the
   // separate merge kernel or with that order.
   const int wg = p.xcd_spans > 0 ? (int)(blockIdx.x % 8) * p.xcd_spans + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+  const int aligned = uniform(p.aligned_parts);
   int g_cur = wg * span;
-  if (g_cur >= total_tiles) return;
-  const int g_end = min(total_tiles, g_cur + span);
+  if (!aligned && g_cur >= total_tiles) return;
+  int g_end = min(total_tiles, g_cur + span);
 
   // Two tile orders.  (sequence, kv head, tile): tile g of the order is Hseg*cum[b] + kvg*nt_b + tile.
   // (kv head, sequence, tile), p.head_major: g = kvg*cum[B] + cum[b] + tile; with eight kv heads and one
@@ -248,8 +258,8 @@ __global__ void __launch_bounds__(kThreads)
   // XCD keeps to one such residue than when all XCDs read all of them (6 960 against 6 850 GB/s).
   const bool head_major = uniform(p.head_major) != 0;
   // first sequence of the span: the last b whose first tile is <= g_cur (sequences without rows own no tile)
-  int b, kvg, tile0;
-  {
+  int b = 0, kvg = 0, tile0 = 0;
+  if (!aligned) {
     const int hm_kvg = head_major ? g_cur / seq_tiles_total : 0;
     const int key = head_major ? g_cur - hm_kvg * seq_tiles_total : g_cur;  // compared with cum[b] * mul
     const int mul = head_major ? 1 : Hseg;
@@ -265,6 +275,19 @@ __global__ void __launch_bounds__(kThreads)
     tile0 = head_major ? rest : rest - kvg * nt;
   }
   int nt_b = uniform(s_cum[b + 1]) - uniform(s_cum[b]);
+  int v2_part = 0;
+  if (aligned) {
+    // one segment, named by the workgroup's index; [g_cur, g_end) only counts its tiles
+    v2_part = wg % aligned;
+    const int sk = wg / aligned;
+    kvg = sk % Hseg;
+    b = sk / Hseg;
+    nt_b = uniform(s_cum[b + 1]) - uniform(s_cum[b]);
+    tile0 = v2_part * span;
+    if (tile0 >= nt_b) return;
+    g_cur = 0;
+    g_end = min(span, nt_b - tile0);
+  }
 
   typedef const __attribute__((address_space(1))) char *gptr;
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
@@ -617,6 +640,16 @@ __global__ void __launch_bounds__(kThreads)
           o += sm_o[(w * 8 + hh) * kD + d];
         }
         const float o_norm = o / lsum;
+        if (aligned && p.v2_tmp_out) {
+          // the reference's per-partition outputs: max logit in natural units, sum of exponentials, and the
+          // partition's normalised result in the model's dtype (csrc/attention/attention_kernels.cu:404-419)
+          const int64_t vi = ((int64_t)b * p.num_heads + kv_head * G + head) * aligned + v2_part;
+          p.v2_tmp_out[vi * kD + d] = vtkv::f32_to_bf16_bits_rne(o_norm * p.v_scale);
+          if (d == 0) {
+            p.v2_max_logits[vi] = mw * 0.6931471805599453f;
+            p.v2_exp_sums[vi] = lsum;
+          }
+        }
         if (whole) {
           store_out(kv_head, head, d, o_norm * p.v_scale);
           continue;
@@ -682,7 +715,14 @@ __global__ void __launch_bounds__(kThreads)
   // ---- arrivals and merges of the shared segments (the rule of decode_attn_reduce_kernel below).
   // Pieces come from other CUs and other L2s: they were written with device-coherent stores, every wave
   // waits until its stores have completed before the arrivals are counted, and the pieces are read with
-  // device-coherent loads.  The workgroup that delivers the last piece of a segment merges it and leaves
+  // device-coherent loads.  Why relaxed atomics are enough here: ordering is not left to the memory model
+  // but made by completion.  An agent-scope atomic store on this part is a write-through store (sc1) that is
+  // acknowledged only once it is visible device-wide; s_waitcnt vmcnt(0) holds each wave until all of its
+  // stores are acknowledged, the barrier collects the waves, and only then does one lane count the arrival,
+  // so a workgroup that reads the full count can only run after every piece is visible, and it reads the
+  // pieces with loads that bypass its own L2.  A release/acquire pair at agent scope would be correct too
+  // but is implemented as a write-back and invalidate of the whole L2 on either side, which tripled the
+  // kernel's time when it was tried.  The workgroup that delivers the last piece of a segment merges it and leaves
   // the counter at zero for the next launch.
   if (p.fused_merge) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -768,7 +808,11 @@ __global__ void __launch_bounds__(kD * GROUPS * HSETS) decode_attn_reduce_kernel
   const int total_tiles = p.cum_tiles[p.num_seqs] * Hseg;
   const int span = span_of(p, total_tiles);
   const int first = p.head_major ? (kvh / hps) * p.cum_tiles[p.num_seqs] + cum_b : cum_b * Hseg + (kvh / hps) * nt;
-  const int w0 = first / span, w1 = (first + nt - 1) / span;
+  int w0 = first / span, w1 = (first + nt - 1) / span;
+  if (p.aligned_parts > 0) {
+    w0 = (b * Hseg + kvh / hps) * p.aligned_parts;
+    w1 = w0 + (nt + span - 1) / span - 1;
+  }
   const int64_t seg = p.head_major ? ((int64_t)(kvh / hps) * p.num_seqs + b) * hps + kvh % hps : (int64_t)b * Hkv + kvh;
   for (int h0 = 4 * hset; h0 < G; h0 += 4 * HSETS) {
     float m[4], wsum[4], o[4];
@@ -847,7 +891,8 @@ __global__ void __launch_bounds__(kD * GROUPS * HSETS) decode_attn_reduce_kernel
 // calls stay queued back to back as they are in production.  Up to kTimedCalls calls are kept.
 constexpr int kTimedCalls = 1024;
 struct KernelTimer {
-  bool on = false;
+  std::atomic<bool> on{false};
+  std::mutex mu;               // held by a timed call from its first event to its last, and by the readers
   std::vector<hipEvent_t> ev;  // three per call, created on first use
   int calls = 0;
 };
@@ -890,8 +935,9 @@ int64_t scratch_floats(int64_t grid, int num_seqs, int num_heads, int head_size)
 // the workspace is fixed (num_kv_heads <= num_heads).
 int64_t counter_bytes(int /*num_seqs*/, int /*num_heads*/) { return (int64_t)kMaxSeqs * kMaxKvHeads * 4; }
 
-int g_fused_merge = -1;  // -1: decide per call, 0: never, 1: always
-int g_head_major = -1;   // likewise for the head-major tile order
+// Process-wide tuning knobs, settable from any thread: every call reads each of them once, at its start.
+std::atomic<int> g_fused_merge{-1};  // -1: decide per call, 0: never, 1: always
+std::atomic<int> g_head_major{-1};   // likewise for the head-major tile order
 
 int64_t fixed_span_grid(int num_seqs, int num_kv_heads_bound, int max_seq_len, int partition_tokens) {
   const int64_t tiles = (int64_t)num_seqs * num_kv_heads_bound * ((max_seq_len + kTile - 1) / kTile);
@@ -899,14 +945,30 @@ int64_t fixed_span_grid(int num_seqs, int num_kv_heads_bound, int max_seq_len, i
   return (tiles + span - 1) / span;
 }
 
-// Shared by both entry points.  new_key == nullptr: attention only.
+// The caller's per-partition buffers of the reference's split-K interface (paged_attention_v2).
+struct V2Side {
+  float *exp_sums, *max_logits;  // [num_seqs, num_heads, max_parts]
+  void *tmp_out;                 // [num_seqs, num_heads, max_parts, head_size], q's dtype
+  int max_parts;
+};
+constexpr int kV2Partition = 512;  // rows per partition (vllm/attention/ops/paged_attn.py:10)
+
+// Shared by the entry points.  new_key == nullptr: attention only.  v2 != nullptr: partitions of 512 rows
+// aligned with the sequences, the caller's side buffers filled.
 int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
                    const int32_t *seq_lens, const int32_t *host_seq_lens, int num_seqs, int num_heads,
                    int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
                    const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale, float v_scale,
                    void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream, const void *new_key,
-                   const void *new_value, int64_t key_stride, int64_t value_stride) {
+                   const void *new_value, int64_t key_stride, int64_t value_stride, const V2Side *v2 = nullptr) {
   const bool append = new_key != nullptr;
+  if (v2) {
+    partition_tokens = kV2Partition;
+    VTKV_REQUIRE(!append, "the split-K interface has no fused append");
+    VTKV_REQUIRE(v2->exp_sums && v2->max_logits && v2->tmp_out, "null argument");
+    VTKV_REQUIRE(max_seq_len > 0 && v2->max_parts >= (max_seq_len + kV2Partition - 1) / kV2Partition,
+                 "%d partitions do not hold %d rows", v2->max_parts, max_seq_len);
+  }
   VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids, "null argument");
   VTKV_REQUIRE((seq_lens != nullptr) != (host_seq_lens != nullptr), "pass either device or host sequence lengths");
   VTKV_REQUIRE(num_seqs >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
@@ -963,7 +1025,10 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
 #undef VTKV_ROW
   void (*kernel)(AttnParams, InlineLens) = kKernels[variant];
   int64_t grid;
-  if (partition_tokens > 0) {
+  if (v2) {
+    grid = (int64_t)num_seqs * (num_kv_heads / seg_heads) * v2->max_parts;
+    VTKV_REQUIRE(grid <= (1ll << 24), "%d partitions per sequence give %lld workgroups", v2->max_parts, (long long)grid);
+  } else if (partition_tokens > 0) {
     // (the fused append adds one tile per sequence and kv head)
     grid = fixed_span_grid(num_seqs, num_kv_heads / seg_heads, max_seq_len + (append ? kTile : 0), partition_tokens);
     VTKV_REQUIRE(grid <= (1ll << 24), "partition_tokens %d gives %lld workgroups", partition_tokens, (long long)grid);
@@ -1004,11 +1069,13 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   // separate, both head-major: 1 segment per workgroup 173 / 174 and 179 / 178 us; 2 segments 190 / 194 and
   // 201 / 203; 4 segments 197 / 205 and 210 / 219; 16 segments 223 / 243 and 247 / 271): inside from two
   // segments per workgroup on.
+  const int knob_merge = g_fused_merge.load(std::memory_order_relaxed);
+  const int knob_hm = g_head_major.load(std::memory_order_relaxed);
   const int segs_per_seq = num_kv_heads / seg_heads;
   const int64_t segs = (int64_t)num_seqs * segs_per_seq;
   const bool hm_fits = partition_tokens == 0 && grid % 8 == 0 && (segs_per_seq % 8 == 0 || 8 % segs_per_seq == 0);
-  const bool hm_auto = g_head_major != 0 && hm_fits;  // the head-major order is open to this call
-  p.fused_merge = g_fused_merge == 1 || (g_fused_merge < 0 && (hm_auto ? segs >= 2 * grid : 2 * segs >= 5 * grid));
+  const bool hm_auto = knob_hm != 0 && hm_fits;  // the head-major order is open to this call
+  p.fused_merge = !v2 && (knob_merge == 1 || (knob_merge < 0 && (hm_auto ? segs >= 2 * grid : 2 * segs >= 5 * grid)));
   p.heads_per_seg = seg_heads;
   p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
   p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);
@@ -1027,9 +1094,9 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   // of the order per XCD, and eight XCDs per whole number of segments of a sequence or the other way round
   // (8 kv heads: one per XCD; 4 pairs of kv heads: a pair per two XCDs).  Without it the per-XCD span order
   // only pays with the separate merge kernel (config 5 with the merge inside lost 1.7 %).
-  p.xcd_spans = partition_tokens == 0 && grid % 8 == 0 && (!p.fused_merge || hm_auto || g_head_major == 1)
+  p.xcd_spans = partition_tokens == 0 && grid % 8 == 0 && (!p.fused_merge || hm_auto || knob_hm == 1)
                     ? (int)(grid / 8) : 0;
-  p.head_major = partition_tokens == 0 && (g_head_major == 1 ? (!p.fused_merge || p.xcd_spans > 0)
+  p.head_major = partition_tokens == 0 && (knob_hm == 1 ? (!p.fused_merge || p.xcd_spans > 0)
                                                               : (hm_auto && p.xcd_spans > 0));
   // x = code * scale: the K scale multiplies every logit, the V scale the whole output
   p.scale_log2 = scale * kLog2e * (fp8 ? k_scale : 1.f);
@@ -1041,11 +1108,17 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.k_quant = k_scale;
   p.v_quant = v_scale;
   p.inline_lens = host_seq_lens != nullptr;
+  p.aligned_parts = v2 ? v2->max_parts : 0;
+  p.v2_exp_sums = v2 ? v2->exp_sums : nullptr;
+  p.v2_max_logits = v2 ? v2->max_logits : nullptr;
+  p.v2_tmp_out = v2 ? (uint16_t *)v2->tmp_out : nullptr;
   InlineLens il;
   if (host_seq_lens) memcpy(il.v, host_seq_lens, (size_t)num_seqs * sizeof(int32_t));
 
   hipStream_t st = (hipStream_t)stream;
-  const bool timed = g_timer.on && g_timer.calls < kTimedCalls;
+  std::unique_lock<std::mutex> timer_lock(g_timer.mu, std::defer_lock);
+  if (g_timer.on.load(std::memory_order_relaxed)) timer_lock.lock();  // timed calls take turns
+  const bool timed = timer_lock.owns_lock() && g_timer.on.load(std::memory_order_relaxed) && g_timer.calls < kTimedCalls;
   hipEvent_t *ev = nullptr;
   if (timed) {
     if ((int)g_timer.ev.size() < 3 * (g_timer.calls + 1)) {
@@ -1102,6 +1175,27 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                         v_scale, workspace, workspace_bytes, partition_tokens, stream, nullptr, nullptr, 0, 0);
 }
 
+int64_t vtkv_decode_attention_v2_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_num_partitions) {
+  if (num_seqs <= 0 || num_heads <= 0 || head_size <= 0 || max_num_partitions <= 0) return 0;
+  const int64_t grid = (int64_t)num_seqs * num_heads * max_num_partitions;  // at most one workgroup per head
+  const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
+  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes +
+         counter_bytes(num_seqs, num_heads);
+}
+
+int vtkv_decode_attention_v2(void *out, float *exp_sums, float *max_logits, void *tmp_out, const void *q,
+                             const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
+                             const int32_t *seq_lens, int num_seqs, int num_heads, int num_kv_heads, int head_size,
+                             int64_t q_stride, float scale, int max_seq_len, int max_num_partitions,
+                             const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                             float v_scale, void *workspace, int64_t workspace_bytes, void *stream) {
+  VTKV_REQUIRE(seq_lens, "null argument");
+  const V2Side side = {exp_sums, max_logits, tmp_out, max_num_partitions};
+  return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, nullptr, num_seqs, num_heads, num_kv_heads,
+                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
+                        v_scale, workspace, workspace_bytes, kV2Partition, stream, nullptr, nullptr, 0, 0, &side);
+}
+
 int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,
                                  int64_t value_stride, const int64_t *k_ptrs, const int64_t *v_ptrs,
                                  const int64_t *slot_ids, const int32_t *seq_lens, const int32_t *host_seq_lens,
@@ -1117,23 +1211,25 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
 }
 
 int vtkv_set_head_major(int on) {
-  g_head_major = on < 0 ? -1 : (on != 0);
+  g_head_major.store(on < 0 ? -1 : (on != 0), std::memory_order_relaxed);
   return VTKV_OK;
 }
 
 int vtkv_set_fused_merge(int on) {
-  g_fused_merge = on < 0 ? -1 : (on != 0);
+  g_fused_merge.store(on < 0 ? -1 : (on != 0), std::memory_order_relaxed);
   return VTKV_OK;
 }
 
 int vtkv_set_kernel_timing(int on) {
-  g_timer.on = on != 0;
+  std::lock_guard<std::mutex> lk(g_timer.mu);
+  g_timer.on.store(on != 0, std::memory_order_relaxed);
   if (on) g_timer.calls = 0;
   return VTKV_OK;
 }
 
 int vtkv_attention_kernel_times(float *stream_ms, float *reduce_ms, int capacity) {
   VTKV_REQUIRE(stream_ms && reduce_ms && capacity >= 0, "null argument");
+  std::lock_guard<std::mutex> lk(g_timer.mu);
   const int n = std::min(capacity, g_timer.calls);
   for (int i = 0; i < n; ++i) {
     hipEvent_t *ev = &g_timer.ev[3 * i];

@@ -607,7 +607,8 @@ vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t 
   if (!(s) || !g_pool.segments.count(const_cast<vtkv_segment *>(s)))                                  \
   return vtkv::fail(VTKV_ESTATE, "not a live segment")
 
-// Before changing a segment: let its map-ahead requests finish, and report one that failed.
+// Before a call that grows a segment: let its map-ahead requests finish, and report one that failed (also
+// when it failed a while ago and nothing is pending any more).
 #define SEG_SETTLE(s)                                                                                 \
   do {                                                                                                \
     settle(lk, (s));                                                                                  \
@@ -618,11 +619,19 @@ vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t 
                         e_ == VTKV_ENOMEM ? "chunk pool exhausted" : "driver error");                 \
     }                                                                                                 \
   } while (0)
+// Before a call that shrinks a segment (preempt, release, destroy): let its map-ahead requests finish and
+// forget one that failed.  A full pool is exactly when the caller preempts to get chunks back, so these calls
+// must do their work whatever became of a request to grow.
+#define SEG_SETTLE_SHRINK(s)                                                                          \
+  do {                                                                                                \
+    settle(lk, (s));                                                                                  \
+    (s)->async_error = 0;                                                                             \
+  } while (0)
 
 int vtkv_seg_destroy(vtkv_segment *s) {
   std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
-  SEG_SETTLE(s);
+  SEG_SETTLE_SHRINK(s);
   int rc = shrink_locked(s, 0);
   if (rc < 0) return rc;
   if (trim_segment_locked(s, 0, -1) < 0) return VTKV_EHIP;
@@ -716,7 +725,7 @@ int vtkv_seg_ensure(vtkv_segment *s, int64_t token_bytes) {
 int vtkv_seg_preempt(vtkv_segment *s) {
   std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
-  SEG_SETTLE(s);
+  SEG_SETTLE_SHRINK(s);
   int rc = shrink_locked(s, 0);
   if (rc < 0) return rc;
   s->used = 0;
@@ -726,7 +735,7 @@ int vtkv_seg_preempt(vtkv_segment *s) {
 int vtkv_seg_release(vtkv_segment *s) {
   std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);
-  SEG_SETTLE(s);
+  SEG_SETTLE_SHRINK(s);
   // vmm_allocator.cpp:393-420: keep the first expand_size bytes mapped when at least that much is
   // mapped, otherwise (fewer bytes mapped than expand_size) unmap everything.
   const int64_t keep = s->mapped >= s->expand_bytes ? s->expand_bytes : 0;
@@ -741,7 +750,7 @@ int vtkv_seg_share_prefix(vtkv_segment *dst, vtkv_segment *src, int64_t bytes, v
   SEG_CHECK(dst);
   SEG_CHECK(src);
   SEG_SETTLE(dst);
-  SEG_SETTLE(src);
+  settle(lk, src);  // the source is not changed: a failed request of its own is its next growth call's to report
   VTKV_REQUIRE(dst != src && dst->layer_num == src->layer_num, "segments must differ and have the same layer count");
   VTKV_REQUIRE(bytes >= 0 && bytes <= src->used && src->used <= src->mapped, "prefix of %lld bytes exceeds the source's %lld",
                (long long)bytes, (long long)src->used);
@@ -852,23 +861,35 @@ int vtkv_extend_kv_cache_batch(vtkv_segment *const *segs, int n, const int64_t *
   std::unique_lock<std::mutex> lk(g_pool.mu);
   VTKV_REQUIRE(n >= 0 && (n == 0 || (segs && token_bytes && slot_m_out)), "null argument");
   for (int i = 0; i < n; ++i) SEG_CHECK(segs[i]);
-  for (int i = 0; i < n; ++i) {
-    vtkv_segment *s = segs[i];
-    if (set_used_tokens && set_used_tokens[i] > 0) s->used = set_used_tokens[i] * kv_size;
-    // rows that need a chunk which is being mapped ahead wait for it here (a prompt always does: its
-    // reservation looks 100 rows ahead)
-    if (s->pending && (!gen || s->used + token_bytes[i] + s->v_skew > s->mapped)) SEG_SETTLE(s);
-    slot_m_out[i] = s->used;
-    if (gen) {
-      int rc = ensure_locked(s, token_bytes[i]);
-      if (rc < 0) return rc;
-      s->used += token_bytes[i];
-    } else {
-      int rc = reserve_locked(s, token_bytes[i], kv_size);
-      if (rc < 0) return rc;
+  // A failure part of the way through (pool exhausted, a failed map-ahead request) leaves every sequence's used
+  // size as it was before the call, so that the caller can preempt a sequence and run the step again; chunks
+  // mapped on the way stay mapped.
+  std::vector<int64_t> before((size_t)n);
+  for (int i = 0; i < n; ++i) before[(size_t)i] = segs[i]->used;
+  auto body = [&]() -> int {
+    for (int i = 0; i < n; ++i) {
+      vtkv_segment *s = segs[i];
+      if (set_used_tokens && set_used_tokens[i] > 0) s->used = set_used_tokens[i] * kv_size;
+      // rows that need a chunk which is being mapped ahead wait for it here (a prompt always does: its
+      // reservation looks 100 rows ahead); a request that failed earlier is reported by this call too
+      if ((s->pending && (!gen || s->used + token_bytes[i] + s->v_skew > s->mapped)) || (!s->pending && s->async_error))
+        SEG_SETTLE(s);
+      slot_m_out[i] = s->used;
+      if (gen) {
+        int rc = ensure_locked(s, token_bytes[i]);
+        if (rc < 0) return rc;
+        s->used += token_bytes[i];
+      } else {
+        int rc = reserve_locked(s, token_bytes[i], kv_size);
+        if (rc < 0) return rc;
+      }
     }
-  }
-  return VTKV_OK;
+    return VTKV_OK;
+  };
+  const int rc = body();
+  if (rc < 0)
+    for (int i = 0; i < n; ++i) segs[i]->used = before[(size_t)i];
+  return rc;
 }
 
 uint64_t vtkv_ptr_table_create(int num_seqs) {

@@ -227,9 +227,13 @@ class KVCache:
 class KV_cache:
     """Per-layer handle the model code passes around (vmm_allocator/vmm_allocator.py:5-19)."""
 
-    def __init__(self, max_seqs: int, layer_index: int) -> None:
+    def __init__(self, max_seqs: int, layer_index: int, kv_cache_dtype: str = "auto") -> None:
         self.max_seqs = max_seqs
         self.layer_index = layer_index
+        # "auto" (rows of the model's element size) or "fp8" (one byte per element): what the ranges behind this
+        # table hold, so that the step prologue can size a row; no counterpart in the reference, whose rows
+        # are always two bytes per element (vllm/model_executor/models/llama.py:315)
+        self.kv_cache_dtype = kv_cache_dtype
         self.kv_cache = KVCache(self.max_seqs)
         self.vmm_ptr = self.kv_cache.getKVCachePtr()
 

@@ -86,7 +86,9 @@ class CacheEngine:
             for seg in self.vmm_kvcache_segment:
                 seg.set_value_skew(self.value_skew)
         # cache_engine.py:111-129: per layer one pointer table for K and one for V
-        self.gpu_cache = [(vmm.KV_cache(max_num_seqs, l), vmm.KV_cache(max_num_seqs, l)) for l in range(num_layers)]
+        self.kv_cache_dtype = "fp8" if _dtype_size(dtype) == 1 else "auto"
+        self.gpu_cache = [(vmm.KV_cache(max_num_seqs, l, self.kv_cache_dtype),
+                           vmm.KV_cache(max_num_seqs, l, self.kv_cache_dtype)) for l in range(num_layers)]
         vmm.copy_kv_cache([k.kv_cache for k, _ in self.gpu_cache], [v.kv_cache for _, v in self.gpu_cache],
                           self.vmm_kvcache_segment)
         # cache_engine.py:98-109: the same pointers as int64 device tensors, one per layer

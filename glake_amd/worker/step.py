@@ -3,41 +3,84 @@
 chunk where a sequence crosses a 2 MiB boundary, and hand the byte offsets to the kernels."""
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
 from .. import vmm_allocator as vmm
 
 
-def prepare_step(attn_metadata, kv_caches: Sequence) -> None:
-    """Fills ``attn_metadata.slot_m`` (and ``decode_seq_len``) for this step.
+def kv_row_bytes(num_kv_heads: int, head_size: int, kv_cache_dtype: str = "auto", model_elem_bytes: int = 2) -> int:
+    """Bytes of one K (or V) row of one token in a sequence's range: one byte per element for an fp8 cache,
+    otherwise the model's element size (the reference hard-codes 2, llama.py:315)."""
+    elem = 1 if kv_cache_dtype in ("fp8", "fp8_e4m3") else int(model_elem_bytes)
+    return int(num_kv_heads) * int(head_size) * elem
+
+
+def prepare_step(attn_metadata, kv_caches: Sequence, kv_cache_dtype: Optional[str] = None,
+                 model_elem_bytes: int = 2) -> None:
+    """Fills ``attn_metadata.slot_m`` (and ``decode_seq_len``, ``query_lens_tensor``, ``cache_seq_lens``)
+    for this step.
 
     kv_caches: per layer a (K, V) pair of ``KV_cache`` handles, or None entries during profiling.
+    kv_cache_dtype: "auto" (rows of the model's element size) or "fp8" (one byte per element); by default
+    what the ``CacheEngine`` that made the handles says (``KV_cache.kv_cache_dtype``), else "auto".
+
+    The batch holds ``num_prefills`` prompts first, then the decode sequences (one new row each).  A prompt
+    writes ``query_lens[i]`` rows when ``attn_metadata.query_lens`` is given (a prompt, or a chunk of one, behind
+    rows that are already cached: ``seq_lens[i]`` then counts the cached rows too), otherwise ``seq_lens[i]``.
     """
     if not kv_caches or kv_caches[0] is None:
         return
     k_cache = [k.kv_cache for k, _ in kv_caches]
     v_cache = [v.kv_cache for _, v in kv_caches]
-    kv_size = attn_metadata.kv_num_heads * attn_metadata.kv_head_size * 2  # llama.py:315, bytes of a bf16 row
+    if kv_cache_dtype is None:
+        kv_cache_dtype = getattr(kv_caches[0][0], "kv_cache_dtype", "auto")
+    kv_size = kv_row_bytes(attn_metadata.kv_num_heads, attn_metadata.kv_head_size, kv_cache_dtype,
+                           model_elem_bytes)  # llama.py:315
     n = len(attn_metadata.slot_mapping_list)
-    if attn_metadata.num_prefills > 0:
-        kv_size_list: List[int] = [seq_len * kv_size for seq_len in attn_metadata.seq_lens]  # llama.py:318-320
-        decode_seq_len = None
-    else:
+    n_pre = attn_metadata.num_prefills
+    device = attn_metadata.slot_mapping.device
+    segs = attn_metadata.kvcache_segment
+    slots = attn_metadata.slot_mapping_list
+    used = attn_metadata.set_used_size
+    slot_m: List[int] = []
+    if n_pre > 0:
+        rows = list(attn_metadata.query_lens[:n_pre]) if attn_metadata.query_lens is not None \
+            else list(attn_metadata.seq_lens[:n_pre])
+        kv_size_list: List[int] = [r * kv_size for r in rows]  # llama.py:318-320
+        slot_m += vmm.extend_kv_cache_batch(k_cache, v_cache, slots[:n_pre], kv_size_list, segs[:n_pre],
+                                            used[:n_pre], kv_size, False)  # llama.py:340, prompt form
+        if attn_metadata.query_lens is not None:
+            attn_metadata.query_lens_tensor = torch.tensor(rows, dtype=torch.int32, device=device)
+        if attn_metadata.query_lens is not None or attn_metadata.cache_seq_lens is None:
+            # where each prompt's rows start in the packed key/value tensors (the reference's cache_seq_lens,
+            # model_runner.py:366-370, which it builds from seq_lens: right only without cached rows)
+            starts = [0] * n_pre
+            for i in range(1, n_pre):
+                starts[i] = starts[i - 1] + rows[i - 1]
+            attn_metadata.cache_seq_lens = torch.tensor(starts, dtype=torch.int32, device=device)
+    decode_seq_len = None
+    if n > n_pre:
         # llama.py:321-337: the reference spins on its background mapper here and then queues
         # eagerExtend requests; here a row that needs a chunk which is still being mapped waits inside
         # extend_kv_cache_batch, so only the requests remain
-        decode_seq_len = torch.ones(n, dtype=torch.int32, device=attn_metadata.slot_mapping.device)
-        kv_size_list = [kv_size] * n
-        for idx, slot_id in enumerate(attn_metadata.extend_seq_list):
-            if slot_id != -1:
-                attn_metadata.kvcache_segment[idx].eagerExtend(kv_size, slot_id)
+        nd = n - n_pre
+        decode_seq_len = torch.ones(nd, dtype=torch.int32, device=device)
+        ext = attn_metadata.extend_seq_list or []
+        for idx, slot_id in enumerate(ext):
+            if slot_id != -1 and idx >= n_pre:
+                segs[idx].eagerExtend(kv_size, slot_id)
+        try:
+            slot_m += vmm.extend_kv_cache_batch(k_cache, v_cache, slots[n_pre:], [kv_size] * nd, segs[n_pre:],
+                                                used[n_pre:], kv_size, True)  # llama.py:340, decode form
+        except Exception:
+            # the step did not happen: the prompts' rows are given back too (the decode half has undone itself)
+            for seg, before in zip(segs[:n_pre], slot_m):
+                seg.set_used_size(before)
+            raise
     attn_metadata.decode_seq_len = decode_seq_len
-    slot_m = vmm.extend_kv_cache_batch(k_cache, v_cache, attn_metadata.slot_mapping_list, kv_size_list,
-                                       attn_metadata.kvcache_segment, attn_metadata.set_used_size, kv_size,
-                                       attn_metadata.num_prefills == 0)  # llama.py:340
-    attn_metadata.slot_m = torch.tensor(slot_m, dtype=torch.int64, device=attn_metadata.slot_mapping.device)
+    attn_metadata.slot_m = torch.tensor(slot_m, dtype=torch.int64, device=device)
 
 
 class DecodeStepPlan:

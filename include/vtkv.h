@@ -148,8 +148,12 @@ int64_t vtkv_pool_shared_chunks(void);
 /* Map `num_chunks` more chunks into every range of the segment on a worker thread and return at once;
  * replaces KVcacheSegment::eagerExtend and the eagerly_extend thread (vmm_allocator.cpp:40-72,307-320).
  * Nothing happens if the ranges are fully mapped.  Any later call that changes the segment, and
- * vtkv_extend_kv_cache_batch when a new row needs the chunk, first waits for the request; a failed
- * request (pool exhausted) is reported by that call.  The driver calls run outside the pool's lock. */
+ * vtkv_extend_kv_cache_batch when a new row needs the chunk, first waits for the request.  A failed
+ * request (pool exhausted) is reported once, by the next call that grows the segment (vtkv_seg_expand,
+ * vtkv_seg_reserve, vtkv_seg_ensure, vtkv_seg_share_prefix as destination, vtkv_extend_kv_cache_batch);
+ * calls that shrink it (vtkv_seg_preempt, vtkv_seg_release, vtkv_seg_destroy) forget the failure and do
+ * their work, since a full pool is when a caller preempts to get chunks back.  The driver calls run
+ * outside the pool's lock. */
 int vtkv_seg_eager_extend(vtkv_segment *s, int num_chunks);
 /* Map-ahead requests of the segment that are queued or running; 0 is the reference's "ready" flag
  * (query_shm, vmm_allocator.cpp:86-92). <0 on error. */
@@ -161,7 +165,9 @@ int vtkv_map_ahead_wait(void);
  * For i < n: if set_used_tokens[i] > 0, used = set_used_tokens[i]*kv_size; slot_m_out[i] = used;
  * then gen ? (ensure mapped, used += token_bytes[i]) : reserve(token_bytes[i], kv_size).
  * Unlike the reference the decode branch maps a chunk itself when the new token crosses the mapped
- * size (the reference leaves that to a racing background thread). */
+ * size (the reference leaves that to a racing background thread).  When the call fails (VTKV_ENOMEM: pool
+ * exhausted) every segment's used size is what it was before the call, so the caller can preempt a
+ * sequence and repeat the step; chunks mapped on the way stay mapped. */
 int vtkv_extend_kv_cache_batch(vtkv_segment *const *segs, int n, const int64_t *token_bytes,
                                const int64_t *set_used_tokens, int64_t kv_size, int gen, int64_t *slot_m_out);
 
@@ -280,6 +286,27 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                           const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
                           float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
                           void *stream);
+
+/* The reference's split-K interface: paged_attention_v2 (csrc/attention/attention_kernels.cu:451-583 kernel and
+ * reduce, :739-914 launcher; CPU twin csrc/cpu/attention.cpp:434-646; Python vllm/attention/ops/paged_attn.py:
+ * 139-166).  Same result as vtkv_decode_attention; the rows of every sequence are cut into partitions of 512,
+ * one workgroup per (sequence, kv head, partition), and the caller's per-partition buffers are filled as the
+ * reference fills them:
+ *   exp_sums, max_logits  float [num_seqs, num_heads, max_num_partitions]: sum of exp(logit - max) over the
+ *              partition's rows, and that max (scaled logits, natural units)
+ *   tmp_out    [num_seqs, num_heads, max_num_partitions, head_size] of q_dtype: the partition's own normalised
+ *              result
+ *   max_num_partitions  >= ceil(max_seq_len / 512); entries of partitions past a sequence's end are not written
+ * `out` is merged from the library's fp32 partials, not from the rounded tmp_out.
+ * workspace: at least vtkv_decode_attention_v2_workspace_bytes(...) bytes, zero-filled before first use like
+ * vtkv_decode_attention's (one buffer of the larger size can serve both). */
+int64_t vtkv_decode_attention_v2_workspace_bytes(int num_seqs, int num_heads, int head_size, int max_num_partitions);
+int vtkv_decode_attention_v2(void *out, float *exp_sums, float *max_logits, void *tmp_out, const void *q,
+                             const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
+                             const int32_t *seq_lens, int num_seqs, int num_heads, int num_kv_heads, int head_size,
+                             int64_t q_stride, float scale, int max_seq_len, int max_num_partitions,
+                             const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                             float v_scale, void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Query tokens one unit may hold: 128 / (num_heads/num_kv_heads) (one workgroup per unit and kv head).
  * 0 for unsupported shapes. */

@@ -7,6 +7,8 @@ holding the same bf16-representable values): a bf16 store alone moves a value by
 relative, so two correctly computed bf16 tensors can differ by more than the tolerance.  For the
 bf16 output the checks are: it is the round-to-nearest-even of the kernel's fp32 result bit for
 bit, and it is never more than one bf16 step from the oracle's bf16 output."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -243,3 +245,73 @@ def test_calls_on_two_streams_do_not_share_scratch(gpu_pool):
             assert torch.equal(b["out"], ref)
     for b in batches:
         b["gpu"].close()
+
+
+def test_two_threads_attend_while_timing_is_on_and_the_knobs_flip(gpu_pool):
+    """The kernel timer and the two tuning knobs are process-wide: two host threads attend on their own
+    streams with timing switched on while the main thread keeps flipping the knobs.  Every result must equal
+    one of the results the same call gives alone (the knobs only change fp32 summation order), the timer must
+    have recorded whole calls, and nothing may crash."""
+    import threading
+
+    import torch
+
+    from glake_amd import _C, _custom_ops as ops
+
+    lib = _C.lib()
+    rng = np.random.default_rng(61)
+    hq, hkv, d = 32, 8, 128
+    scale = d ** -0.5
+    lens = [900, 1500, 700, 64, 2100, 33]
+    gpu = GpuSeqs(gpu_pool, len(lens), hkv, d, 2, max(lens))
+    ks, vs = [], []
+    for i, t in enumerate(lens):
+        ks.append(bf16_randn(rng, (t, hkv, d)))
+        vs.append(bf16_randn(rng, (t, hkv, d)))
+        gpu.upload(i, ks[-1], vs[-1])
+    kt, vt = gpu.table_tensors()
+    q = bf16_randn(rng, (len(lens), hq, d))
+    q_t = torch_bf16_from_bits(q)
+    sl = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    slot = torch.arange(len(lens), dtype=torch.int64, device="cuda")
+    want = O.paged_attention_v1(O.bf16_to_f32(q), O.VTensorCache(ks, vs, np.arange(len(lens)), hkv, d), scale, lens)
+    errors, results = [], [[], []]
+
+    def worker(idx):
+        try:
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                for _ in range(60):
+                    out = torch.empty(len(lens), hq, d, dtype=torch.float32, device="cuda")
+                    ops.paged_attention_v1(out, q_t, kt, vt, hkv, scale, sl, 1, max(lens), None, "auto", 1.0, slot)
+                    results[idx].append(out)
+            st.synchronize()
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    _C.check(lib.vtkv_set_kernel_timing(1))
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    flips = 0
+    while any(t.is_alive() for t in threads):
+        _C.check(lib.vtkv_set_fused_merge(flips % 3 - 1))
+        _C.check(lib.vtkv_set_head_major((flips // 3) % 3 - 1))
+        flips += 1
+    for t in threads:
+        t.join()
+    _C.check(lib.vtkv_set_fused_merge(-1))
+    _C.check(lib.vtkv_set_head_major(-1))
+    _C.check(lib.vtkv_set_kernel_timing(0))
+    assert not errors, errors
+    t_stream = (C.c_float * 200)()
+    t_reduce = (C.c_float * 200)()
+    n = _C.check(lib.vtkv_attention_kernel_times(t_stream, t_reduce, 200))
+    assert n == 120 and all(0.0 < t_stream[i] < 100.0 and 0.0 <= t_reduce[i] < 100.0 for i in range(n))
+    torch.cuda.synchronize()
+    for outs in results:
+        assert len(outs) == 60
+        for o in outs:
+            err = np.abs(o.cpu().numpy() - want)
+            assert np.all(err <= ATOL + RTOL * np.abs(want))
+    gpu.close()

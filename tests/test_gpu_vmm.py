@@ -248,6 +248,50 @@ def test_map_ahead_requests_run_on_the_worker_and_settle(gpu_pool):
     assert vmm.showFreeBlocks() == free0
 
 
+def test_failed_map_ahead_does_not_stop_a_preemption(gpu_pool):
+    """Pool exhausted, a map-ahead request fails: calls that shrink the segment still do their work (that is how
+    the scheduler gets chunks back), the failure is reported once by the next call that grows it, and a step
+    that fails part of the way leaves every sequence's used size as it was."""
+    from glake_amd import _C
+
+    vmm = gpu_pool
+    vmm.trim()
+    free0 = vmm.showFreeBlocks()
+    row = 2048
+    segs = [vmm.KVcacheSegment(1, 4 * CHUNK, 0, False) for _ in range(3)]
+    for s in segs:
+        s.expandMultiSegment(1)
+        s.set_used_size(CHUNK - 2 * row)
+    hog = vmm.KVcacheSegment(1, (vmm.showFreeBlocks() // 2 + 2) * CHUNK, 0, False)
+    hog.expandMultiSegment(vmm.showFreeBlocks() // 2)            # at most one chunk left: no room for a K+V pair
+    assert vmm.showFreeBlocks() < 2
+    for s in segs:
+        s.eagerExtend(row, 0)
+    vmm.wait_map_ahead()
+    assert all(s.actual_size == CHUNK for s in segs)              # nothing half-mapped
+    # shrinking calls carry on and give the chunks back
+    segs[0].preempt_seq(0)
+    assert segs[0].actual_size == 0 and segs[0].used_size == 0
+    assert vmm.showFreeBlocks() >= 2
+    segs[0].expandMultiSegment(1)                                # the old failure is forgotten, not reported here
+    segs[0].preempt_seq(0)
+    # a growing call reports the stale failure once, although nothing is pending, and rolls the step back
+    used = [s.used_size for s in segs[1:]]
+    with pytest.raises(_C.VtkvOutOfChunks):
+        vmm.extend_kv_cache_batch(None, None, [1, 2], [row, row], segs[1:], [0, 0], row, True)
+    assert [s.used_size for s in segs[1:]] == used
+    with pytest.raises(_C.VtkvOutOfChunks):                      # segs[2]'s own failure, reported in its turn
+        vmm.extend_kv_cache_batch(None, None, [1, 2], [row, row], segs[1:], [0, 0], row, True)
+    assert [s.used_size for s in segs[1:]] == used
+    slot_m = vmm.extend_kv_cache_batch(None, None, [1, 2], [row, row], segs[1:], [0, 0], row, True)
+    assert slot_m == used and [s.used_size for s in segs[1:]] == [u + row for u in used]
+    segs[1].release_seq(1)
+    hog.destroy()
+    for s in segs:
+        s.destroy()
+    assert vmm.showFreeBlocks() == free0
+
+
 def test_shared_prefix_maps_whole_chunks_twice_and_copies_the_tail(gpu_pool):
     """A new sequence that starts with another one's prefix: whole chunks become visible at a second
     address without taking chunks from the pool, the partly filled chunk is copied, both sequences go on
