@@ -299,7 +299,7 @@ def main() -> int:
         lens = state["lens"] = [n + 1 for n in state["lens"]]
         max_len = max(lens)
         meta = VTensorBackend.make_metadata(
-            num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B, slot_mapping=slot_t, seq_lens=None,
+            num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B, slot_mapping=slot_t, seq_lens=lens,
             seq_lens_tensor=torch.tensor(lens, dtype=torch.int32, device=dev), max_query_len=None,
             max_prefill_seq_len=0, max_decode_seq_len=max_len, query_start_loc=None, seq_start_loc=None,
             context_lens_tensor=None, block_tables=None, is_extend=0, kv_batch_stride=engine.kv_batch_stride,

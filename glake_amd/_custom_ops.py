@@ -167,7 +167,8 @@ def decode_append_attention(
     else:
         if len(seq_lens) != num_seqs:
             raise _C.VtkvError(_C.EINVAL, "one sequence length per query row")
-        dev_lens, host_lens = None, (C.c_int32 * num_seqs)(*[int(x) for x in seq_lens])
+        # (a ctypes int32 array made by an earlier call is taken as it is: a step's lengths serve every layer)
+        dev_lens, host_lens = None, seq_lens if isinstance(seq_lens, C.Array) else (C.c_int32 * num_seqs)(*seq_lens)
     qd = _dt(query)
     lib = _C.lib()
     need = lib.vtkv_decode_attention_workspace_bytes(num_seqs, num_heads, head_size, max_seq_len, partition_tokens)

@@ -76,6 +76,7 @@ class VTensorMetadata(AttentionMetadata, PagedAttentionMetadata):
     # prefix, a later chunk of a long prompt); None: every prompt is attended in full (query = all rows)
     query_lens: Optional[List[int]] = None
     query_lens_tensor: Optional[torch.Tensor] = None  # the same on the GPU (int32), made by prepare_step
+    _host_decode_lens: Optional[object] = None  # the decode sequences' lengths as a C array, made on first use
     _cached_prefill_metadata: Optional["VTensorMetadata"] = None
     _cached_decode_metadata: Optional["VTensorMetadata"] = None
 
@@ -202,16 +203,27 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
 
         if num_decode_tokens > 0:
             # xformers.py:388-431: one query token per decode sequence over its whole range.
-            d_query = query[num_prefill_tokens:]
-            d_key, d_value = key[num_prefill_tokens:], value[num_prefill_tokens:]
-            d_slots = meta.slot_mapping[n_pre:]
-            d_lens = meta.seq_lens_tensor[n_pre:]
-            d_out = output[num_prefill_tokens:]
+            if n_pre == 0:  # the common case, a pure decode step: no views to make
+                d_query, d_key, d_value, d_out = query, key, value, output
+                d_slots, d_lens = meta.slot_mapping, meta.seq_lens_tensor
+            else:
+                d_query = query[num_prefill_tokens:]
+                d_key, d_value = key[num_prefill_tokens:], value[num_prefill_tokens:]
+                d_slots = meta.slot_mapping[n_pre:]
+                d_lens = meta.seq_lens_tensor[n_pre:]
+                d_out = output[num_prefill_tokens:]
             max_len = meta.max_decode_seq_len if n_pre > 0 and meta.max_decode_seq_len else meta.max_seq_len
             if self.fuse_decode_append and query.dtype == torch.bfloat16:
                 # the cache write (xformers.py:310-312) and the decode attention (:357-371) in one launch.
                 # The row goes to position seq_len - 1 of each range, which is where slot_m points in the
-                # reference's flow (llama.py:340: the bytes used before this step).
+                # reference's flow (llama.py:340: the bytes used before this step).  Where the metadata also
+                # holds the lengths on the host (model_runner.py:607 passes both), up to 512 of them travel
+                # with the kernel arguments, which spares the kernel a dependent load at its start.
+                if meta.seq_lens is not None and num_decode_tokens <= 512 and len(meta.seq_lens) == n_pre + num_decode_tokens:
+                    if meta._host_decode_lens is None:  # once per step, shared by the layers
+                        import ctypes
+                        meta._host_decode_lens = (ctypes.c_int32 * num_decode_tokens)(*meta.seq_lens[n_pre:])
+                    d_lens = meta._host_decode_lens
                 ops.decode_append_attention(
                     d_out, d_query, d_key, d_value, k_table, v_table, self.num_kv_heads, self.scale, d_lens, max_len,
                     self.alibi_slopes, d_slots, kv_cache_dtype=self.kv_cache_dtype, kv_scale=kv_scale, v_scale=vs)
