@@ -85,6 +85,9 @@ SIGNATURES = {
     "vtkv_decode_attention_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
     "vtkv_decode_attention": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f, _i, _p, _i, _i, _i, _f, _f, _p,
                                     _i64, _i, _p]),
+    "vtkv_decode_attention_noalloc_max_bytes": (_i64, []),
+    "vtkv_decode_attention_noalloc": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f, _i, _p, _i, _i, _i, _f, _f,
+                                            _p]),
     "vtkv_decode_attention_v2_workspace_bytes": (_i64, [_i, _i, _i, _i]),
     "vtkv_decode_attention_v2": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f, _i, _i, _p, _i,
                                        _i, _i, _f, _f, _p, _i64, _p]),

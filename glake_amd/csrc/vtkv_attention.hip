@@ -886,6 +886,47 @@ __global__ void __launch_bounds__(kD * GROUPS * HSETS) decode_attn_reduce_kernel
   }
 }
 
+__global__ void clear_counters_kernel(uint32_t *counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0u;
+}
+
+// Scratch of vtkv_decode_attention_noalloc: partial results, prefix sums and arrival counters of one call, in
+// device memory that belongs to the loaded library itself, so that the entry point has nothing to allocate.
+// Every device the library runs on holds its own copy of the array at its own address until the process ends.
+// In host code `g_static_scratch` only names the symbol; the address kernels can use comes from
+// hipGetSymbolAddress, once per device (static_scratch_ptr below).
+constexpr int64_t kStaticScratchBytes = 32ll << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+struct StaticScratch {
+  std::mutex mu;
+  void *ptr[kMaxDevices] = {};
+};
+StaticScratch g_scratch_ptrs;
+
+// Device address of the current device's copy of g_static_scratch; nullptr (and the error set) on failure.
+void *static_scratch_ptr() {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    vtkv::fail(VTKV_EHIP, "hipGetDevice failed or device %d is beyond %d: %s", dev, kMaxDevices, hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lk(g_scratch_ptrs.mu);
+  if (!g_scratch_ptrs.ptr[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
+    if (e != hipSuccess || !ptr) {
+      vtkv::fail(VTKV_EHIP, "hipGetSymbolAddress of the static scratch failed: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptrs.ptr[dev] = ptr;
+  }
+  return g_scratch_ptrs.ptr[dev];
+}
+
 // Optional per-kernel timing for benchmarks: when switched on, every vtkv_decode_attention call
 // records events around its two launches on the caller's stream, without waiting for them, so the
 // calls stay queued back to back as they are in production.  Up to kTimedCalls calls are kept.
@@ -960,7 +1001,8 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
                    int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
                    const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale, float v_scale,
                    void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream, const void *new_key,
-                   const void *new_value, int64_t key_stride, int64_t value_stride, const V2Side *v2 = nullptr) {
+                   const void *new_value, int64_t key_stride, int64_t value_stride, const V2Side *v2 = nullptr,
+                   bool static_scratch = false) {
   const bool append = new_key != nullptr;
   if (v2) {
     partition_tokens = kV2Partition;
@@ -1041,6 +1083,10 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   const int64_t count_bytes = counter_bytes(num_seqs, num_heads);
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
   const int64_t need = n_float * (int64_t)sizeof(float) + cum_bytes + count_bytes;
+  if (static_scratch && workspace_bytes < need)
+    return vtkv::fail(VTKV_EINVAL, "%d sequences of %d heads need %lld bytes of scratch, the library's static scratch "
+                      "holds %lld: use vtkv_decode_attention with a workspace of the caller's", num_seqs, num_heads,
+                      (long long)need, (long long)workspace_bytes);
   if (!workspace || workspace_bytes < need)
     return vtkv::fail(VTKV_ENOMEM, "workspace of %lld bytes is smaller than the %lld needed",
                       (long long)workspace_bytes, (long long)need);
@@ -1116,8 +1162,16 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   if (host_seq_lens) memcpy(il.v, host_seq_lens, (size_t)num_seqs * sizeof(int32_t));
 
   hipStream_t st = (hipStream_t)stream;
+  if (static_scratch && p.fused_merge) {
+    // The static scratch is shared by every call on this device and keeps what the last one left: the arrival
+    // counters of this call's (sequence, kv head) pairs are cleared first (by a kernel, not a memset, so that
+    // the call can be recorded into a HIP graph).
+    const int n_count = num_seqs * num_kv_heads;
+    hipLaunchKernelGGL(clear_counters_kernel, dim3((n_count + 255) / 256), dim3(256), 0, st, p.seg_count, n_count);
+  }
   std::unique_lock<std::mutex> timer_lock(g_timer.mu, std::defer_lock);
-  if (g_timer.on.load(std::memory_order_relaxed)) timer_lock.lock();  // timed calls take turns
+  // timed calls take turns; the entry point that must not allocate is never timed (events are created on demand)
+  if (!static_scratch && g_timer.on.load(std::memory_order_relaxed)) timer_lock.lock();
   const bool timed = timer_lock.owns_lock() && g_timer.on.load(std::memory_order_relaxed) && g_timer.calls < kTimedCalls;
   hipEvent_t *ev = nullptr;
   if (timed) {
@@ -1194,6 +1248,21 @@ int vtkv_decode_attention_v2(void *out, float *exp_sums, float *max_logits, void
   return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, nullptr, num_seqs, num_heads, num_kv_heads,
                         head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
                         v_scale, workspace, workspace_bytes, kV2Partition, stream, nullptr, nullptr, 0, 0, &side);
+}
+
+int64_t vtkv_decode_attention_noalloc_max_bytes(void) { return kStaticScratchBytes; }
+
+int vtkv_decode_attention_noalloc(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                                  const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
+                                  int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                                  const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                                  float v_scale, void *stream) {
+  VTKV_REQUIRE(seq_lens, "null argument");
+  void *scratch = static_scratch_ptr();
+  if (!scratch) return VTKV_EHIP;
+  return attention_impl(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, nullptr, num_seqs, num_heads, num_kv_heads,
+                        head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
+                        v_scale, scratch, kStaticScratchBytes, 0, stream, nullptr, nullptr, 0, 0, nullptr, true);
 }
 
 int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,

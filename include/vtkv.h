@@ -287,6 +287,23 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
                           float v_scale, void *workspace, int64_t workspace_bytes, int partition_tokens,
                           void *stream);
 
+/* vtkv_decode_attention without a workspace argument and without any allocation.  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory around the call, i.e. code under HIP graph
+ * capture, tight serving loops and harnesses that forbid hipMalloc.  The scratch (partial results, prefix sums,
+ * arrival counters) is an array of vtkv_decode_attention_noalloc_max_bytes() = 32 MiB of device memory that is
+ * part of the loaded library: every GPU the library runs on holds it until the process ends.  The call makes no
+ * hipMalloc / hipFree and calls no allocating library routine; it launches the same kernels as
+ * vtkv_decode_attention with partition_tokens = 0 and gives the same result bit for bit.  Sizes whose scratch
+ * does not fit (roughly num_seqs * num_heads above 45 000) are refused with VTKV_EINVAL.  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race on it and must
+ * be ordered by the caller; vtkv_set_kernel_timing does not apply to this entry point. */
+int64_t vtkv_decode_attention_noalloc_max_bytes(void);
+int vtkv_decode_attention_noalloc(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
+                                  const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
+                                  int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                                  const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
+                                  float v_scale, void *stream);
+
 /* The reference's split-K interface: paged_attention_v2 (csrc/attention/attention_kernels.cu:451-583 kernel and
  * reduce, :739-914 launcher; CPU twin csrc/cpu/attention.cpp:434-646; Python vllm/attention/ops/paged_attn.py:
  * 139-166).  Same result as vtkv_decode_attention; the rows of every sequence are cut into partitions of 512,
