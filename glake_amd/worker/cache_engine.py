@@ -104,16 +104,19 @@ class CacheEngine:
         self._swapped: Dict[int, Tuple[int, int]] = {}  # slot -> (arena offset, used bytes per range)
 
     # ------------------------------------------------------------------ swap (whole sequences)
-    def swap_out(self, slots: Sequence[int]) -> int:
+    def swap_out(self, slots: Sequence[int], keys: Optional[Sequence] = None) -> int:
         """Copy the used part of every K and V range of `slots` to pinned host memory on the current
-        stream, then unmap the slots (their chunks return to the pool).  Returns bytes moved."""
+        stream, then unmap the slots (their chunks return to the pool).  Returns bytes moved.
+        `keys` name the saved sequences (by default the slot numbers): with keys of its own a sequence can
+        come back into another slot while its old one serves someone else."""
         src, dst, nbytes = [], [], []
         total = 0
-        if len(set(slots)) != len(slots):
-            raise _C.VtkvError(_C.EINVAL, "swap_out: a slot is listed twice")
-        for slot in slots:
-            if slot in self._swapped:
-                raise _C.VtkvError(_C.ESTATE, f"slot {slot} is already swapped out")
+        keys = list(slots) if keys is None else list(keys)
+        if len(set(slots)) != len(slots) or len(keys) != len(slots) or len(set(keys)) != len(keys):
+            raise _C.VtkvError(_C.EINVAL, "swap_out: a slot or a key is listed twice, or keys and slots differ in number")
+        for key in keys:
+            if key in self._swapped:
+                raise _C.VtkvError(_C.ESTATE, f"sequence {key} is already swapped out")
         # room for all of them first: a full arena must leave every slot as it was
         placed: List[Tuple[int, int, int]] = []
         try:
@@ -125,9 +128,9 @@ class CacheEngine:
                 if used:
                     self._arena.release(off, 2 * self.num_layers * used)
             raise
-        for slot, off, used in placed:
+        for (slot, off, used), key in zip(placed, keys):
             seg = self.vmm_kvcache_segment[slot]
-            self._swapped[slot] = (off, used)
+            self._swapped[key] = (off, used)
             for l in range(self.num_layers):
                 for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):
                     if used:
@@ -142,14 +145,19 @@ class CacheEngine:
             self.vmm_kvcache_segment[slot].preempt_seq(slot)
         return total
 
-    def swap_in(self, slots: Sequence[int]) -> int:
-        """Map chunks for `slots` again and copy their KV back from host memory."""
-        src, dst, nbytes = [], [], []
+    def swap_in(self, slots: Sequence[int], keys: Optional[Sequence] = None) -> int:
+        """Map chunks for `slots` again and copy the KV saved under `keys` (by default the slot numbers) back
+        from host memory; a slot that receives another slot's sequence must hold no rows.
+        The copies of a slot are queued as soon as its chunks are mapped, so that they run while the host maps
+        the next slot's chunks (mapping a chunk takes longer than copying it)."""
         total = 0
-        for slot in slots:
-            if slot not in self._swapped:
-                raise _C.VtkvError(_C.ESTATE, f"slot {slot} is not swapped out")
-            off, used = self._swapped[slot]
+        keys = list(slots) if keys is None else list(keys)
+        if len(keys) != len(slots):
+            raise _C.VtkvError(_C.EINVAL, "swap_in: keys and slots differ in number")
+        for slot, key in zip(slots, keys):
+            if key not in self._swapped:
+                raise _C.VtkvError(_C.ESTATE, f"sequence {key} is not swapped out")
+            off, used = self._swapped[key]
             seg = self.vmm_kvcache_segment[slot]
             # the V rows start value_skew bytes into their range, so that much more must be mapped
             span = used + self.value_skew if used else 0
@@ -157,6 +165,7 @@ class CacheEngine:
             if need > 0:
                 seg.expandMultiSegment(need)
             seg.set_used_size(used)
+            src, dst, nbytes = [], [], []
             for l in range(self.num_layers):
                 for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):
                     if used:
@@ -164,10 +173,11 @@ class CacheEngine:
                         dst.append(base)
                         nbytes.append(used)
                         total += used
-        ops.swap_ranges(src, dst, nbytes, "in")
+            if src:
+                ops.swap_ranges(src, dst, nbytes, "in")
         torch.cuda.current_stream().synchronize()  # the arena space is reused after this
-        for slot in slots:
-            off, used = self._swapped.pop(slot)
+        for key in keys:
+            off, used = self._swapped.pop(key)
             if used:
                 self._arena.release(off, 2 * self.num_layers * used)
         return total

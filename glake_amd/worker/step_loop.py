@@ -1,0 +1,92 @@
+"""One serving step around the vTensor KV cache, as the reference's engine runs it
+(``vllm/engine/llm_engine.py:686-715`` ``LLMEngine.step`` and ``:565-625`` ``_process_model_outputs``,
+``vllm/worker/worker.py:213-225,284-304`` ``cache_swap`` / ``execute_model``, ``vllm/worker/model_runner.py:
+595-622,749-755`` metadata, ``vllm/model_executor/models/llama.py:307-351`` prologue and layers):
+
+1. ``StepScheduler.schedule()`` decides what runs;
+2. the slots of preempted sequences are unmapped (``preempt_seq``), swapped sequences move out or in;
+3. the attention metadata of the batch is built, ``prepare_step`` advances every scheduled sequence's range
+   (announcing the growth the scheduler foresaw to the map-ahead worker) and the caller's ``run_model`` runs the
+   layers through the attention backend;
+4. every scheduled sequence gets its sampled token accounted, and finished sequences release their slots
+   (``release_seq``).
+
+The model itself (projections, sampling) is not part of this package: ``run_model(metadata, outputs)`` is the
+caller's, and it calls ``VTensorImpl.forward`` once per layer with ``engine.gpu_cache[layer]``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, List, Optional
+
+import torch
+
+from ..attention.backends.vtensor import VTensorBackend, VTensorMetadata
+from ..core.scheduler import Request, SchedulerOutputs, StepScheduler
+from .cache_engine import CacheEngine
+from .step import prepare_step
+
+
+@dataclass
+class StepResult:
+    outputs: SchedulerOutputs
+    metadata: Optional[VTensorMetadata]   # None when nothing ran
+    finished: List[Request]
+
+
+class StepLoop:
+    def __init__(self, engine: CacheEngine, scheduler: StepScheduler, device: Optional[torch.device] = None):
+        self.engine = engine
+        self.scheduler = scheduler
+        self.device = torch.device("cuda", engine.device) if device is None else device
+
+    def build_metadata(self, out: SchedulerOutputs) -> VTensorMetadata:
+        """model_runner.py:595-622: prompts first, then decodes; per-sequence slot ids; ``extend_seq_list``
+        names, at its place in the batch, every sequence whose ranges grow in this step."""
+        eng, dev = self.engine, self.device
+        seqs = out.prompts + out.decodes
+        slots = [r.slot for r in seqs]
+        seq_lens = [r.total_len for r in seqs]
+        n_pre = len(out.prompts)
+        grow = set(out.extend_list)
+        meta = VTensorBackend.make_metadata(
+            num_prefills=n_pre, num_prefill_tokens=sum(seq_lens[:n_pre]), num_decode_tokens=len(out.decodes),
+            slot_mapping=torch.tensor(slots, dtype=torch.int64, device=dev), seq_lens=seq_lens,
+            seq_lens_tensor=torch.tensor(seq_lens, dtype=torch.int32, device=dev),
+            max_query_len=max(seq_lens[:n_pre]) if n_pre else None,
+            max_prefill_seq_len=max(seq_lens[:n_pre]) if n_pre else 0,
+            max_decode_seq_len=max(seq_lens[n_pre:]) if out.decodes else 0, query_start_loc=None, seq_start_loc=None,
+            context_lens_tensor=None, block_tables=None, is_extend=int(bool(grow)), kv_batch_stride=eng.kv_batch_stride,
+            kv_num_heads=eng.num_kv_heads, kv_head_size=eng.head_size, max_seq_len=max(seq_lens),
+            slot_mapping_list=slots, set_used_size=[0] * len(slots),
+            extend_seq_list=[s if s in grow else -1 for s in slots], use_cuda_graph=False)
+        meta.k_cache_segment_ptr_list = eng.k_cache_ptr          # model_runner.py:749-755
+        meta.v_cache_segment_ptr_list = eng.v_cache_ptr
+        meta.kvcache_segment = [eng.vmm_kvcache_segment[s] for s in slots]
+        return meta
+
+    def step(self, run_model: Callable[[VTensorMetadata, SchedulerOutputs], None]) -> StepResult:
+        eng = self.engine
+        out = self.scheduler.schedule()
+        stream = torch.cuda.current_stream(self.device)
+        if out.preempted_slot:                                            # llm_engine.py:700-701
+            # (the engine has read the last step's sampled tokens by now; a caller that queues steps without
+            # reading anything back must not lose chunks under kernels that are still running)
+            stream.synchronize()
+            for slot in out.preempted_slot:
+                eng.vmm_kvcache_segment[slot].preempt_seq(slot)
+        if out.swapped_out:                                               # worker.py:213-225
+            eng.swap_out([r.swap_slot for r in out.swapped_out], keys=[("req", r.request_id) for r in out.swapped_out])
+        if out.swapped_in:
+            eng.swap_in([r.slot for r in out.swapped_in], keys=[("req", r.request_id) for r in out.swapped_in])
+        meta = None
+        if out.prompts or out.decodes:
+            meta = self.build_metadata(out)
+            prepare_step(meta, eng.gpu_cache)                             # llama.py:307-341
+            run_model(meta, out)                                          # llama.py:343-351
+        finished = self.scheduler.on_step_done(out)
+        if finished:                                                      # llm_engine.py:607-618
+            stream.synchronize()                                          # the step's kernels have read the ranges
+            for req in finished:
+                eng.vmm_kvcache_segment[req.final_slot].release_seq(req.final_slot)
+        return StepResult(out, meta, finished)
