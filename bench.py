@@ -391,21 +391,25 @@ def main() -> int:
         engine.swap_out(swap_slots)  # untimed: first use of the pinned arena and of the copy streams
         engine.swap_in(swap_slots)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        moved = engine.swap_out(swap_slots)
-        t1 = time.perf_counter()
-        engine.swap_in(swap_slots)
-        t2 = time.perf_counter()
-        engine.swap_out(swap_slots)
-        t3 = time.perf_counter()
-        trimmed = vmm.trim()
-        t4 = time.perf_counter()
-        engine.swap_in(swap_slots)
-        t5 = time.perf_counter()
-        swap = {"bytes_per_direction": moved, "out_gbps": round(moved / (t1 - t0) / 1e9, 2),
-                "in_gbps": round(moved / (t2 - t1) / 1e9, 2), "in_cold_gbps": round(moved / (t5 - t4) / 1e9, 2),
-                "unmap_us_per_chunk": round((t4 - t3) / max(trimmed, 1) * 1e6, 1), "chunks": trimmed,
-                "sequences": nswap}
+        rounds = []
+        for _ in range(5):   # single transfers of a few milliseconds scatter: five rounds, the median of each figure
+            t0 = time.perf_counter()
+            moved = engine.swap_out(swap_slots)
+            t1 = time.perf_counter()
+            engine.swap_in(swap_slots)
+            t2 = time.perf_counter()
+            engine.swap_out(swap_slots)
+            t3 = time.perf_counter()
+            trimmed = vmm.trim()
+            t4 = time.perf_counter()
+            engine.swap_in(swap_slots)
+            t5 = time.perf_counter()
+            rounds.append((moved / (t1 - t0) / 1e9, moved / (t2 - t1) / 1e9, moved / (t5 - t4) / 1e9,
+                           (t4 - t3) / max(trimmed, 1) * 1e6))
+        med = [sorted(r[k] for r in rounds)[len(rounds) // 2] for k in range(4)]
+        swap = {"bytes_per_direction": moved, "out_gbps": round(med[0], 2), "in_gbps": round(med[1], 2),
+                "in_cold_gbps": round(med[2], 2), "unmap_us_per_chunk": round(med[3], 1), "chunks": trimmed,
+                "sequences": nswap, "rounds": len(rounds)}
 
     G = Hq // Hkv
     result = {

@@ -23,9 +23,7 @@ class PagedAttentionMetadata:
 class PagedAttention:
     @staticmethod
     def get_supported_head_sizes() -> List[int]:
-        # the reference lists [64, 80, 96, 112, 128, 256] (paged_attn.py:33-34); the HIP decode
-        # kernel is specialised for 128
-        return [128]
+        return [64, 80, 96, 112, 128, 256]  # paged_attn.py:33-34
 
     @staticmethod
     def get_kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int) -> Tuple[int, ...]:

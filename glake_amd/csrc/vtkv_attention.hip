@@ -107,6 +107,8 @@ struct AttnParams {
   int out_f32;
   int64_t q_stride;
   int num_seqs, num_heads, num_kv_heads, group;  // B, Hq, Hkv, G
+  int head_size;    // D as the caller's tensors have it (the kernels hold it padded to their tile sizes)
+  int out_f16;      // 16-bit outputs are fp16 (else bf16)
   int span_tiles;   // tiles per workgroup; 0 = all tiles / gridDim.x
   int grid;         // workgroups of the streaming kernel
   int xcd_spans;    // > 0: workgroup i takes span (i % 8) * xcd_spans + i / 8 (see the kernel)
@@ -159,17 +161,32 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // own at the end of the sequence's tile list, loaded from new_k / new_v, and the wave that handles it
 // also stores the row into the cache.  One launch then does reshape_and_cache and attention, and each
 // byte of the new rows is read once.
-template <bool ALIBI, bool FP8, bool APPEND, int HPS>
+//
+// D, F16: the head size (64, 80, 96, 112, 128 or 256) and whether q / K / V / out are fp16 instead of bf16.  The
+// kernel was shaped for D = 128 and bf16, where every constant below takes the value it always had; the other
+// sizes run the same code with fewer or more 16-byte pieces per row, MFMA steps and accumulator blocks.  A head
+// size that is no multiple of the MFMA depth is held padded (80 as 96, 112 as 128; with fp8 rows, whose pieces
+// carry 16 elements, 80, 96 and 112 as 128): the padding of the K and V tiles in LDS is cleared once and q is
+// zero there, so padded columns add nothing to the logits and yield output columns that are never stored.
+template <bool ALIBI, bool FP8, bool APPEND, int HPS, int D = 128, bool F16 = false>
 __global__ void __launch_bounds__(kThreads)
-    __attribute__((amdgpu_waves_per_eu(FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES)))
+    __attribute__((amdgpu_waves_per_eu(D > 128 ? 1 : (FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES))))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
+  static_assert(D % 16 == 0 && D >= 64 && D <= 256, "head sizes are multiples of 16 from 64 to 256");
+  static_assert(!APPEND || (D == 128 && !F16), "the fused append is built for bf16 rows of 128 only");
+  constexpr int kHD = FP8 ? (D + 63) / 64 * 64 : (D + 31) / 32 * 32;  // head size as held in LDS and registers
+  constexpr int kKSteps = kHD / 32;                                  // MFMA steps of S^T = K.Q^T
+  constexpr int kDBlocks = kHD / 16;                                 // 16-row blocks of O^T
+  constexpr int kPitch = kHD * 2 < 256 ? 256 : kHD * 2;              // bytes of a tile row in LDS (16-bit elements)
+  constexpr int kPitch8 = kHD < 128 ? 128 : kHD;                     // likewise for a K tile of fp8 codes
+  constexpr int kTileBytes = kTile * kPitch;
   // An fp8 tile is half the bytes of a bf16 tile for the same chain of dependent steps, so that variant
   // is bound by latency, not by HBM: it runs three waves per SIMD (it fits 168 registers with one
   // register tile per wave, refilled as soon as its contents have gone to LDS) instead of two.
   constexpr int kStages = FP8 ? kStagesFp8 : kStagesBf16;
   // wave-private V tiles (4 KiB each); reused at the end of a segment for the cross-wave merge
   // then the merge statistics (1 KiB) and the wave-private K tiles
-  __shared__ __attribute__((aligned(16))) char smem[2 * kWaves * kTile * kRowBytes + 1024];
+  __shared__ __attribute__((aligned(16))) char smem[2 * kWaves * kTileBytes + 1024];
   __shared__ int s_cum[kMaxSeqs + 1];  // s_cum[b] = tiles (of one kv head) of sequences before b
   __shared__ int s_wave_tot[kWaves];
   // pieces of shared (sequence, kv head) segments this workgroup has written: segment, first and last
@@ -291,11 +308,32 @@ __global__ void __launch_bounds__(kThreads)
 
   typedef const __attribute__((address_space(1))) char *gptr;
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
-  constexpr int kKvRowBytes = FP8 ? kD : kRowBytes;  // bytes of one head row in global memory
-  constexpr int kLoads = FP8 ? 2 : 4;                // 16-byte loads per lane for a K (or V) tile
+  constexpr int kKvRowBytes = FP8 ? D : 2 * D;       // bytes of one head row in global memory
+  constexpr int kPieces = kKvRowBytes / 16;          // 16-byte pieces of a head row
+  constexpr int kTilePieces = kTile * kPieces;       // ... of a 16-row tile, dealt to the lanes in order:
+  constexpr int kLoads = (kTilePieces + 63) / 64;    // load j of lane l takes piece 64 j + l, i.e. row (64 j + l) / kPieces
+  constexpr bool kEvenLoads = kTilePieces % 64 == 0; // every load of every lane carries a piece of the tile
+  constexpr int kKa = FP8 ? kHD / 64 : kKSteps;      // 16-byte A-operand pieces a lane reads back per K tile
   const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;  // bytes between consecutive tokens
-  char *v_tile = smem + wave * (kTile * kRowBytes);
-  char *k_tile = smem + kWaves * kTile * kRowBytes + 1024 + wave * (kTile * kRowBytes);
+  char *v_tile = smem + wave * kTileBytes;
+  char *k_tile = smem + kWaves * kTileBytes + 1024 + wave * kTileBytes;
+  // tile layouts in LDS (see vtkv_attn_common.h for the swizzles), with this head size's row pitch
+  auto v_off = [](int row, int piece16) { return row * kPitch + ((piece16 ^ ((row & 7) << 1)) << 4); };
+  auto k_off = [](int row, int piece16) {
+    return FP8 ? row * kPitch8 + ((piece16 ^ ((row >> 1) & 7)) << 4) : row * kPitch + ((piece16 ^ (row & 15)) << 4);
+  };
+  // where this lane's j-th load of a tile goes: (row, piece) of the tile, or nothing
+  auto load_row = [&](int j) { return (64 * j + lane) / kPieces; };
+  auto load_piece = [&](int j) { return (64 * j + lane) % kPieces; };
+  auto load_live = [&](int j) { return kEvenLoads || 64 * j + lane < kTilePieces; };
+  if constexpr ((FP8 ? kHD / 16 : kHD / 8) != kPieces) {
+    // padded head size: the pad pieces of both tiles are cleared once; no load ever writes them
+    constexpr int kPadK = (FP8 ? kHD / 16 : kHD / 8) - kPieces, kPadV = kHD / 8 - D / 8;
+    for (int i = lane; i < kTile * kPadK; i += 64)
+      *reinterpret_cast<u32x4 *>(k_tile + k_off(i / kPadK, kPieces + i % kPadK)) = (u32x4){0, 0, 0, 0};
+    for (int i = lane; i < kTile * kPadV; i += 64)
+      *reinterpret_cast<u32x4 *>(v_tile + v_off(i / kPadV, D / 8 + i % kPadV)) = (u32x4){0, 0, 0, 0};
+  }
 
   // ---- one segment = the part of the span that lies in one (sequence, kv head or pair of kv heads)
   while (g_cur < g_end) {
@@ -314,31 +352,32 @@ __global__ void __launch_bounds__(kThreads)
     gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
     gptr nk_base = k_base, nv_base = v_base;
     if (APPEND) {
-      nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kvh * kRowBytes;
-      nv_base = (gptr)(uintptr_t)p.new_v + (int64_t)b * p.new_v_stride + kvh * kRowBytes;
+      nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kvh * (2 * D);
+      nv_base = (gptr)(uintptr_t)p.new_v + (int64_t)b * p.new_v_stride + kvh * (2 * D);
     }
 
     // B operand of S^T = K.Q^T: for MFMA step ks lane (n, g) holds the eight q[head n][d] whose K
     // elements the lane's 16-byte K operand pieces hold: d = 32*ks + 8*g + j for bf16 rows; for fp8 rows one
     // load carries 16 elements, so steps 2c and 2c+1 take d = 64*c + 16*g + j and + 8.  Zero for
     // padded heads.
-    bf16x8 qop[4];
+    u32x4 qop[kKSteps];
     {
-      const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * kD;
+      const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * D;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
+      for (int ks = 0; ks < kKSteps; ++ks) {
         const int d0 = FP8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
-        u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + d0);
+        u32x4 raw = (u32x4){0, 0, 0, 0};
+        if (kHD == D || d0 < D) raw = *reinterpret_cast<const u32x4 *>(qrow + d0);  // (pieces are all in or all out)
         if (n >= G) raw = (u32x4){0, 0, 0, 0};
-        qop[ks] = __builtin_bit_cast(bf16x8, raw);
+        qop[ks] = raw;
       }
     }
     float slope_log2 = 0.f;
-    if (ALIBI) slope_log2 = n < G ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
+    if (ALIBI) slope_log2 = (n < G && p.alibi_slopes) ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
 
-    f32x4 acc[8];
+    f32x4 acc[kDBlocks];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < kDBlocks; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY;  // running max of scaled logits (log2 units) of head n
     float l_run = 0.f;        // this lane's share of the running sum
 
@@ -361,8 +400,9 @@ __global__ void __launch_bounds__(kThreads)
     for (int j = 0; j < kLoads; ++j) t_off_new[j] = FP8 ? ((lane & 7) * 2 + j) * 16 : n * 16;
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-      const int row = FP8 ? 8 * j + (lane >> 3) : 4 * j + g;
-      const int col = FP8 ? (lane & 7) * 16 : n * 16;
+      // (lanes past the end of the tile, where the head size leaves some, fetch its last row's first piece)
+      const int row = load_live(j) ? load_row(j) : kTile - 1;
+      const int col = load_live(j) ? load_piece(j) * 16 : 0;
       t_off[j] = (uint32_t)row * row_stride + col;
       t_off_last[j] = (uint32_t)min(row, valid_last - 1) * row_stride + col;
     }
@@ -438,39 +478,35 @@ __global__ void __launch_bounds__(kThreads)
       f32x4 s = {0.f, 0.f, 0.f, 0.f};
       // K tile through LDS: in as loaded, out as A operand (lane (n, g): row n, bytes [16g, +16) of
       // each 64-byte quarter)
-      u32x4 ka[kLoads];
+      u32x4 ka[kKa];
 #pragma unroll
-      for (int j = 0; j < kLoads; ++j) {
-        const int off = FP8 ? k8_lds_offset(8 * j + (lane >> 3), lane & 7) : k_lds_offset(4 * j + g, n);
-        *reinterpret_cast<u32x4 *>(k_tile + off) = kreg[j];
-      }
+      for (int j = 0; j < kLoads; ++j)
+        if (load_live(j)) *reinterpret_cast<u32x4 *>(k_tile + k_off(load_row(j), load_piece(j))) = kreg[j];
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 #pragma unroll
-      for (int c = 0; c < kLoads; ++c) {
-        const int off = FP8 ? k8_lds_offset(n, 4 * c + g) : k_lds_offset(n, 4 * c + g);
-        ka[c] = *reinterpret_cast<const u32x4 *>(k_tile + off);
-      }
+      for (int c = 0; c < kKa; ++c) ka[c] = *reinterpret_cast<const u32x4 *>(k_tile + k_off(n, 4 * c + g));
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       if (kStages == 1) load_k(i + 1, kreg);  // the K registers are free again: refill them
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
+      for (int ks = 0; ks < kKSteps; ++ks) {
         const u32x4 kop =
-            FP8 ? fp8x8_to_bf16x8(ka[ks >> 1][2 * (ks & 1)], ka[ks >> 1][2 * (ks & 1) + 1]) : ka[ks];
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kop), qop[ks], s, 0, 0, 0);
+            FP8 ? fp8x8_widen<F16>(ka[ks >> 1][2 * (ks & 1)], ka[ks >> 1][2 * (ks & 1) + 1]) : ka[ks];
+        s = mfma_16x16x32<F16>(kop, qop[ks], s);
       }
 
-      // stage V (as bf16) for the transposing read
+      // stage V (as 16-bit values) for the transposing read
       if constexpr (FP8) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int row = 8 * j + (lane >> 3), piece = 2 * (lane & 7);
-          *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece)) = fp8x8_to_bf16x8(vreg[j][0], vreg[j][1]);
-          *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(row, piece + 1)) = fp8x8_to_bf16x8(vreg[j][2], vreg[j][3]);
+        for (int j = 0; j < kLoads; ++j) {
+          if (!load_live(j)) continue;
+          const int row = load_row(j), piece = 2 * load_piece(j);
+          *reinterpret_cast<u32x4 *>(v_tile + v_off(row, piece)) = fp8x8_widen<F16>(vreg[j][0], vreg[j][1]);
+          *reinterpret_cast<u32x4 *>(v_tile + v_off(row, piece + 1)) = fp8x8_widen<F16>(vreg[j][2], vreg[j][3]);
         }
       } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          *reinterpret_cast<u32x4 *>(v_tile + v_lds_offset(4 * j + g, n)) = vreg[j];
+        for (int j = 0; j < kLoads; ++j)
+          if (load_live(j)) *reinterpret_cast<u32x4 *>(v_tile + v_off(load_row(j), load_piece(j))) = vreg[j];
       }
       if (kStages == 1) load_v(i + 1, vreg);  // likewise the V registers once they are in LDS
 
@@ -496,25 +532,24 @@ __global__ void __launch_bounds__(kThreads)
       l_run = l_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-        for (int d = 0; d < 8; ++d) acc[d] *= alpha;
+        for (int d = 0; d < kDBlocks; ++d) acc[d] *= alpha;
       }
       // P^T as B operand, split into a bf16 head and a bf16 tail so that P.V keeps ~16 mantissa bits of
       // P (the result then tracks an fp32-P reference, not just a bf16-P one).  Head and tail share one
       // K=32 MFMA: reduction slot (g, j) of v_mfma_f32_16x16x32_bf16 stands for row 4g+j with the head of
       // P for j < 4 and for row 4g+j-4 with the tail for j >= 4, so the B operand is [head(4), tail(4)]
       // straight from this lane's four logits and the A operand is the lane's V^T quad twice.
+      // (fp16 rows: head and tail are fp16, 22 bits of P between them; a tail below 2^-24 is lost, which is
+      // an absolute error of that size in a weight that is at most 1)
       float plo[4];
       u32x4 pb;
-      pb[0] = pack_bf16x2(pr[0], pr[1]);
-      pb[1] = pack_bf16x2(pr[2], pr[3]);
+      pb[0] = pack_16x2<F16>(pr[0], pr[1]);
+      pb[1] = pack_16x2<F16>(pr[2], pr[3]);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const unsigned hi_bits = (r & 1) ? (pb[r >> 1] & 0xffff0000u) : (pb[r >> 1] << 16);
-        plo[r] = pr[r] - __builtin_bit_cast(float, hi_bits);
-      }
-      pb[2] = pack_bf16x2(plo[0], plo[1]);
-      pb[3] = pack_bf16x2(plo[2], plo[3]);
-      const bf16x8 pop = __builtin_bit_cast(bf16x8, pb);
+      for (int r = 0; r < 4; ++r) plo[r] = pr[r] - unpack_16<F16>(pb[r >> 1], r & 1);
+      pb[2] = pack_16x2<F16>(plo[0], plo[1]);
+      pb[3] = pack_16x2<F16>(plo[2], plo[3]);
+      const u32x4 pop = pb;
 
       // O^T[d, head] += sum_row V[row, d] P[row, head], 16 d per MFMA.  LDS operations of one wave
       // execute in order, so the fences only pin the compiler's ordering of tile writes and reads.
@@ -522,14 +557,16 @@ __global__ void __launch_bounds__(kThreads)
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       {
         const int row = 4 * g + (n >> 2);
-        const int base = row * kRowBytes + ((n & 1) << 3);
+        const int base = row * kPitch + ((n & 1) << 3);
         const int swz = (row & 7) << 1;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          u32x4 vop[4];
+        for (int d0 = 0; d0 < kDBlocks; d0 += 4) {
+          constexpr int kGroup = 4;  // blocks whose reads are issued together (the last group may be shorter)
+          u32x4 vop[kGroup];
 #pragma unroll
-          for (int d4 = 0; d4 < 4; ++d4) {
-            const int db = 4 * half + d4;
+          for (int d4 = 0; d4 < kGroup; ++d4) {
+            const int db = d0 + d4;
+            if (db >= kDBlocks) break;
             const int off = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
             const s16x4 quad =
                 __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(v_tile + off));
@@ -537,9 +574,10 @@ __global__ void __launch_bounds__(kThreads)
             vop[d4] = (u32x4){qd[0], qd[1], qd[0], qd[1]};
           }
 #pragma unroll
-          for (int d4 = 0; d4 < 4; ++d4)
-            acc[4 * half + d4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[d4]), pop,
-                                                                         acc[4 * half + d4], 0, 0, 0);
+          for (int d4 = 0; d4 < kGroup; ++d4) {
+            if (d0 + d4 >= kDBlocks) break;
+            acc[d0 + d4] = mfma_16x16x32<F16>(vop[d4], pop, acc[d0 + d4]);
+          }
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -548,7 +586,7 @@ __global__ void __launch_bounds__(kThreads)
     // A ring of kStages register tiles per wave: while one tile is consumed the loads of the wave's next
     // kStages-1 tiles are in flight.  The steady-state path has no join after a load, only exits.
     if (my_tiles > 0) {
-      u32x4 kbuf[kStages][4], vbuf[kStages][4];
+      u32x4 kbuf[kStages][kLoads], vbuf[kStages][kLoads];
       if constexpr (kStages == 1) {
         // one register tile per wave, refilled inside consume() as soon as its contents have been used:
         // the loads of tile i+1 fly during the softmax and P.V of tile i at no extra register cost
@@ -582,9 +620,9 @@ __global__ void __launch_bounds__(kThreads)
     // ---- merge the waves of each head.  l_run is still split over the four row groups of a lane column.
     l_run = sum_over_row_groups(l_run);
     __syncthreads();  // every wave is done with its V tile: smem is free for the merge
-    float *sm_m = reinterpret_cast<float *>(smem + kWaves * kTile * kRowBytes);  // [4][16]
-    float *sm_l = sm_m + kWaves * 16;                                               // [4][16]
-    float *sm_o = reinterpret_cast<float *>(smem);                                  // [4][8][128] = 16 KiB
+    float *sm_m = reinterpret_cast<float *>(smem + kWaves * kTileBytes);  // [4][16]
+    float *sm_l = sm_m + kWaves * 16;                                        // [4][16]
+    float *sm_o = reinterpret_cast<float *>(smem);                           // [4][8][kHD]: at most the V tiles' size
     if (g == 0) {
       sm_m[wave * 16 + n] = m_run;
       sm_l[wave * 16 + n] = l_run;
@@ -607,28 +645,29 @@ __global__ void __launch_bounds__(kThreads)
     const int w0 = first_tile / span, w1 = (first_tile + nt_b - 1) / span;
     const bool whole = p.fused_merge && w0 == w1;  // no other workgroup: the result is final
     auto store_out = [&](int kv_head, int head, int d, float r) {
-      const int64_t oi = ((int64_t)b * p.num_heads + kv_head * G + head) * kD + d;
+      const int64_t oi = ((int64_t)b * p.num_heads + kv_head * G + head) * D + d;
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
-        reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
+        reinterpret_cast<uint16_t *>(p.out)[oi] = f32_to_16<F16>(r);
     };
     // G <= 8 fits the 16 KiB; for larger groups the merge runs in two halves of 8 heads
     for (int h0 = 0; h0 < G; h0 += 8) {
       if (h0 > 0) __syncthreads();
       if (n >= h0 && n < min(G, h0 + 8)) {
 #pragma unroll
-        for (int db = 0; db < 8; ++db)
+        for (int db = 0; db < kDBlocks; ++db)
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            sm_o[(wave * 8 + (n - h0)) * kD + db * 16 + 4 * g + i] = acc[db][i] * f;
+            sm_o[(wave * 8 + (n - h0)) * kHD + db * 16 + 4 * g + i] = acc[db][i] * f;
       }
       __syncthreads();
       const int nh = min(G, h0 + 8) - h0;
-      for (int idx = threadIdx.x; idx < kHps * nh * kD; idx += kThreads) {
-        const int sd = PAIR ? idx / (nh * kD) : 0;
-        const int rem = idx - sd * (nh * kD);
-        const int hh = rem / kD, d = rem % kD;
+      for (int idx = threadIdx.x; idx < kHps * nh * kHD; idx += kThreads) {
+        const int sd = PAIR ? idx / (nh * kHD) : 0;
+        const int rem = idx - sd * (nh * kHD);
+        const int hh = rem / kHD, d = rem % kHD;
+        if (kHD != D && d >= D) continue;  // a padded column
         const int head = h0 + hh;
         const int kv_head = kvg * kHps + sd;
         const float mw = head_max(sd, head);
@@ -637,14 +676,14 @@ __global__ void __launch_bounds__(kThreads)
         for (int j = 0; j < kWph; ++j) {
           const int w = sd + kHps * j;
           lsum += sm_l[w * 16 + head] * __builtin_amdgcn_exp2f(sm_m[w * 16 + head] - mw);
-          o += sm_o[(w * 8 + hh) * kD + d];
+          o += sm_o[(w * 8 + hh) * kHD + d];
         }
         const float o_norm = o / lsum;
         if (aligned && p.v2_tmp_out) {
           // the reference's per-partition outputs: max logit in natural units, sum of exponentials, and the
           // partition's normalised result in the model's dtype (csrc/attention/attention_kernels.cu:404-419)
           const int64_t vi = ((int64_t)b * p.num_heads + kv_head * G + head) * aligned + v2_part;
-          p.v2_tmp_out[vi * kD + d] = vtkv::f32_to_bf16_bits_rne(o_norm * p.v_scale);
+          p.v2_tmp_out[vi * D + d] = f32_to_16<F16>(o_norm * p.v_scale);
           if (d == 0) {
             p.v2_max_logits[vi] = mw * 0.6931471805599453f;
             p.v2_exp_sums[vi] = lsum;
@@ -658,13 +697,13 @@ __global__ void __launch_bounds__(kThreads)
         const int64_t seg_rank = head_major ? ((int64_t)kvg * B + b) * kHps + sd : (int64_t)b * Hkv + kv_head;
         const int64_t pidx = ((int64_t)kHps * wg + seg_rank) * G + head;
         if (p.fused_merge) {
-          store_device_coherent(&p.part_out[pidx * kD + d], o_norm);
+          store_device_coherent(&p.part_out[pidx * kHD + d], o_norm);
           if (d == 0) {
             store_device_coherent(&p.part_max[pidx], mw);
             store_device_coherent(&p.part_sum[pidx], lsum);
           }
         } else {
-          p.part_out[pidx * kD + d] = o_norm;
+          p.part_out[pidx * kHD + d] = o_norm;
           if (d == 0) {
             p.part_max[pidx] = mw;  // log2 units
             p.part_sum[pidx] = lsum;
@@ -738,11 +777,12 @@ __global__ void __launch_bounds__(kThreads)
       s_pend[k][3] = last_piece;
     }
     __syncthreads();
-    const int per_seg = G * kD;
+    const int per_seg = G * kHD;
     for (int idx = threadIdx.x; idx < np * per_seg; idx += kThreads) {
       const int j = idx / per_seg;
       if (!s_pend[j][3]) continue;
-      const int head = (idx - j * per_seg) / kD, d = idx % kD;
+      const int head = (idx - j * per_seg) / kHD, d = idx % kHD;
+      if (kHD != D && d >= D) continue;
       const int64_t seg = s_pend[j][0], seg_rank = s_pend[j][4];
       const int w0 = s_pend[j][1], w1 = s_pend[j][2];
       // four pieces at a time, all their loads in flight together; running (max, sum, out) across batches
@@ -754,7 +794,7 @@ __global__ void __launch_bounds__(kThreads)
           const int64_t pidx = ((int64_t)kHps * min(wb + jj, w1) + seg_rank) * G + head;
           pm[jj] = load_device_coherent(&p.part_max[pidx]);
           ps[jj] = load_device_coherent(&p.part_sum[pidx]);
-          po[jj] = load_device_coherent(&p.part_out[pidx * kD + d]);
+          po[jj] = load_device_coherent(&p.part_out[pidx * kHD + d]);
         }
         float bm = pm[0];
 #pragma unroll
@@ -773,11 +813,11 @@ __global__ void __launch_bounds__(kThreads)
       }
       const float r = o / wsum * p.v_scale;
       // segment = sequence * Hkv + kv head, so (segment * G + head) is (sequence * Hq + query head)
-      const int64_t oi = (seg * G + head) * kD + d;
+      const int64_t oi = (seg * G + head) * D + d;
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
-        reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
+        reinterpret_cast<uint16_t *>(p.out)[oi] = f32_to_16<F16>(r);
     }
   }
 }
@@ -794,9 +834,12 @@ __global__ void __launch_bounds__(kThreads)
 // of dependent round trips is GROUPS times shorter (config 3: 37 pieces per segment).
 // HSETS > 1 (only with GROUPS == 1, which has no barrier): HSETS sets of kD threads take the group's heads
 // four at a time in turn, so a group of eight heads is merged in one pass instead of two.
-template <int GROUPS, int HSETS>
-__global__ void __launch_bounds__(kD * GROUPS * HSETS) decode_attn_reduce_kernel(AttnParams p) {
+// HD: the head size as the stream kernel pads it (the row length of a partial result); thread d handles
+// column d and stores it if it is a real one (d < p.head_size).
+template <int GROUPS, int HSETS, int HD = 128>
+__global__ void __launch_bounds__(HD * GROUPS * HSETS) decode_attn_reduce_kernel(AttnParams p) {
   static_assert(GROUPS == 1 || HSETS == 1, "head sets only without piece groups");
+  constexpr int kD = HD;  // (shadows the library-wide 128 inside this kernel)
   const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x % kD;
   const int grp = GROUPS > 1 ? threadIdx.x / kD : 0, hset = HSETS > 1 ? threadIdx.x / kD : 0;
   __shared__ float sm_red[GROUPS > 1 ? 3 * GROUPS * 4 * kD : 1];
@@ -876,12 +919,13 @@ __global__ void __launch_bounds__(kD * GROUPS * HSETS) decode_attn_reduce_kernel
 #pragma unroll
     for (int hh = 0; hh < 4; ++hh) {
       if (h0 + hh >= G) break;
+      if (d >= p.head_size) break;  // a padded column
       const float r = o[hh] / wsum[hh] * p.v_scale;
-      const int64_t oi = ((int64_t)b * p.num_heads + kvh * G + h0 + hh) * kD + d;
+      const int64_t oi = ((int64_t)b * p.num_heads + kvh * G + h0 + hh) * p.head_size + d;
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
-        reinterpret_cast<uint16_t *>(p.out)[oi] = vtkv::f32_to_bf16_bits_rne(r);
+        reinterpret_cast<uint16_t *>(p.out)[oi] = p.out_f16 ? f32_to_16<true>(r) : f32_to_16<false>(r);
     }
   }
 }
@@ -940,7 +984,20 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16;  // instantiations of the streaming kernel
+constexpr int kVariants = 16 + 24;  // instantiations of the streaming kernel: 16 of the tuned shape, 24 others
+
+// 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
+int head_size_index(int head_size) {
+  switch (head_size) {
+    case 64: return 0;
+    case 80: return 1;
+    case 96: return 2;
+    case 112: return 3;
+    case 128: return 4;
+    case 256: return 5;
+    default: return -1;
+  }
+}
 struct Residency {
   std::mutex mu;
   int device = -1;
@@ -1018,10 +1075,13 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   VTKV_REQUIRE(num_seqs <= kMaxSeqs, "at most %d sequences per call, got %d", kMaxSeqs, num_seqs);
   VTKV_REQUIRE(!host_seq_lens || num_seqs <= kInlineLens, "at most %d sequence lengths can be passed from the host, got %d",
                kInlineLens, num_seqs);
-  VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
-  VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
-  VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
-  VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be BF16 or FP8_E4M3");
+  const int d_index = head_size_index(head_size);
+  VTKV_REQUIRE(d_index >= 0, "head_size %d is not supported (64, 80, 96, 112, 128, 256)", head_size);
+  VTKV_REQUIRE(q_dtype == VTKV_BF16 || q_dtype == VTKV_F16, "q_dtype must be BF16 or F16");
+  VTKV_REQUIRE(out_dtype == q_dtype || out_dtype == VTKV_F32, "out_dtype must be q_dtype or F32");
+  VTKV_REQUIRE(kv_dtype == q_dtype || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be q_dtype or FP8_E4M3");
+  const bool f16 = q_dtype == VTKV_F16;
+  const bool tuned = head_size == 128 && !f16;  // the shape the kernel was built around, with all its variants
   if (kv_dtype == VTKV_FP8_E4M3) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
   const int group = num_heads / num_kv_heads;
   VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
@@ -1036,7 +1096,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
                "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
   if (append) {
     VTKV_REQUIRE(new_value != nullptr, "null argument");
-    VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "the fused append needs a bf16 or fp8 cache");
+    VTKV_REQUIRE(tuned, "the fused append needs bf16 queries and head size 128");
     const int64_t row = (int64_t)num_kv_heads * head_size;
     VTKV_REQUIRE(key_stride >= row && value_stride >= row && key_stride % 8 == 0 && value_stride % 8 == 0 &&
                      (uintptr_t)new_key % 16 == 0 && (uintptr_t)new_value % 16 == 0,
@@ -1054,18 +1114,27 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   // num_seqs * num_kv_heads of `group` heads each, which the workspace (16 heads per workgroup) holds for
   // groups up to 8.
   const bool many_short = (int64_t)num_seqs * num_kv_heads >= 4096;
-  const bool pair = (fp8 ? VTKV_ATTN_FP8_PAIR != 0 : many_short) && num_kv_heads % 2 == 0 && group <= 8;
+  const bool pair = tuned && (fp8 ? VTKV_ATTN_FP8_PAIR != 0 : many_short) && num_kv_heads % 2 == 0 && group <= 8;
   const int seg_heads = pair ? 2 : 1;
-  // kernel variant: bit 0 alibi, bit 1 fused append, bit 2 paired kv heads, bit 3 fp8
-  const int variant = (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0);
+  // kernel variant of the tuned shape: bit 0 alibi, bit 1 fused append, bit 2 paired kv heads, bit 3 fp8; the
+  // other head sizes and fp16 have one variant per (head size, type, cache type), ALiBi decided at run time
+  const int variant = tuned ? (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0)
+                            : 16 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
 #define VTKV_ROW(F8, H)                                                                                      \
   decode_attn_stream_kernel<false, F8, false, H>, decode_attn_stream_kernel<true, F8, false, H>,             \
       decode_attn_stream_kernel<false, F8, true, H>, decode_attn_stream_kernel<true, F8, true, H>
+#define VTKV_SIZE(DD)                                                                                         \
+  decode_attn_stream_kernel<true, false, false, 1, DD, false>, decode_attn_stream_kernel<true, true, false, 1, DD, false>, \
+      decode_attn_stream_kernel<true, false, false, 1, DD, true>, decode_attn_stream_kernel<true, true, false, 1, DD, true>
   static void (*const kKernels[kVariants])(AttnParams, InlineLens) = {
       VTKV_ROW(false, 1), VTKV_ROW(false, 2), VTKV_ROW(true, 1), VTKV_ROW(true, 2),
+      VTKV_SIZE(64), VTKV_SIZE(80), VTKV_SIZE(96), VTKV_SIZE(112), VTKV_SIZE(128), VTKV_SIZE(256),
   };
 #undef VTKV_ROW
+#undef VTKV_SIZE
   void (*kernel)(AttnParams, InlineLens) = kKernels[variant];
+  // the head size as the kernels hold it: padded to the MFMA depth (to 64 elements for fp8 rows)
+  const int hd = fp8 ? (head_size + 63) / 64 * 64 : (head_size + 31) / 32 * 32;
   int64_t grid;
   if (v2) {
     grid = (int64_t)num_seqs * (num_kv_heads / seg_heads) * v2->max_parts;
@@ -1079,7 +1148,7 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
     if (g <= 0) return vtkv::fail(VTKV_EHIP, "cannot query the kernel's occupancy");
     grid = g;
   }
-  const int64_t n_float = scratch_floats(grid, num_seqs, num_heads, head_size);
+  const int64_t n_float = scratch_floats(grid, num_seqs, num_heads, hd);
   const int64_t count_bytes = counter_bytes(num_seqs, num_heads);
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
   const int64_t need = n_float * (int64_t)sizeof(float) + cum_bytes + count_bytes;
@@ -1125,10 +1194,12 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   p.heads_per_seg = seg_heads;
   p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
   p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);
-  p.part_max = p.part_out + n_stat * kD;
+  p.part_max = p.part_out + n_stat * hd;
   p.part_sum = p.part_max + n_stat;
   p.out = out;
   p.out_f32 = out_dtype == VTKV_F32;
+  p.out_f16 = f16;
+  p.head_size = head_size;
   p.q_stride = q_stride;
   p.num_seqs = num_seqs;
   p.num_heads = num_heads;
@@ -1187,12 +1258,23 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   if (timed) VTKV_HIP(hipEventRecord(ev[1], st));
   if (!p.fused_merge) {
     // segments of at least four pieces on average: four sets of threads share a segment's pieces
-    if (4 * segs <= grid)
-      hipLaunchKernelGGL((decode_attn_reduce_kernel<4, 1>), dim3(num_kv_heads, num_seqs), dim3(4 * kD), 0, st, p);
-    else if (group > 4)
-      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 2>), dim3(num_kv_heads, num_seqs), dim3(2 * kD), 0, st, p);
-    else
-      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 1>), dim3(num_kv_heads, num_seqs), dim3(kD), 0, st, p);
+    const dim3 rgrid(num_kv_heads, num_seqs);
+#define VTKV_REDUCE(HD)                                                                                       \
+  do {                                                                                                        \
+    if (4 * segs <= grid)                                                                                     \
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<4, 1, HD>), rgrid, dim3(4 * HD), 0, st, p);               \
+    else if (group > 4)                                                                                       \
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 2, HD>), rgrid, dim3(2 * HD), 0, st, p);               \
+    else                                                                                                      \
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 1, HD>), rgrid, dim3(HD), 0, st, p);                   \
+  } while (0)
+    switch (hd) {
+      case 64: VTKV_REDUCE(64); break;
+      case 96: VTKV_REDUCE(96); break;
+      case 256: VTKV_REDUCE(256); break;
+      default: VTKV_REDUCE(128); break;
+    }
+#undef VTKV_REDUCE
   }
   if (timed) {
     VTKV_HIP(hipEventRecord(ev[2], st));

@@ -89,6 +89,64 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(unsigned lo, unsigned hi) {
   return r;
 }
 
+// The same helpers for either 16-bit type of the model (F16 = false: bf16, true: fp16).
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+template <bool F16>
+__device__ __forceinline__ f32x4 mfma_16x16x32(u32x4 a, u32x4 b, f32x4 c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// two floats -> two 16-bit values in one dword (a in the low half), round to nearest even
+template <bool F16>
+__device__ __forceinline__ unsigned pack_16x2(float a, float b) {
+  if constexpr (F16) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    f16x2 v = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(unsigned, v);
+  } else {
+    return pack_bf16x2(a, b);
+  }
+}
+
+// the low (which = 0) or high half of such a dword as a float
+template <bool F16>
+__device__ __forceinline__ float unpack_16(unsigned pair, int which) {
+  if constexpr (F16) {
+    const unsigned short h = (unsigned short)(which ? pair >> 16 : pair & 0xffffu);
+    return (float)__builtin_bit_cast(_Float16, h);
+  } else {
+    return __builtin_bit_cast(float, which ? (pair & 0xffff0000u) : (pair << 16));
+  }
+}
+
+template <bool F16>
+__device__ __forceinline__ uint16_t f32_to_16(float r) {
+  if constexpr (F16)
+    return __builtin_bit_cast(unsigned short, (_Float16)r);  // v_cvt_f16_f32: round to nearest even
+  else
+    return vtkv::f32_to_bf16_bits_rne(r);
+}
+
+// eight e4m3fn codes -> eight fp16 values; exact (e4m3fn has 3 mantissa bits and exponents -9..8)
+__device__ __forceinline__ u32x4 fp8x8_to_f16x8(unsigned lo, unsigned hi) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  u32x4 r;
+  r[0] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false));
+  r[1] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true));
+  r[2] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false));
+  r[3] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true));
+  return r;
+}
+
+template <bool F16>
+__device__ __forceinline__ u32x4 fp8x8_widen(unsigned lo, unsigned hi) {
+  if constexpr (F16) return fp8x8_to_f16x8(lo, hi); else return fp8x8_to_bf16x8(lo, hi);
+}
+
 // Loads and stores that are coherent across the whole device (they go past the per-XCD L2), for the
 // few values that workgroups hand to each other inside one launch.  A device-scope fence would also
 // do, but it writes back and invalidates a whole L2 each time, which costs far more than these.

@@ -148,15 +148,18 @@ class CacheEngine:
     def swap_in(self, slots: Sequence[int], keys: Optional[Sequence] = None) -> int:
         """Map chunks for `slots` again and copy the KV saved under `keys` (by default the slot numbers) back
         from host memory; a slot that receives another slot's sequence must hold no rows.
-        The copies of a slot are queued as soon as its chunks are mapped, so that they run while the host maps
-        the next slot's chunks (mapping a chunk takes longer than copying it)."""
+        The slots are taken in batches of about 48 MiB: the copies of a batch are queued (one asynchronous
+        call) as soon as its chunks are mapped, and run while the host maps the next batch's chunks (mapping a
+        chunk takes longer than copying it, so a swap-in of unmapped sequences is bound by the mapping)."""
         total = 0
         keys = list(slots) if keys is None else list(keys)
         if len(keys) != len(slots):
             raise _C.VtkvError(_C.EINVAL, "swap_in: keys and slots differ in number")
-        for slot, key in zip(slots, keys):
+        for key in keys:
             if key not in self._swapped:
                 raise _C.VtkvError(_C.ESTATE, f"sequence {key} is not swapped out")
+        src, dst, nbytes, queued = [], [], [], 0
+        for slot, key in zip(slots, keys):
             off, used = self._swapped[key]
             seg = self.vmm_kvcache_segment[slot]
             # the V rows start value_skew bytes into their range, so that much more must be mapped
@@ -165,7 +168,6 @@ class CacheEngine:
             if need > 0:
                 seg.expandMultiSegment(need)
             seg.set_used_size(used)
-            src, dst, nbytes = [], [], []
             for l in range(self.num_layers):
                 for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):
                     if used:
@@ -173,8 +175,12 @@ class CacheEngine:
                         dst.append(base)
                         nbytes.append(used)
                         total += used
-            if src:
+                        queued += used
+            if queued >= 48 << 20:
                 ops.swap_ranges(src, dst, nbytes, "in")
+                src, dst, nbytes, queued = [], [], [], 0
+        if src:
+            ops.swap_ranges(src, dst, nbytes, "in")
         torch.cuda.current_stream().synchronize()  # the arena space is reused after this
         for key in keys:
             off, used = self._swapped.pop(key)

@@ -279,7 +279,9 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  *                > 0 (a multiple of 16, at least 64): every workgroup takes that many rows, the
  *                reference's fixed partitions (512 in paged_attention_v2, csrc/attention/attention_kernels.cu:739-914).
  *                The result does not depend on the choice beyond fp32 summation order.
- * Supported: q_dtype VTKV_BF16, kv_dtype VTKV_BF16 or VTKV_FP8_E4M3, head_size 128, num_heads/num_kv_heads in 1..16. */
+ * Supported: q_dtype VTKV_BF16 or VTKV_F16, kv_dtype = q_dtype or VTKV_FP8_E4M3, head_size 64, 80, 96, 112, 128 or
+ * 256 (the reference's list, vllm/attention/ops/paged_attn.py:33-34), num_heads/num_kv_heads in 1..16.  The kernel
+ * is tuned for bf16 and head size 128; the other shapes run the same code with their own tile constants. */
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                           const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,

@@ -21,6 +21,12 @@ ATTENTION_CASES = {
     "bf16_v2_gqa4": ("bf16", 2, 8, 2, False),
     "bf16_v1_gqa8": ("bf16", 1, 8, 1, False),
     "bf16_v2_alibi": ("bf16", 2, 8, 2, True),
+    # the other head sizes of the reference (vllm/attention/ops/paged_attn.py:33-34); a sixth field is the head size
+    "bf16_v1_d64": ("bf16", 1, 8, 2, False, 64),
+    "f32_v1_d80": ("f32", 1, 8, 2, False, 80),
+    "bf16_v2_d96": ("bf16", 2, 8, 1, False, 96),
+    "f32_v2_d112_alibi": ("f32", 2, 8, 2, True, 112),
+    "bf16_v1_d256": ("bf16", 1, 4, 4, False, 256),
 }
 
 
@@ -53,9 +59,9 @@ def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
 
 def attention_case(name: str):
     """Inputs of one attention case in the reference's paged layout (block 16)."""
-    dtype, version, hq, hkv, alibi = ATTENTION_CASES[name]
+    dtype, version, hq, hkv, alibi = ATTENTION_CASES[name][:5]
     seed = sum(ord(c) for c in name) * 1000
-    d, bs = HEAD_SIZE, BLOCK_SIZE
+    d, bs = (ATTENTION_CASES[name][5] if len(ATTENTION_CASES[name]) > 5 else HEAD_SIZE), BLOCK_SIZE
     x = 4 if dtype == "f32" else 8
     lens = np.array(LENS, np.int32)
     nblk = (lens + bs - 1) // bs

@@ -1,0 +1,132 @@
+"""Decode attention over the reference's whole surface of head sizes and 16-bit types
+(vllm/attention/ops/paged_attn.py:33-34 [64, 80, 96, 112, 128, 256]; tests/kernels/test_attention.py:23-31
+DTYPES half / bfloat16, NUM_HEADS (40, 40) and (64, 8), kv_cache_dtype auto / fp8, ALiBi), through the C ABI
+against the oracle.
+
+The oracle carries fp32 and bf16; an fp16 case is checked the way config 1 is: the oracle runs in fp32 on the
+very values the GPU gets (they are exact in fp32), and the comparison is made on the kernel's fp32 output, i.e.
+before the final rounding, at 2e-3 + 2e-3 |x| (fp8 caches: 3e-2 against the reference's protocol of dequantising
+to the model's type first, 2e-3 against exact dequantisation).  The 16-bit output must be the round-to-nearest
+of that fp32 output: numpy's float16 cast for fp16, the oracle's bf16 rounding for bf16."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+from kvharness import GpuSeqs, bits_from_torch_bf16
+
+pytestmark = pytest.mark.gpu
+
+HEAD_SIZES = [64, 80, 96, 112, 128, 256]
+LENS = [1, 15, 16, 17, 63, 64, 65, 257, 511, 512, 513, 1030, 2500]
+
+
+def to_model(x32, dtype):
+    """fp32 values -> (bits for upload, the same values in fp32)."""
+    if dtype == "f16":
+        h = x32.astype(np.float16)
+        return h, h.astype(np.float32)
+    b = O.f32_to_bf16(x32)
+    return b, O.bf16_to_f32(b)
+
+
+def run_case(vmm, seed, lens, hq, hkv, d, dtype, fp8=False, alibi=False, version="v1", partition_tokens=0):
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(seed)
+    b = len(lens)
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    k_scale = v_scale = 1.0
+    ks, vs, k32, v32, kref, vref = [], [], [], [], [], []
+    for n in lens:
+        kf = rng.standard_normal((n, hkv, d)).astype(np.float32)
+        vf = rng.standard_normal((n, hkv, d)).astype(np.float32)
+        ks.append(kf)
+        vs.append(vf)
+    if fp8:
+        k_scale = float(max(np.abs(x).max() for x in ks) / 448.0)
+        v_scale = float(max(np.abs(x).max() for x in vs) / 448.0)
+        ks = [O.fp8_encode(x, k_scale) for x in ks]
+        vs = [O.fp8_encode(x, v_scale) for x in vs]
+        k32, v32 = [O.fp8_decode(c, k_scale) for c in ks], [O.fp8_decode(c, v_scale) for c in vs]
+        # the reference's protocol: the cache converted back to the model's type (one more rounding)
+        kref = [to_model(x, dtype)[1] for x in k32]
+        vref = [to_model(x, dtype)[1] for x in v32]
+    else:
+        pairs_k, pairs_v = [to_model(x, dtype) for x in ks], [to_model(x, dtype) for x in vs]
+        ks, vs = [p[0] for p in pairs_k], [p[0] for p in pairs_v]
+        k32, v32 = [p[1] for p in pairs_k], [p[1] for p in pairs_v]
+    q_bits, q32 = to_model(rng.standard_normal((b, hq, d)).astype(np.float32), dtype)
+    scale = float(d) ** -0.5
+    slopes = (rng.standard_normal(hq) * 0.1).astype(np.float32) if alibi else None
+    gpu = GpuSeqs(vmm, b, hkv, d, 1 if fp8 else 2, max(lens), value_skew=256)
+    for i in range(b):
+        gpu.upload(i, ks[i], vs[i])
+    kt, vt = gpu.table_tensors()
+    q_t = torch.from_numpy(q_bits.view(np.int16).copy()).view(tdt).cuda()
+    sl = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    slots = torch.arange(b, dtype=torch.int64, device="cuda")
+    al = None if slopes is None else torch.from_numpy(slopes).cuda()
+    out32 = torch.empty(b, hq, d, dtype=torch.float32, device="cuda")
+    out16 = torch.empty(b, hq, d, dtype=tdt, device="cuda")
+    for o in (out32, out16):
+        if version == "v1":
+            ops.paged_attention_v1(o, q_t, kt, vt, hkv, scale, sl, 1, max(lens), al, "fp8" if fp8 else "auto", k_scale,
+                                   slots, v_scale=v_scale, partition_tokens=partition_tokens)
+        else:
+            parts = (max(lens) + 511) // 512
+            es = torch.zeros(b, hq, parts, dtype=torch.float32, device="cuda")
+            ml = torch.zeros_like(es)
+            tmp = torch.zeros(b, hq, parts, d, dtype=tdt, device="cuda")
+            ops.paged_attention_v2(o, es, ml, tmp, q_t, kt, vt, hkv, scale, sl, 1, max(lens), al,
+                                   "fp8" if fp8 else "auto", k_scale, slots, v_scale=v_scale)
+    torch.cuda.synchronize()
+    gpu.close()
+    got = out32.cpu().numpy()
+    assert np.isfinite(got).all()
+    want = O.paged_attention_v1(q32, O.VTensorCache(k32, v32, np.arange(b), hkv, d), scale, lens, slopes)
+    err = np.abs(got - want)
+    ok = bool(np.all(err <= 2e-3 + 2e-3 * np.abs(want)))
+    assert ok, f"max err {err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}"
+    if fp8:
+        want_ref = O.paged_attention_v1(q32, O.VTensorCache(kref, vref, np.arange(b), hkv, d), scale, lens, slopes)
+        assert bool(np.all(np.abs(got - want_ref) <= 3e-2 + 3e-2 * np.abs(want_ref)))
+    if dtype == "f16":
+        got16 = out16.cpu().numpy()
+        assert np.array_equal(got16.view(np.uint16), got.astype(np.float16).view(np.uint16)), "fp16 out is not RNE(fp32 out)"
+    else:
+        assert np.array_equal(bits_from_torch_bf16(out16), O.f32_to_bf16(got)), "bf16 out is not RNE(fp32 out)"
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("d", HEAD_SIZES)
+def test_every_head_size_gqa8(gpu_pool, d, dtype):
+    run_case(gpu_pool, d, LENS, 64, 8, d, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("d", HEAD_SIZES)
+def test_every_head_size_with_an_fp8_cache(gpu_pool, d, dtype):
+    run_case(gpu_pool, 100 + d, LENS, 32, 8, d, dtype, fp8=True)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("d", [64, 80, 128, 256])
+def test_forty_heads_without_grouping_and_alibi(gpu_pool, d, dtype):
+    # NUM_HEADS = (40, 40) of the reference's matrix: every query head has its own kv head
+    run_case(gpu_pool, 200 + d, [33, 700, 1, 2049, 130], 40, 40, d, dtype, alibi=True)
+
+
+@pytest.mark.parametrize("d,dtype,fp8", [(64, "f16", False), (80, "bf16", True), (96, "f16", True), (112, "bf16", False),
+                                         (256, "f16", False)])
+def test_split_k_interface_and_fixed_partitions_on_other_head_sizes(gpu_pool, d, dtype, fp8):
+    run_case(gpu_pool, 300 + d, [513, 2000, 100, 1025], 32, 8, d, dtype, fp8=fp8, version="v2")
+    run_case(gpu_pool, 400 + d, [513, 2000, 100, 1025], 32, 8, d, dtype, fp8=fp8, partition_tokens=256)
+
+
+def test_long_context_on_a_small_head_and_a_large_one(gpu_pool):
+    # many workgroups per (sequence, kv head): the merge of partial results of 64 and 256 columns
+    run_case(gpu_pool, 7, [40000, 9000], 32, 8, 64, "f16")
+    run_case(gpu_pool, 8, [30000, 100], 16, 4, 256, "bf16")
