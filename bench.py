@@ -219,7 +219,8 @@ def main() -> int:
     k_scale = v_scale = 6.0 / 448.0 if fp8 else 1.0
     for b in range(B):
         nbytes = ctx0[b] * row
-        segs[b].ensure_mapped(nbytes)  # counts the V offset
+        # (counts the V offset; the engine's accounting, which the backend path follows, maps 100 rows ahead)
+        segs[b].ensure_mapped(nbytes + (100 * row if backend_path else 0))
         for l in range(L):
             for base in (segs[b].getKeyDevicePtr(l), segs[b].getValueDevicePtr(l)):
                 t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -294,17 +295,33 @@ def main() -> int:
     impl = VTensorBackend.get_impl_cls()(Hq, D, scale, Hkv, None, None, kv_dtype)
     impl.fuse_decode_append = not args.unfused
     no_extend = [-1] * B
+    # the engine-side accounting claims every sequence's rows 100 ahead of what is written (sequence.py:343) and
+    # names the slots whose claim crosses a chunk in a step (block_manager_v1.py:436-455): prepare_step hands
+    # those to the map-ahead worker, so the chunk is there long before a row needs it
+    from glake_amd.core import ChunkSpaceManager, SequenceChunks
+    mgr = ChunkSpaceManager(B, 2 * B * chunks_per_range + 16, watermark=0.0)
+    claims = []
+    for b in range(B):
+        c = SequenceChunks(row, value_skew=args.value_skew)
+        c.append_tokens(ctx0[b])
+        assert mgr.allocate(c)
+        claims.append(c)
 
     def step_backend() -> int:
         lens = state["lens"] = [n + 1 for n in state["lens"]]
         max_len = max(lens)
+        grow = []
+        for c in claims:                                  # scheduler.py:1119-1150 _append_slots
+            c.append_tokens(1)
+            mgr.append_slots(c, grow)
+        extend = [s if s in grow else -1 for s in slot_ids] if grow else no_extend
         meta = VTensorBackend.make_metadata(
             num_prefills=0, num_prefill_tokens=0, num_decode_tokens=B, slot_mapping=slot_t, seq_lens=lens,
             seq_lens_tensor=torch.tensor(lens, dtype=torch.int32, device=dev), max_query_len=None,
             max_prefill_seq_len=0, max_decode_seq_len=max_len, query_start_loc=None, seq_start_loc=None,
             context_lens_tensor=None, block_tables=None, is_extend=0, kv_batch_stride=engine.kv_batch_stride,
             kv_num_heads=Hkv, kv_head_size=D, max_seq_len=max_len, slot_mapping_list=slot_ids, set_used_size=zeros,
-            extend_seq_list=no_extend, use_cuda_graph=False)
+            extend_seq_list=extend, use_cuda_graph=False)
         meta.k_cache_segment_ptr_list = engine.k_cache_ptr          # model_runner.py:749-755
         meta.v_cache_segment_ptr_list = engine.v_cache_ptr
         meta.kvcache_segment = segs

@@ -183,9 +183,10 @@ def decode_append_attention(
         _ptr(ws), ws.numel(), int(partition_tokens), _stream()))
 
 
-def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], per_unit: int):
+def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], per_unit: int, order: str = "sequence"):
     """Cut each sequence's query tokens into runs of up to ``per_unit`` consecutive tokens: int32 rows
-    [sequence index, first query row, tokens, position of the first token], longest context first."""
+    [sequence index, first query row, tokens, position of the first token]; ``order`` is "sequence"
+    (sequence by sequence, longest context first inside each) or "rows" (longest context first over the batch)."""
     import numpy as np
 
     parts, row = [], 0
@@ -203,8 +204,16 @@ def prefill_units(query_lens: Sequence[int], seq_lens: Sequence[int], per_unit: 
     if not parts:
         return np.empty((0, 4), np.int32)
     units = np.concatenate(parts)
-    order = np.argsort(-(units[:, 2] + units[:, 3]), kind="stable")  # most rows first: the tail stays short
-    return np.ascontiguousarray(units[order])
+    if order == "rows":
+        idx = np.argsort(-(units[:, 2] + units[:, 3]), kind="stable")   # most rows first over the whole batch
+    else:
+        # Sequence by sequence, most rows first inside a sequence.  The workgroups that run at the same time then
+        # read the rows of one or two sequences, which stay in the L2 of the XCD that serves their kv head: with
+        # the batch-wide order the kernel fetched every row three times over (8 prompts of 2048 tokens: 618 MB
+        # against 201 MB), with this one once (201.5 MB); the time is the same, the rows came from the last-level
+        # cache either way.  The short units of the last sequence still close the launch.
+        idx = np.lexsort((-(units[:, 2] + units[:, 3]), units[:, 0]))
+    return np.ascontiguousarray(units[idx])
 
 
 def prefill_attention(

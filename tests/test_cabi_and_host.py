@@ -132,7 +132,7 @@ def test_bench_refuses_more_than_one_gpu():
 def test_prefill_units_cover_every_query_token_once():
     """Host logic of the prompt attention: the unit table (sequence, first query row, tokens, position of
     the first token) covers each packed query row exactly once, keeps units inside one sequence, respects
-    the per-unit limit, places chunk queries at the end of their sequence and lists longest contexts first."""
+    the per-unit limit, places chunk queries at the end of their sequence and lists the units in the documented order."""
     import numpy as np
 
     from glake_amd._custom_ops import prefill_units
@@ -148,8 +148,14 @@ def test_prefill_units_cover_every_query_token_once():
             assert starts[b] <= row0 and row0 + ntok <= starts[b + 1]                 # inside its sequence
             assert pos0 == seq_lens[b] - query_lens[b] + (row0 - starts[b])           # lower-right aligned
         assert (seen == 1).all()
-        reach = u[:, 2] + u[:, 3]
-        assert (np.diff(reach) <= 0).all()
+        # sequence by sequence, the longest context first inside each; "rows": longest first over the batch
+        assert (np.diff(u[:, 0]) >= 0).all()
+        for b in set(u[:, 0].tolist()):
+            own = u[u[:, 0] == b]
+            assert (np.diff(own[:, 2] + own[:, 3]) <= 0).all()
+        by_rows = prefill_units(query_lens, seq_lens, per_unit, order="rows")
+        assert (np.diff(by_rows[:, 2] + by_rows[:, 3]) <= 0).all()
+        assert sorted(map(tuple, by_rows.tolist())) == sorted(map(tuple, u.tolist()))
     assert prefill_units([], [], 4).shape == (0, 4)
     import pytest
 

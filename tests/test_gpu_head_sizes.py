@@ -130,3 +130,37 @@ def test_long_context_on_a_small_head_and_a_large_one(gpu_pool):
     # many workgroups per (sequence, kv head): the merge of partial results of 64 and 256 columns
     run_case(gpu_pool, 7, [40000, 9000], 32, 8, 64, "f16")
     run_case(gpu_pool, 8, [30000, 100], 16, 4, 256, "bf16")
+
+
+@pytest.mark.parametrize("d,dtype", [(64, "f16"), (80, "bf16"), (128, "f16"), (256, "bf16")])
+def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype):
+    """The prompt kernel is built for bf16 and head size 128; every other shape runs a prompt as one decode step
+    per query token.  Plain prompts and prompts behind cached rows, against the prompt oracle."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+    from glake_amd.attention.backends.vtensor import VTensorBackend
+
+    VTensorBackend.get_impl_cls()(32, d, d ** -0.5, 8, None, None, "auto")     # the backend takes the head size
+    rng = np.random.default_rng(d)
+    hq, hkv = 32, 8
+    seq_lens, query_lens = [700, 33, 1, 1300], [700, 20, 1, 400]
+    b = len(seq_lens)
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    pairs_k = [to_model(rng.standard_normal((n, hkv, d)).astype(np.float32), dtype) for n in seq_lens]
+    pairs_v = [to_model(rng.standard_normal((n, hkv, d)).astype(np.float32), dtype) for n in seq_lens]
+    n_tok = sum(query_lens)
+    q_bits, q32 = to_model(rng.standard_normal((n_tok, hq, d)).astype(np.float32), dtype)
+    gpu = GpuSeqs(gpu_pool, b, hkv, d, 2, max(seq_lens), value_skew=256)
+    for i in range(b):
+        gpu.upload(i, pairs_k[i][0], pairs_v[i][0])
+    kt, vt = gpu.table_tensors()
+    out = torch.empty(n_tok, hq, d, dtype=torch.float32, device="cuda")
+    ops.prefill_attention(out, torch.from_numpy(q_bits.view(np.int16).copy()).view(tdt).cuda(), kt, vt, hkv, d ** -0.5,
+                          query_lens, seq_lens, torch.arange(b, dtype=torch.int64, device="cuda"))
+    torch.cuda.synchronize()
+    gpu.close()
+    want = O.prefill_attention(q32, O.VTensorCache([p[1] for p in pairs_k], [p[1] for p in pairs_v], np.arange(b), hkv, d),
+                               d ** -0.5, query_lens, seq_lens)
+    err = np.abs(out.cpu().numpy() - want)
+    assert bool(np.all(err <= 2e-3 + 2e-3 * np.abs(want))), f"max err {err.max():.3e}"
