@@ -15,8 +15,11 @@
 //    LDS and the softmax weights are rounded to fp16 (2^-12 relative per weight, 16 times finer than the
 //    bf16 weights of flash-attention kernels; the decode kernel's bf16 head + tail is finer still but costs
 //    twice the P.V MFMAs).  bf16 V values convert exactly for magnitudes in [2^-24, 65504]; smaller ones
-//    lose low bits (absolute error below 2^-25), larger ones saturate at 65504.  Softmax statistics live in
-//    registers, each lane applies its column's causal limit to the logits of the stages that reach it.
+//    lose low bits (absolute error below 2^-25); a larger one becomes infinity, the workgroup finds its
+//    result non-finite at the end and computes the unit a second time with V kept in bf16 and the decode
+//    kernel's bf16 head + tail of P, so prompt and decode attention agree for every bf16 input.  Softmax
+//    statistics live in registers, each lane applies its column's causal limit to the logits of the stages
+//    that reach it.
 //  * The kv head is the fastest index of the grid: with 8 kv heads the workgroups of one kv head all land
 //    on one XCD, whose L2 then serves the re-reads of that head's rows by later query blocks.
 //
@@ -64,12 +67,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-// Two floats to two fp16 in one register.  Round toward zero: a value beyond the fp16 range becomes the
-// largest finite fp16 instead of infinity.
-__device__ __forceinline__ unsigned pack_f16x2_sat(float a, float b) {
-  return __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-// Round to nearest (for the softmax weights, which lie in [0, 256]).
+// Two floats to two fp16 in one register, round to nearest; a value beyond the fp16 range becomes infinity.
 __device__ __forceinline__ unsigned pack_f16x2(float a, float b) {
   f16x2 v = {(_Float16)a, (_Float16)b};
   return __builtin_bit_cast(unsigned, v);
@@ -99,12 +97,13 @@ __device__ __forceinline__ float wave_max_over_row_groups(float v) {
   return fmax2(a, b);
 }
 // Eight bf16 values (one 16-byte piece of a V row) to eight fp16 values.  Exact for magnitudes in
-// [2^-24, 65504]; larger ones saturate.
+// [2^-24, 65504]; a larger one becomes infinity, which makes the unit's result non-finite: the kernel sees that
+// at the end and computes the unit again with V kept in bf16 (see WIDE).
 __device__ __forceinline__ u32x4 bf16x8_to_f16x8(u32x4 v) {
   u32x4 r;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
-    r[i] = pack_f16x2_sat(__builtin_bit_cast(float, v[i] << 16), __builtin_bit_cast(float, v[i] & 0xffff0000u));
+    r[i] = pack_f16x2(__builtin_bit_cast(float, v[i] << 16), __builtin_bit_cast(float, v[i] & 0xffff0000u));
   return r;
 }
 // Eight e4m3fn codes (two dwords) to eight fp16 values; exact.
@@ -170,13 +169,16 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
 
   f32x4 acc[kNB][8];
   float m_run[kNB], l_run[kNB];
+  auto reset = [&]() {
 #pragma unroll
-  for (int nb = 0; nb < kNB; ++nb) {
-    m_run[nb] = -INFINITY;
-    l_run[nb] = 0.f;
+    for (int nb = 0; nb < kNB; ++nb) {
+      m_run[nb] = -INFINITY;
+      l_run[nb] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[nb][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  }
+      for (int i = 0; i < 8; ++i) acc[nb][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  reset();
 
   // ---- cooperative stage loads of a block of kKeyBlock rows.  bf16 rows: thread t takes piece t%16 of
   // rows t/16 + 16j.  fp8 rows have 8 pieces of 16 codes: thread t takes piece t%8 of rows t/8 + 32j and
@@ -189,8 +191,11 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   const uint32_t last_off = (uint32_t)(kv_len - 1) * row_stride + ld_piece * 16;
   const uint32_t stage_step = kKeyBlock * row_stride;
   uint32_t ld_off[kLd];
+  auto rewind = [&]() {
 #pragma unroll
-  for (int j = 0; j < kLd; ++j) ld_off[j] = (uint32_t)(j * (kKeyBlock / kLd) + ld_row) * row_stride + ld_piece * 16;
+    for (int j = 0; j < kLd; ++j) ld_off[j] = (uint32_t)(j * (kKeyBlock / kLd) + ld_row) * row_stride + ld_piece * 16;
+  };
+  rewind();
   u32x4 kst[kLd], vst[kLd];
   auto gload = [&]() {  // loads the next stage's rows and moves on
 #pragma unroll
@@ -214,7 +219,10 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
       st_v[j] = kKeyBlock * kRowBytes + j * kTile * kRowBytes + v_lds_offset(ld_row, ld_piece);
     }
   }
-  auto lstore = [&](auto bufc) {
+  // WIDE (bf16 rows only): V stays bf16 in LDS and P.V runs on the bf16 MFMA with P as a bf16 head plus a bf16
+  // tail, the decode kernel's arithmetic: twice the P.V MFMAs, no limit on |V|.  Used for a unit's second pass.
+  auto lstore = [&](auto bufc, auto widec) {
+    constexpr bool WIDE = decltype(widec)::value;
     char *base = smem + decltype(bufc)::value * kStageBytes;
 #pragma unroll
     for (int j = 0; j < kLd; ++j) {
@@ -226,7 +234,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
         *reinterpret_cast<u32x4 *>(base + (st_v[j] ^ 16)) = fp8x8_to_f16x8(vst[j][2], vst[j][3]);
       } else {
         *reinterpret_cast<u32x4 *>(base + st_k[j]) = kst[j];
-        *reinterpret_cast<u32x4 *>(base + st_v[j]) = bf16x8_to_f16x8(vst[j]);
+        *reinterpret_cast<u32x4 *>(base + st_v[j]) = WIDE ? vst[j] : bf16x8_to_f16x8(vst[j]);
       }
     }
   };
@@ -251,8 +259,9 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   // scale is applied inside the exponent's fused multiply-add.
   const float lazy = ALIBI ? 8.f : 8.f / sl;
 
-  auto stage = [&](auto bufc, int kb) {
+  auto stage = [&](auto bufc, auto widec, int kb) {
     constexpr int buf = decltype(bufc)::value;
+    constexpr bool WIDE = decltype(widec)::value;
     gload();  // always issued: past the last stage it re-reads the last row and nobody uses it
     const char *st = smem + buf * kStageBytes;
     const int t0 = kb * kKeyBlock;
@@ -336,31 +345,73 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
         }
         // P^T as fp16 (11 significant bits: the rounding stays below 2^-12 relative, which a bf16 P would
         // miss by a factor 16); the normaliser sums the same rounded weights
-        u32x4 pb;
+        if constexpr (WIDE) {
+          u32x4 ph, pt;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) pb[r] = pack_f16x2(pr[2 * r], pr[2 * r + 1]);
-        float l = l_run[nb];
+          for (int r = 0; r < 4; ++r) {
+            ph[r] = pack_bf16x2(pr[2 * r], pr[2 * r + 1]);
+            pt[r] = pack_bf16x2(pr[2 * r] - __builtin_bit_cast(float, ph[r] << 16),
+                                pr[2 * r + 1] - __builtin_bit_cast(float, ph[r] & 0xffff0000u));
+          }
+          float l = l_run[nb];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) l = add_f16x2(pb[r], l);
-        l_run[nb] = l;
-        const f16x8 pop = __builtin_bit_cast(f16x8, pb);
+          for (int r = 0; r < 8; ++r) l += pr[r];
+          l_run[nb] = l;
 #pragma unroll
-        for (int db = 0; db < 8; ++db)
-          acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, vop[db]), pop, acc[nb][db], 0, 0,
-                                                               0);
+          for (int db = 0; db < 8; ++db) {
+            acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[db]),
+                                                                  __builtin_bit_cast(bf16x8, ph), acc[nb][db], 0, 0, 0);
+            acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[db]),
+                                                                  __builtin_bit_cast(bf16x8, pt), acc[nb][db], 0, 0, 0);
+          }
+        } else {
+          u32x4 pb;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) pb[r] = pack_f16x2(pr[2 * r], pr[2 * r + 1]);
+          float l = l_run[nb];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) l = add_f16x2(pb[r], l);
+          l_run[nb] = l;
+          const f16x8 pop = __builtin_bit_cast(f16x8, pb);
+#pragma unroll
+          for (int db = 0; db < 8; ++db)
+            acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, vop[db]), pop, acc[nb][db], 0,
+                                                                 0, 0);
+        }
       }
     }
     // the other stage: its readers finished before the last barrier
-    lstore(std::integral_constant<int, buf ^ 1>{});
+    lstore(std::integral_constant<int, buf ^ 1>{}, widec);
     __syncthreads();
   };
 
-  gload();
-  lstore(std::integral_constant<int, 0>{});
-  __syncthreads();
-  for (int kb = 0; kb < nblocks; kb += 2) {
-    stage(std::integral_constant<int, 0>{}, kb);
-    if (kb + 1 < nblocks) stage(std::integral_constant<int, 1>{}, kb + 1);
+  auto run = [&](auto widec) {
+    gload();
+    lstore(std::integral_constant<int, 0>{}, widec);
+    __syncthreads();
+    for (int kb = 0; kb < nblocks; kb += 2) {
+      stage(std::integral_constant<int, 0>{}, widec, kb);
+      if (kb + 1 < nblocks) stage(std::integral_constant<int, 1>{}, widec, kb + 1);
+    }
+  };
+  run(std::false_type{});
+  if constexpr (!FP8) {
+    // A V value beyond the fp16 range went into LDS as infinity and has made some accumulator of the workgroup
+    // infinite or NaN (a weight of exactly zero gives NaN).  Then the whole unit is computed again with V in
+    // bf16; e4m3fn codes always fit fp16.  Inputs that are themselves non-finite take the second pass too and
+    // come out non-finite again.
+    unsigned expo = 0;
+#pragma unroll
+    for (int nb = 0; nb < kNB; ++nb)
+#pragma unroll
+      for (int db = 0; db < 8; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) expo = max(expo, __builtin_bit_cast(unsigned, acc[nb][db][i]) & 0x7f800000u);
+    if (__syncthreads_or(expo == 0x7f800000u)) {
+      reset();
+      rewind();
+      run(std::true_type{});
+    }
   }
 
   // ---- normalise and store: lane (n, g) holds O[column n][d = 16*db + 4g + i]

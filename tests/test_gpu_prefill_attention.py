@@ -191,9 +191,11 @@ def test_logit_peaks_move_the_reference_point_mid_sequence(gpu_pool):
     run_case(gpu_pool, 8, [400], [400], 16, 8, alibi=True, shape_inputs=peaks)
 
 
-def test_large_values_stay_finite(gpu_pool):
-    """V travels as fp16 inside the prompt kernel: values up to 6e4 are exact to bf16 precision there, and
-    a value beyond the fp16 range saturates at 65504 instead of becoming infinite."""
+def test_values_beyond_the_fp16_range(gpu_pool):
+    """V travels as fp16 inside the prompt kernel; a bf16 cache can hold values fp16 cannot.  Values up to 6e4
+    stay on the fast path; a unit that meets a larger one is computed a second time with V in bf16, so the
+    prompt kernel agrees with the oracle (and with decode) for every bf16 input: huge values in a few rows, in
+    all rows, next to ordinary ones whose weights they must not disturb, and behind masked positions."""
     import torch
 
     from glake_amd import _custom_ops as ops
@@ -204,7 +206,22 @@ def test_large_values_stay_finite(gpu_pool):
 
     run_case(gpu_pool, 9, [70, 33], [70, 33 + 64], 32, 8, shape_inputs=clip, out_scale=1.5e4)
 
-    # one key, value 1e5: the output is the saturated value
+    def a_few_huge(q, ks, vs):
+        # rows 5 and 300 of the first sequence and the last row of the second hold values around 1e8 and -3e20
+        vs[0][5] = O.f32_to_bf16(np.full(vs[0][5].shape, 1.0e8, np.float32))
+        vs[0][300, :, ::2] = O.f32_to_bf16(np.float32(-3.0e20))
+        vs[1][-1] = O.f32_to_bf16(np.full(vs[1][-1].shape, 7.0e4, np.float32))
+
+    # (the tolerance scales with the magnitude of V: 2e-3 relative to the largest value that enters an output)
+    run_case(gpu_pool, 12, [400, 90, 64], [400, 90 + 40, 64], 32, 8, shape_inputs=a_few_huge, out_scale=3.0e20)
+
+    def all_huge(q, ks, vs):
+        for v in vs:
+            v[...] = O.f32_to_bf16(O.bf16_to_f32(v) * np.float32(1.0e9))
+
+    run_case(gpu_pool, 13, [130, 17], [130, 17 + 200], 16, 8, shape_inputs=all_huge, out_scale=1.0e9, fp8=False)
+
+    # one key, value 1e5: the output is that value, bit for bit
     rng = np.random.default_rng(10)
     hq, hkv = 8, 8
     gpu = GpuSeqs(gpu_pool, 1, hkv, d := 128, 2, 1)
@@ -216,6 +233,31 @@ def test_large_values_stay_finite(gpu_pool):
                           torch.zeros(1, dtype=torch.int64, device="cuda"))
     torch.cuda.synchronize()
     gpu.close()
-    # (round toward zero lands on the largest finite fp16)
-    assert torch.all(out == 65504.0)
+    assert np.array_equal(out.cpu().numpy().reshape(hq, d), np.repeat(O.bf16_to_f32(v[0]), hq // hkv, axis=0))
 
+
+def test_prompt_and_decode_agree_on_huge_values(gpu_pool):
+    """The same rows through the prompt kernel (last position) and through the decode kernel: both keep V in
+    bf16 where it matters, so they differ by fp32 summation order only."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(14)
+    hq, hkv, d, n = 32, 8, 128, 777
+    k = bf16_randn(rng, (n, hkv, d))
+    v = O.f32_to_bf16(rng.standard_normal((n, hkv, d)).astype(np.float32) * np.float32(2.0e6))
+    gpu = GpuSeqs(gpu_pool, 1, hkv, d, 2, n)
+    gpu.upload(0, k, v)
+    kt, vt = gpu.table_tensors()
+    q = torch_bf16_from_bits(bf16_randn(rng, (n, hq, d)))
+    slots = torch.zeros(1, dtype=torch.int64, device="cuda")
+    out_p = torch.empty(n, hq, d, dtype=torch.float32, device="cuda")
+    ops.prefill_attention(out_p, q, kt, vt, hkv, d ** -0.5, [n], [n], slots)
+    out_d = torch.empty(1, hq, d, dtype=torch.float32, device="cuda")
+    ops.paged_attention_v1(out_d, q[n - 1:], kt, vt, hkv, d ** -0.5, torch.tensor([n], dtype=torch.int32, device="cuda"), 1, n,
+                           None, "auto", 1.0, slots)
+    torch.cuda.synchronize()
+    gpu.close()
+    a, b = out_p[n - 1].cpu().numpy(), out_d[0].cpu().numpy()
+    assert np.isfinite(a).all() and np.all(np.abs(a - b) <= 1e-4 * 2.0e6 + 1e-4 * np.abs(b))
