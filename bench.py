@@ -61,6 +61,9 @@ CONFIGS = {
     # configs[4] without its swap events: 256 sequences
     "c5": dict(name="growth-bf16 B=256 Hq=32 Hkv=8 D=128 ctx~U[256,2048]", batch=256, hq=32, hkv=8, d=128, lo=256,
                hi=2048, seed=1004, kv="bf16"),
+    # outside BASELINE.json: very many short sequences (every workgroup meets many segment starts and ends)
+    "t1k": dict(name="many-short-bf16 B=1024 Hq=32 Hkv=8 D=128 ctx~U[64,512]", batch=1024, hq=32, hkv=8, d=128, lo=64,
+                hi=512, seed=1007, kv="bf16"),
     # outside BASELINE.json: a prompt run (cache write + causal attention over the ranges), 8 prompts of 2048
     "p2k": dict(name="llama3-8b-prompt-run-bf16 B=8 Hq=32 Hkv=8 D=128 prompt=2048", batch=8, hq=32, hkv=8, d=128,
                 lo=2048, hi=2048, seed=1006, kv="bf16", prefill=True),

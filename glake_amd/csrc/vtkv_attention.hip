@@ -1295,7 +1295,8 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
                            ? fixed_span_grid(num_seqs, num_heads, max_seq_len + kTile, partition_tokens)
                            : kDefaultMaxGrid;
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
-  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes +
+  // (the kernels hold a head size padded to 32 elements, to 64 for fp8 rows: sized for the larger)
+  return scratch_floats(grid, num_seqs, num_heads, (head_size + 63) / 64 * 64) * (int64_t)sizeof(float) + cum_bytes +
          counter_bytes(num_seqs, num_heads);
 }
 
@@ -1315,7 +1316,8 @@ int64_t vtkv_decode_attention_v2_workspace_bytes(int num_seqs, int num_heads, in
   if (num_seqs <= 0 || num_heads <= 0 || head_size <= 0 || max_num_partitions <= 0) return 0;
   const int64_t grid = (int64_t)num_seqs * num_heads * max_num_partitions;  // at most one workgroup per head
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
-  return scratch_floats(grid, num_seqs, num_heads, head_size) * (int64_t)sizeof(float) + cum_bytes +
+  // (the kernels hold a head size padded to 32 elements, to 64 for fp8 rows: sized for the larger)
+  return scratch_floats(grid, num_seqs, num_heads, (head_size + 63) / 64 * 64) * (int64_t)sizeof(float) + cum_bytes +
          counter_bytes(num_seqs, num_heads);
 }
 

@@ -164,3 +164,11 @@ def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype):
                                d ** -0.5, query_lens, seq_lens)
     err = np.abs(out.cpu().numpy() - want)
     assert bool(np.all(err <= 2e-3 + 2e-3 * np.abs(want))), f"max err {err.max():.3e}"
+
+
+def test_workspace_is_sized_for_the_padded_head_size(gpu_pool):
+    """A head size of 112 is held as 128 (fp8 rows pad to 64 elements): the workspace the library asks for must
+    be sized for that, also through the split-K interface, where the grid and with it the scratch is exact."""
+    run_case(gpu_pool, 964028853, [9, 4, 4, 10, 11, 6, 4, 10, 6, 5, 4261], 8, 8, 112, "f16", fp8=True, version="v2")
+    run_case(gpu_pool, 5, [100, 3000, 17], 8, 8, 80, "bf16", fp8=True, version="v2")
+    run_case(gpu_pool, 6, [100, 3000, 17], 16, 16, 80, "bf16", partition_tokens=64)

@@ -93,3 +93,39 @@ def test_random_sweep_fp8_decode(gpu_pool, seed):
     finally:
         _C.check(lib.vtkv_set_fused_merge(-1))
         _C.check(lib.vtkv_set_head_major(-1))
+
+
+@pytest.mark.parametrize("seed", [606, 707])
+def test_random_sweep_over_head_sizes_and_types(gpu_pool, seed):
+    """The same sweep over the other head sizes (64, 80, 96, 112, 256, and 128 in fp16), fp16 and bf16, plain and
+    fp8 caches, the plain entry point with stream-K or fixed partitions and the split-K interface."""
+    import test_gpu_head_sizes as H
+    from glake_amd import _C
+
+    lib = _C.lib()
+    rng = np.random.default_rng(seed)
+    try:
+        for case in range(40):
+            hq, hkv = HEADS[rng.integers(len(HEADS))]
+            d = int(rng.choice(H.HEAD_SIZES))
+            dtype = "f16" if (d == 128 or rng.integers(2)) else "bf16"
+            b = int(rng.integers(1, 16))
+            kind = rng.integers(3)
+            if kind == 0:
+                lens = rng.integers(1, 40, b)
+            elif kind == 1:
+                lens = rng.integers(1, 900, b)
+            else:
+                lens = np.concatenate([rng.integers(1, 20, b), rng.integers(2000, 5000, 1)])
+            lens = [int(x) for x in lens]
+            fp8, alibi = bool(rng.integers(3) == 0), bool(rng.integers(4) == 0)
+            version = "v2" if rng.integers(4) == 0 else "v1"
+            pt = int(rng.choice([0, 0, 64, 256, 512])) if version == "v1" else 0
+            merge = int(rng.integers(-1, 2))
+            sub = int(rng.integers(1 << 30))
+            _C.check(lib.vtkv_set_fused_merge(merge))
+            print(f"case {case}: seed {sub} heads {hq}/{hkv} d {d} {dtype} fp8 {fp8} lens {lens} {version} partition {pt} "
+                  f"alibi {alibi} merge {merge}", flush=True)
+            H.run_case(gpu_pool, sub, lens, hq, hkv, d, dtype, fp8=fp8, alibi=alibi, version=version, partition_tokens=pt)
+    finally:
+        _C.check(lib.vtkv_set_fused_merge(-1))
