@@ -49,6 +49,8 @@
 #include <mutex>
 #include <vector>
 
+#include <hip/hip_ext.h>
+
 #include "vtkv_common.h"
 #ifndef VTKV_ATTN_STAGES
 // Register tiles per wave of the bf16 variants.  One (the next tile's K loads are issued as soon as the K
@@ -972,13 +974,17 @@ void *static_scratch_ptr() {
 }
 
 // Optional per-kernel timing for benchmarks: when switched on, every vtkv_decode_attention call
-// records events around its two launches on the caller's stream, without waiting for them, so the
-// calls stay queued back to back as they are in production.  Up to kTimedCalls calls are kept.
+// launches its kernels with a start and a stop event each (hipExtLaunchKernelGGL: the events take the
+// begin and the end of that kernel's own dispatch on the caller's stream, which is what a kernel trace
+// reports; events recorded before and after a launch also contain the dispatch of the kernel and the
+// completion of the event markers, 5 to 6 us here).  Nothing waits for them, so the calls stay queued
+// back to back as they are in production.  Up to kTimedCalls calls are kept.
 constexpr int kTimedCalls = 1024;
 struct KernelTimer {
   std::atomic<bool> on{false};
   std::mutex mu;               // held by a timed call from its first event to its last, and by the readers
-  std::vector<hipEvent_t> ev;  // three per call, created on first use
+  std::vector<hipEvent_t> ev;  // four per call (start and stop of either kernel), created on first use
+  std::vector<char> merged;    // per call: the merge ran inside the streaming kernel (no second kernel)
   int calls = 0;
 };
 KernelTimer g_timer;
@@ -1246,27 +1252,35 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
   const bool timed = timer_lock.owns_lock() && g_timer.on.load(std::memory_order_relaxed) && g_timer.calls < kTimedCalls;
   hipEvent_t *ev = nullptr;
   if (timed) {
-    if ((int)g_timer.ev.size() < 3 * (g_timer.calls + 1)) {
-      hipEvent_t e3[3];
-      for (auto &e : e3) VTKV_HIP(hipEventCreate(&e));
-      g_timer.ev.insert(g_timer.ev.end(), e3, e3 + 3);
+    if ((int)g_timer.ev.size() < 4 * (g_timer.calls + 1)) {
+      hipEvent_t e4[4];
+      for (auto &e : e4) VTKV_HIP(hipEventCreate(&e));
+      g_timer.ev.insert(g_timer.ev.end(), e4, e4 + 4);
     }
-    ev = &g_timer.ev[3 * g_timer.calls];
-    VTKV_HIP(hipEventRecord(ev[0], st));
+    ev = &g_timer.ev[4 * g_timer.calls];
+    hipExtLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, ev[0], ev[1], 0, p, il);
+  } else {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, p, il);
   }
-  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, p, il);
-  if (timed) VTKV_HIP(hipEventRecord(ev[1], st));
   if (!p.fused_merge) {
     // segments of at least four pieces on average: four sets of threads share a segment's pieces
     const dim3 rgrid(num_kv_heads, num_seqs);
+#define VTKV_REDUCE_LAUNCH(G, S, HD)                                                                          \
+  do {                                                                                                        \
+    if (timed)                                                                                                \
+      hipExtLaunchKernelGGL((decode_attn_reduce_kernel<G, S, HD>), rgrid, dim3(G * S * HD), 0, st, ev[2],     \
+                            ev[3], 0, p);                                                                     \
+    else                                                                                                      \
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<G, S, HD>), rgrid, dim3(G * S * HD), 0, st, p);           \
+  } while (0)
 #define VTKV_REDUCE(HD)                                                                                       \
   do {                                                                                                        \
     if (4 * segs <= grid)                                                                                     \
-      hipLaunchKernelGGL((decode_attn_reduce_kernel<4, 1, HD>), rgrid, dim3(4 * HD), 0, st, p);               \
+      VTKV_REDUCE_LAUNCH(4, 1, HD);                                                                           \
     else if (group > 4)                                                                                       \
-      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 2, HD>), rgrid, dim3(2 * HD), 0, st, p);               \
+      VTKV_REDUCE_LAUNCH(1, 2, HD);                                                                           \
     else                                                                                                      \
-      hipLaunchKernelGGL((decode_attn_reduce_kernel<1, 1, HD>), rgrid, dim3(HD), 0, st, p);                   \
+      VTKV_REDUCE_LAUNCH(1, 1, HD);                                                                           \
   } while (0)
     switch (hd) {
       case 64: VTKV_REDUCE(64); break;
@@ -1275,9 +1289,11 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
       default: VTKV_REDUCE(128); break;
     }
 #undef VTKV_REDUCE
+#undef VTKV_REDUCE_LAUNCH
   }
   if (timed) {
-    VTKV_HIP(hipEventRecord(ev[2], st));
+    g_timer.merged.resize(g_timer.calls + 1);
+    g_timer.merged[g_timer.calls] = p.fused_merge != 0;
     ++g_timer.calls;
   }
   VTKV_HIP(hipGetLastError());
@@ -1385,10 +1401,14 @@ int vtkv_attention_kernel_times(float *stream_ms, float *reduce_ms, int capacity
   std::lock_guard<std::mutex> lk(g_timer.mu);
   const int n = std::min(capacity, g_timer.calls);
   for (int i = 0; i < n; ++i) {
-    hipEvent_t *ev = &g_timer.ev[3 * i];
-    VTKV_HIP(hipEventSynchronize(ev[2]));
+    hipEvent_t *ev = &g_timer.ev[4 * i];
+    VTKV_HIP(hipEventSynchronize(ev[1]));
     VTKV_HIP(hipEventElapsedTime(&stream_ms[i], ev[0], ev[1]));
-    VTKV_HIP(hipEventElapsedTime(&reduce_ms[i], ev[1], ev[2]));
+    reduce_ms[i] = 0.f;
+    if (!g_timer.merged[i]) {
+      VTKV_HIP(hipEventSynchronize(ev[3]));
+      VTKV_HIP(hipEventElapsedTime(&reduce_ms[i], ev[2], ev[3]));
+    }
   }
   return n;
 }

@@ -148,9 +148,11 @@ class CacheEngine:
     def swap_in(self, slots: Sequence[int], keys: Optional[Sequence] = None) -> int:
         """Map chunks for `slots` again and copy the KV saved under `keys` (by default the slot numbers) back
         from host memory; a slot that receives another slot's sequence must hold no rows.
-        The slots are taken in batches of about 48 MiB: the copies of a batch are queued (one asynchronous
-        call) as soon as its chunks are mapped, and run while the host maps the next batch's chunks (mapping a
-        chunk takes longer than copying it, so a swap-in of unmapped sequences is bound by the mapping)."""
+        All chunks are mapped first and the copies queued after that in one call: this runtime's mapping calls
+        wait for copies in flight (mapping 166 chunks takes 7 ms alone and 11.7 ms when a 4.7 ms copy was
+        queued just before), so mapping and copying do not overlap and a swap-in of unmapped sequences costs
+        the sum of the two (mapping in steps with the copies queued in between measured 3 to 15 % slower than
+        this order on the same machine)."""
         total = 0
         keys = list(slots) if keys is None else list(keys)
         if len(keys) != len(slots):
@@ -158,27 +160,20 @@ class CacheEngine:
         for key in keys:
             if key not in self._swapped:
                 raise _C.VtkvError(_C.ESTATE, f"sequence {key} is not swapped out")
-        src, dst, nbytes, queued = [], [], [], 0
+        src, dst, nbytes = [], [], []
         for slot, key in zip(slots, keys):
             off, used = self._swapped[key]
             seg = self.vmm_kvcache_segment[slot]
-            # the V rows start value_skew bytes into their range, so that much more must be mapped
-            span = used + self.value_skew if used else 0
-            need = (span + self.chunk_bytes - 1) // self.chunk_bytes - seg.actual_size // self.chunk_bytes
-            if need > 0:
-                seg.expandMultiSegment(need)
+            seg.ensure_mapped(used)
             seg.set_used_size(used)
+            if not used:
+                continue
             for l in range(self.num_layers):
                 for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):
-                    if used:
-                        src.append(self._arena.base + off + (2 * l + which) * used)
-                        dst.append(base)
-                        nbytes.append(used)
-                        total += used
-                        queued += used
-            if queued >= 48 << 20:
-                ops.swap_ranges(src, dst, nbytes, "in")
-                src, dst, nbytes, queued = [], [], [], 0
+                    src.append(self._arena.base + off + (2 * l + which) * used)
+                    dst.append(base)
+                    nbytes.append(used)
+                    total += used
         if src:
             ops.swap_ranges(src, dst, nbytes, "in")
         torch.cuda.current_stream().synchronize()  # the arena space is reused after this

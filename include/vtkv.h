@@ -384,10 +384,12 @@ int vtkv_set_head_major(int on);
 
 /* Benchmark aid without a counterpart in the reference (its kernel benchmark times from the host,
  * benchmarks/kernels/benchmark_paged_attention.py:147-157): while switched on, each vtkv_decode_attention
- * call (up to 1024 of them) records HIP events around its kernels on the caller's stream without waiting
- * for them.  vtkv_attention_kernel_times waits for the recorded calls and writes, for the first
+ * call (up to 1024 of them) launches its kernels with a start and a stop HIP event each on the caller's
+ * stream (the begin and the end of that kernel's own dispatch, as a kernel trace reports them) without
+ * waiting for them.  vtkv_attention_kernel_times waits for the recorded calls and writes, for the first
  * min(capacity, calls) of them in call order, the duration of the streaming kernel and of the merge
- * kernel in milliseconds; it returns that count.  Switching timing on again starts a new series. */
+ * kernel in milliseconds (0 where the merge ran inside the streaming kernel); it returns that count.
+ * Switching timing on again starts a new series. */
 int vtkv_set_kernel_timing(int on);
 int vtkv_attention_kernel_times(float *stream_ms, float *reduce_ms, int capacity);
 
