@@ -1057,15 +1057,15 @@ struct V2Side {
 };
 constexpr int kV2Partition = 512;  // rows per partition (vllm/attention/ops/paged_attn.py:10)
 
-// Shared by the entry points.  new_key == nullptr: attention only.  v2 != nullptr: partitions of 512 rows
-// aligned with the sequences, the caller's side buffers filled.
-int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
+// One batch of at most kMaxSeqs sequences (kInlineLens with host lengths).  new_key == nullptr: attention only.
+// v2 != nullptr: partitions of 512 rows aligned with the sequences, the caller's side buffers filled.
+int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
                    const int32_t *seq_lens, const int32_t *host_seq_lens, int num_seqs, int num_heads,
                    int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
                    const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale, float v_scale,
                    void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream, const void *new_key,
-                   const void *new_value, int64_t key_stride, int64_t value_stride, const V2Side *v2 = nullptr,
-                   bool static_scratch = false) {
+                   const void *new_value, int64_t key_stride, int64_t value_stride, const V2Side *v2,
+                   bool static_scratch) {
   const bool append = new_key != nullptr;
   if (v2) {
     partition_tokens = kV2Partition;
@@ -1297,6 +1297,46 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
     ++g_timer.calls;
   }
   VTKV_HIP(hipGetLastError());
+  return VTKV_OK;
+}
+
+// Shared by the entry points: larger batches run as consecutive batches of kMaxSeqs sequences (kInlineLens
+// when the lengths come from the host) on the caller's stream; rows of different sequences are independent and
+// the scratch of a batch is free again when the next one starts on the same stream.
+int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
+                   const int32_t *seq_lens, const int32_t *host_seq_lens, int num_seqs, int num_heads,
+                   int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                   const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale, float v_scale,
+                   void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream, const void *new_key,
+                   const void *new_value, int64_t key_stride, int64_t value_stride, const V2Side *v2 = nullptr,
+                   bool static_scratch = false) {
+  const int per_call = host_seq_lens ? kInlineLens : kMaxSeqs;
+  if (num_seqs <= per_call || !out || !q || !slot_ids || num_heads <= 0 || head_size <= 0)
+    return attention_batch(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, host_seq_lens, num_seqs, num_heads, num_kv_heads,
+                           head_size, q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale,
+                           v_scale, workspace, workspace_bytes, partition_tokens, stream, new_key, new_value, key_stride,
+                           value_stride, v2, static_scratch);
+  const int64_t out_row = (int64_t)num_heads * head_size * (out_dtype == VTKV_F32 ? 4 : 2);
+  for (int at = 0; at < num_seqs; at += per_call) {
+    const int n = std::min(per_call, num_seqs - at);
+    V2Side side;
+    if (v2) {
+      const int64_t rows = (int64_t)at * num_heads * v2->max_parts;
+      side = *v2;
+      if (side.exp_sums) side.exp_sums += rows;
+      if (side.max_logits) side.max_logits += rows;
+      if (side.tmp_out) side.tmp_out = (char *)side.tmp_out + rows * head_size * 2;
+    }
+    int rc = attention_batch((char *)out + at * out_row, (const char *)q + (int64_t)at * q_stride * 2, k_ptrs, v_ptrs,
+                             slot_ids + at, seq_lens ? seq_lens + at : nullptr,
+                             host_seq_lens ? host_seq_lens + at : nullptr, n, num_heads, num_kv_heads, head_size,
+                             q_stride, scale, max_seq_len, alibi_slopes, q_dtype, out_dtype, kv_dtype, k_scale, v_scale,
+                             workspace, workspace_bytes, partition_tokens, stream,
+                             new_key ? (const char *)new_key + (int64_t)at * key_stride * 2 : nullptr,
+                             new_value ? (const char *)new_value + (int64_t)at * value_stride * 2 : nullptr, key_stride,
+                             value_stride, v2 ? &side : nullptr, static_scratch);
+    if (rc < 0) return rc;
+  }
   return VTKV_OK;
 }
 

@@ -101,6 +101,8 @@ class CacheEngine:
             self.v_cache_ptr.append(torch.tensor([s.getValueDevicePtr(l) for s in self.vmm_kvcache_segment],
                                                  dtype=torch.long, device=dev))
         self._arena = _HostArena(swap_space_bytes)
+        self.swap_in_map_bytes = 32 << 20     # swap_in maps this much of every range, queues its copies, maps on
+        self.swap_in_flush_bytes = 64 << 20   # ... and hands the queued copies over when they add up to this
         self._swapped: Dict[int, Tuple[int, int]] = {}  # slot -> (arena offset, used bytes per range)
 
     # ------------------------------------------------------------------ swap (whole sequences)
@@ -148,11 +150,13 @@ class CacheEngine:
     def swap_in(self, slots: Sequence[int], keys: Optional[Sequence] = None) -> int:
         """Map chunks for `slots` again and copy the KV saved under `keys` (by default the slot numbers) back
         from host memory; a slot that receives another slot's sequence must hold no rows.
-        All chunks are mapped first and the copies queued after that in one call: this runtime's mapping calls
-        wait for copies in flight (mapping 166 chunks takes 7 ms alone and 11.7 ms when a 4.7 ms copy was
-        queued just before), so mapping and copying do not overlap and a swap-in of unmapped sequences costs
-        the sum of the two (mapping in steps with the copies queued in between measured 3 to 15 % slower than
-        this order on the same machine)."""
+        Mapping and copying take turns on the host and overlap on the device: the ranges are mapped
+        ``swap_in_map_bytes`` at a time, and the copies into what is mapped are handed over (one asynchronous
+        call) whenever ``swap_in_flush_bytes`` are queued, so they run while the host maps on.  Mapping a chunk
+        takes about as long as copying it (42 us against 38 us), so a swap-in of unmapped sequences stays bound
+        by the mapping: 32 to 34 GB/s for one 347 MB sequence against 27 GB/s with everything mapped first.
+        The overlap needs the current stream to be a non-blocking one: this runtime's mapping calls wait for
+        everything queued on the null stream, the copies included, and the two then run one after the other."""
         total = 0
         keys = list(slots) if keys is None else list(keys)
         if len(keys) != len(slots):
@@ -160,20 +164,41 @@ class CacheEngine:
         for key in keys:
             if key not in self._swapped:
                 raise _C.VtkvError(_C.ESTATE, f"sequence {key} is not swapped out")
-        src, dst, nbytes = [], [], []
+        src, dst, nbytes, queued = [], [], [], 0
+        step = max(1, self.swap_in_map_bytes // self.chunk_bytes)   # chunks per range mapped between two rounds of copies
         for slot, key in zip(slots, keys):
             off, used = self._swapped[key]
             seg = self.vmm_kvcache_segment[slot]
-            seg.ensure_mapped(used)
-            seg.set_used_size(used)
             if not used:
+                seg.set_used_size(0)
                 continue
-            for l in range(self.num_layers):
-                for which, base in ((0, seg.getKeyDevicePtr(l)), (1, seg.getValueDevicePtr(l))):
-                    src.append(self._arena.base + off + (2 * l + which) * used)
-                    dst.append(base)
-                    nbytes.append(used)
-                    total += used
+            # the V rows start value_skew bytes into their range, so that much more must be mapped
+            need = (used + self.value_skew + self.chunk_bytes - 1) // self.chunk_bytes
+            mapped = seg.actual_size // self.chunk_bytes
+            ptrs = [(seg.getKeyDevicePtr(l), seg.getValueDevicePtr(l)) for l in range(self.num_layers)]
+            done_k = done_v = 0
+            while True:
+                if mapped < need:
+                    grow = min(step, need - mapped)
+                    seg.expandMultiSegment(grow)
+                    mapped += grow
+                ready_k = min(used, mapped * self.chunk_bytes)
+                ready_v = min(used, max(0, mapped * self.chunk_bytes - self.value_skew))
+                for l, (kp, vp) in enumerate(ptrs):
+                    for which, base, lo, hi in ((0, kp, done_k, ready_k), (1, vp, done_v, ready_v)):
+                        if hi > lo:
+                            src.append(self._arena.base + off + (2 * l + which) * used + lo)
+                            dst.append(base + lo)
+                            nbytes.append(hi - lo)
+                            total += hi - lo
+                            queued += hi - lo
+                done_k, done_v = ready_k, ready_v
+                if queued >= self.swap_in_flush_bytes:
+                    ops.swap_ranges(src, dst, nbytes, "in")
+                    src, dst, nbytes, queued = [], [], [], 0
+                if mapped >= need:
+                    break
+            seg.set_used_size(used)
         if src:
             ops.swap_ranges(src, dst, nbytes, "in")
         torch.cuda.current_stream().synchronize()  # the arena space is reused after this

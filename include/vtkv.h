@@ -279,6 +279,8 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  *                > 0 (a multiple of 16, at least 64): every workgroup takes that many rows, the
  *                reference's fixed partitions (512 in paged_attention_v2, csrc/attention/attention_kernels.cu:739-914).
  *                The result does not depend on the choice beyond fp32 summation order.
+ * A launch takes up to 1024 sequences; a larger batch runs as consecutive launches of 1024 on `stream` within
+ * the one call.
  * Supported: q_dtype VTKV_BF16 or VTKV_F16, kv_dtype = q_dtype or VTKV_FP8_E4M3, head_size 64, 80, 96, 112, 128 or
  * 256 (the reference's list, vllm/attention/ops/paged_attn.py:33-34), num_heads/num_kv_heads in 1..16.  The kernel
  * is tuned for bf16 and head size 128; the other shapes run the same code with their own tile constants. */
@@ -356,9 +358,9 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
  * in elements) are appended at row seq_lens[b]-1 of sequence b's ranges, which must be mapped that far, and
  * attention runs over all seq_lens[b] rows.  The cache contents and the result are those of
  * vtkv_reshape_and_cache followed by vtkv_decode_attention (the result up to fp32 summation order).
- * Lengths come either from the device (seq_lens) or from the host (host_seq_lens, at most 512 sequences;
- * copied into the kernel arguments during the call, so no upload is needed and the array may be reused
- * at once); pass NULL for the other.  kv_dtype is VTKV_BF16, or VTKV_FP8_E4M3 with k_scale / v_scale: the new
+ * Lengths come either from the device (seq_lens) or from the host (host_seq_lens: copied into the kernel
+ * arguments during the call, 512 per launch, so no upload is needed and the array may be reused at once);
+ * pass NULL for the other.  kv_dtype is VTKV_BF16, or VTKV_FP8_E4M3 with k_scale / v_scale: the new
  * rows are then stored as e4m3fn(x / scale), bit for bit as vtkv_reshape_and_cache stores them, and attended
  * to in that form.  Other arguments as for vtkv_decode_attention. */
 int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,

@@ -200,6 +200,16 @@ def test_very_many_short_sequences_pair_their_kv_heads(gpu_pool, mode):
         _C.check(lib.vtkv_set_fused_merge(-1))
 
 
+def test_more_sequences_than_one_launch_takes(gpu_pool):
+    """A launch takes 1024 sequences; 1300 in one call run as two launches on the same stream and scratch.
+    Lengths differ on either side of the cut, a few sequences are long enough to be shared by workgroups."""
+    rng = np.random.default_rng(78)
+    lens = [int(x) for x in rng.integers(1, 40, 1296)] + [700, 1, 1500, 16]
+    lens[1023], lens[1024] = 300, 2
+    run_case(gpu_pool, 44, lens, 8, 2)
+    run_case(gpu_pool, 45, lens, 8, 2, partition_tokens=256)
+
+
 def test_calls_on_two_streams_do_not_share_scratch(gpu_pool):
     """Two batches attend at the same time on two streams, twenty times over; each result equals the one
     the same call gives when it runs alone (the wrapper keeps one scratch buffer per device and stream)."""
