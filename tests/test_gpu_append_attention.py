@@ -151,7 +151,16 @@ def test_long_sequence_many_workgroups_per_segment(gpu_pool):
     run_case(gpu_pool, 9, [40000, 1, 2, 5000], 32, 8, lens_from="device")
 
 
-def test_rejects_other_cache_types_and_too_many_host_lengths(gpu_pool):
+def test_more_host_lengths_than_one_launch_carries(gpu_pool):
+    """512 lengths fit the kernel arguments of one launch; 700 sequences with host lengths run as two launches
+    inside the one call (cache rows exact, attention within tolerance, as for every other case)."""
+    rng = np.random.default_rng(6)
+    lens = [int(x) for x in rng.integers(1, 50, 697)] + [900, 1, 17]
+    lens[511], lens[512] = 333, 2
+    run_case(gpu_pool, 23, lens, 16, 4, lens_from="host")
+
+
+def test_rejects_other_cache_types_and_shapes(gpu_pool):
     import ctypes as C
 
     import torch
@@ -161,12 +170,7 @@ def test_rejects_other_cache_types_and_too_many_host_lengths(gpu_pool):
     lib = _C.lib()
     t = torch.zeros(1024, dtype=torch.uint8, device="cuda")
     p = C.c_void_p(t.data_ptr())
-    host = (C.c_int32 * 600)(*([1] * 600))
     ws = torch.empty(lib.vtkv_decode_attention_workspace_bytes(600, 8, 128, 16, 0), dtype=torch.uint8, device="cuda")
-    rc = lib.vtkv_decode_append_attention(p, p, p, p, 128, 128, p, p, p, None, host, 600, 8, 1, 128, 1024, 1.0, 16, None,
-                                          _C.BF16, _C.BF16, _C.BF16, 1.0, 1.0, C.c_void_p(ws.data_ptr()), ws.numel(), 0,
-                                          None)
-    assert rc == _C.EINVAL and "512" in _C.last_error()
     rc = lib.vtkv_decode_append_attention(p, p, p, p, 128, 128, p, p, p, p, None, 1, 8, 1, 128, 1024, 1.0, 16, None,
                                           _C.BF16, _C.BF16, _C.F32, 1.0, 1.0, C.c_void_p(ws.data_ptr()), ws.numel(), 0, None)
     assert rc == _C.EINVAL and "q_dtype or FP8_E4M3" in _C.last_error()          # an fp32 cache
