@@ -207,7 +207,13 @@ class RadixCache:
         new_node.ref_counter = child.ref_counter
         new_node.prefix_len = p_len
         new_node.last_access_time = child.last_access_time
-        new_node.value.append(self.split(child.value[0], self.token_size * p_len))
+        # the callable may evict to make room for the new holder: not the node it is cutting from, nor its
+        # ancestors (a raise leaves the tree as it was)
+        child.ref_counter += 1
+        try:
+            new_node.value.append(self.split(child.value[0], self.token_size * p_len))
+        finally:
+            child.ref_counter -= 1
         child.parent = new_node
         del new_node.parent.children[key]
         new_node.parent.children[key[:split_len]] = new_node

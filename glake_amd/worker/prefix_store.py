@@ -69,7 +69,11 @@ class PrefixStore:
         segs = self.engine.vmm_kvcache_segment
         segs[new].share_prefix(segs[run_slot], len(tokens) * self.token_size, self._stream())
         self.rows[new] = len(tokens)
-        known = self.tree.insert(tokens, new)
+        try:
+            known = self.tree.insert(tokens, new)
+        except Exception:                                # no slot for a split: the tree is as it was
+            self._drop(new)
+            raise
         if known == len(tokens):                         # nothing new: the tree did not take the holder
             self._drop(new)
         return known

@@ -110,6 +110,35 @@ def test_a_split_node_inherits_the_references_and_inner_nodes_are_evicted_after_
     assert order == [40, 25]                             # the leaf first, then the node that became a leaf
 
 
+def test_a_split_that_must_evict_for_room_spares_the_node_it_cuts():
+    """The split callable of a full store evicts to get a holder.  The least recently used leaf may be the very
+    node being cut: it must survive, and when nothing else can go the lookup fails with the tree unchanged."""
+    tree = None
+    budget = {"free": 0}
+
+    def split(value, nbytes):
+        if budget["free"] == 0:
+            tree.evict(1, lambda v: (budget.__setitem__("free", budget["free"] + 1), v[0].rows)[1])
+        if budget["free"] == 0:
+            raise RuntimeError("no holder left")
+        budget["free"] -= 1
+        return Holder(nbytes // TOKEN, value)
+
+    tree = RadixCache(TOKEN, split)
+    old, young = tuple(range(30)), (7,) * 12
+    tree.insert(old, Holder(30))                         # the least recently used leaf
+    tree.insert(young, Holder(12))
+    _, n = tree.match_prefix(old[:20] + (99,))           # cuts `old` at 20; room comes from evicting `young`
+    assert n == 20 and tree.match_prefix(young) == (None, 0)
+    assert tree.match_prefix(old)[1] == 30               # the node that was cut is still there
+    leaf = tree.match_node(old)
+    tree.inc_ref_counter(leaf)                           # the sequence is in use: nothing can be evicted now
+    with pytest.raises(RuntimeError):
+        tree.match_prefix(old[:10] + (98,))
+    assert tree.match_prefix(old)[1] == 30 and tree.match_prefix(old[:20])[1] == 20 and tree.total_size() == 2
+    assert leaf.ref_counter == 1 and leaf.parent.ref_counter == 1
+
+
 def test_disabled_tree_matches_nothing():
     tree = RadixCache(TOKEN, lambda v, n: v, disable=True)
     assert tree.insert((1, 2, 3), Holder(3)) == 3 and tree.match_prefix((1, 2, 3)) == (None, 0)
