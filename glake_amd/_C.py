@@ -64,6 +64,7 @@ SIGNATURES = {
     "vtkv_seg_share_prefix": (_i, [_p, _p, _i64, _p]),
     "vtkv_pool_shared_chunks": (_i64, []),
     "vtkv_seg_eager_extend": (_i, [_p, _i]),
+    "vtkv_map_ahead_batch": (_i, [_p, _i, _i64]),
     "vtkv_seg_pending": (_i, [_p]),
     "vtkv_map_ahead_wait": (_i, []),
     "vtkv_extend_kv_cache_batch": (_i, [_p, _i, _p, _p, _i64, _i, _p]),

@@ -839,6 +839,31 @@ int vtkv_seg_eager_extend(vtkv_segment *s, int num_chunks) {
   return VTKV_OK;
 }
 
+int vtkv_map_ahead_batch(vtkv_segment *const *segs, int n, int64_t ahead_bytes) {
+  std::unique_lock<std::mutex> lk(g_pool.mu);
+  VTKV_REQUIRE(n >= 0 && (n == 0 || segs) && ahead_bytes >= 0, "bad segment list or distance");
+  for (int i = 0; i < n; ++i) SEG_CHECK(segs[i]);
+  // only what the pool can serve now is asked for: a request that fails is reported by the segment's next
+  // growth, and a sequence may finish before it needs the chunk
+  int64_t spare = (int64_t)g_pool.free_chunks.size() + g_pool.retired;
+  int queued = 0;
+  for (int i = 0; i < n; ++i) {
+    vtkv_segment *s = segs[i];
+    if (s->pending || s->async_error || s->mapped >= s->context_max) continue;
+    if (s->used + s->v_skew + ahead_bytes <= s->mapped) continue;
+    const int64_t revive = s->held > s->mapped ? 1 : 0;  // a retired chunk of its own comes back without a driver call
+    const int64_t need = revive ? 0 : 2ll * s->layer_num;
+    if (spare < need) continue;
+    spare -= need;
+    if (!g_pool.worker.joinable()) g_pool.worker = std::thread(worker_main);
+    ++s->pending;
+    g_pool.requests.push_back({s, 1});
+    ++queued;
+  }
+  if (queued) g_pool.work_cv.notify_one();
+  return queued;
+}
+
 int vtkv_seg_pending(const vtkv_segment *s) {
   std::unique_lock<std::mutex> lk(g_pool.mu);
   SEG_CHECK(s);

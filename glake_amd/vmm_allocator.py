@@ -287,6 +287,14 @@ def query_cycle(seq_ids: Sequence[int]) -> bool:
     return not query_shm(seq_ids)
 
 
+def map_ahead_batch(segments: Sequence["KVcacheSegment"], ahead_bytes: int) -> int:
+    """``eagerExtend`` for every segment whose rows have come within ``ahead_bytes`` of the end of what is mapped,
+    that has no request under way and that the pool can serve now (``vtkv_map_ahead_batch``); returns how many
+    requests were queued.  No counterpart in the reference, whose scheduler names the sequences one by one."""
+    arr = (C.c_void_p * len(segments))(*[s._h for s in segments])
+    return int(_C.check(_C.lib().vtkv_map_ahead_batch(arr, len(segments), int(ahead_bytes))))
+
+
 def wait_map_ahead() -> None:
     """Block until every map-ahead request has been carried out."""
     _C.check(_C.lib().vtkv_map_ahead_wait())

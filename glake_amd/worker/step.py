@@ -103,7 +103,7 @@ class DecodeStepPlan:
     def __init__(self, segments: Sequence, slot_ids: Sequence[int], key_cache, value_cache, num_heads: int,
                  num_kv_heads: int, head_size: int, scale: float, kv_cache_dtype: str = "auto", k_scale: float = 1.0,
                  v_scale: float = 1.0, model_dtype: torch.dtype = torch.bfloat16, device=None, ring: int = 128,
-                 fused: bool = True):
+                 fused: bool = True, map_ahead_rows: int = 64):
         import ctypes as C
 
         import numpy as np
@@ -145,6 +145,12 @@ class DecodeStepPlan:
         self._events = [torch.cuda.Event(), torch.cuda.Event()]
         self._recorded = [False, False]
         self._row = 0
+        # Every 16th step the sequences that have come within `map_ahead_rows` rows of the end of what is mapped
+        # are announced to the map-ahead worker (what the scheduler's extend_seq_list does for an engine), so
+        # that no step maps a chunk in the calling thread: a synchronous mapping costs 0.1 ms, which an empty
+        # launch queue (the first steps after a wait) passes on to the GPU.  0 switches it off.
+        self._ahead_bytes = int(map_ahead_rows) * self.kv_size
+        self._steps = 0
         need = self._lib.vtkv_decode_attention_workspace_bytes(n, self.num_heads, self.head_size, 1, 0)
         # its own scratch (zero-filled once, as the library asks): plans may run on different streams at once
         self._ws = torch.zeros(max(int(need), 1 << 20), dtype=torch.uint8, device=self.device)
@@ -166,6 +172,9 @@ class DecodeStepPlan:
             h = 0 if i == 0 else 1
             if self._recorded[h]:
                 self._events[h].synchronize()
+        if self._ahead_bytes and self._steps % 16 == 0:
+            check(lib.vtkv_map_ahead_batch(self._segs, n, self._ahead_bytes))
+        self._steps += 1
         check(lib.vtkv_extend_kv_cache_batch(self._segs, n, self._tok, None, self.kv_size, 1, self._row_p[i]))
         lens = self._lens[i]
         self._np.floor_divide(self._offs[i], self.kv_size, out=lens, casting="unsafe")

@@ -155,6 +155,13 @@ int64_t vtkv_pool_shared_chunks(void);
  * their work, since a full pool is when a caller preempts to get chunks back.  The driver calls run
  * outside the pool's lock. */
 int vtkv_seg_eager_extend(vtkv_segment *s, int num_chunks);
+/* vtkv_seg_eager_extend(s, 1) for every segment of the list whose rows have come within `ahead_bytes` of the end
+ * of what is mapped (used + ahead_bytes > mapped, the V offset counted), that has no request under way and that
+ * the pool can serve at the time of the call.  Returns how many requests were queued.  This is what the
+ * reference's scheduler does through extend_seq_list (vllm/core/scheduler.py:425-522 -> llama.py:328-337) for
+ * callers that hold the segments but no scheduler: called every few steps with a distance of a few dozen rows,
+ * no decode step maps a chunk in the calling thread. */
+int vtkv_map_ahead_batch(vtkv_segment *const *segs, int n, int64_t ahead_bytes);
 /* Map-ahead requests of the segment that are queued or running; 0 is the reference's "ready" flag
  * (query_shm, vmm_allocator.cpp:86-92). <0 on error. */
 int vtkv_seg_pending(const vtkv_segment *s);

@@ -248,6 +248,47 @@ def test_map_ahead_requests_run_on_the_worker_and_settle(gpu_pool):
     assert vmm.showFreeBlocks() == free0
 
 
+def test_map_ahead_batch_asks_for_what_is_about_to_be_needed(gpu_pool):
+    """One call names every sequence that has come within the given distance of the end of its mapped part:
+    those get a chunk per range from the worker, the others nothing; a second call asks for nothing more; with
+    the pool too empty to serve a request it is not made (and no error is left behind)."""
+    vmm = gpu_pool
+    vmm.trim()
+    free0 = vmm.showFreeBlocks()
+    layers, row = 2, 2048
+    # used bytes: 3 rows, 39 rows and 40 rows short of the chunk's end, far from it, one row short with the V offset
+    near = [CHUNK - 3 * row, CHUNK - 39 * row, CHUNK - 40 * row, 5 * row, CHUNK - 256 - row]
+    segs = [vmm.KVcacheSegment(layers, 4 * CHUNK, 0, False) for _ in near]
+    segs[4].set_value_skew(256)
+    for s, used in zip(segs, near):
+        s.expandMultiSegment(1)
+        s.set_used_size(used)
+    assert vmm.map_ahead_batch(segs, 40 * row) == 3
+    vmm.wait_map_ahead()
+    assert [s.actual_size // CHUNK for s in segs] == [2, 2, 1, 1, 2] and all(s.pending == 0 for s in segs)
+    assert vmm.showFreeBlocks() == free0 - (5 + 3) * 2 * layers
+    assert vmm.map_ahead_batch(segs, 40 * row) == 0          # nothing is that close any more
+    # rows crossing into the chunks that were mapped ahead: no growth in the calling thread
+    for _ in range(5):
+        vmm.extend_kv_cache_batch(None, None, [0, 4], [row] * 2, [segs[0], segs[4]], [0] * 2, row, True)
+    assert segs[0].used_size == CHUNK + 2 * row and segs[0].actual_size == 2 * CHUNK and segs[4].actual_size == 2 * CHUNK
+    # a pool that cannot serve the request: nothing is asked, nothing fails later
+    spare = vmm.showFreeBlocks()
+    hog = vmm.KVcacheSegment(1, (spare // 2 + 2) * CHUNK, 0, False)
+    hog.expandMultiSegment((spare - 2) // 2)                 # leaves 2 or 3 chunks: fewer than one per range of a segment
+    segs[2].set_used_size(CHUNK - 2 * row)
+    assert vmm.map_ahead_batch(segs[2:3], 40 * row) == 0
+    hog.preempt_seq(0)
+    assert vmm.map_ahead_batch(segs[2:3], 40 * row) == 1
+    vmm.wait_map_ahead()
+    assert segs[2].actual_size == 2 * CHUNK
+    vmm.extend_kv_cache_batch(None, None, [2], [3 * row], segs[2:3], [0], row, True)   # no stale error
+    for s in segs + [hog]:
+        s.destroy()
+    vmm.trim()
+    assert vmm.showFreeBlocks() == free0
+
+
 def test_failed_map_ahead_does_not_stop_a_preemption(gpu_pool):
     """Pool exhausted, a map-ahead request fails: calls that shrink the segment still do their work (that is how
     the scheduler gets chunks back), the failure is reported once by the next call that grows it, and a step
