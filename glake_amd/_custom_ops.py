@@ -247,8 +247,8 @@ def prefill_attention(
     qd = _dt(query)
     kvd = _kv_dtype(kv_cache_dtype, qd)
     lib = _C.lib()
-    if head_size != 128 or qd != _C.BF16:
-        # the prompt kernel is built for bf16 and head size 128; the other head sizes and fp16 take the
+    if head_size != 128:
+        # the prompt kernel is built for head size 128 (bf16 or fp16); the other head sizes take the
         # general route: every query token is one decode step over the rows up to its own
         return _prefill_through_decode(out, query, key_cache, value_cache, num_kv_heads, scale, query_lens, seq_lens,
                                        slot_mapping, alibi_slopes, kv_cache_dtype, kv_scale, v_scale)

@@ -106,17 +106,9 @@ __device__ __forceinline__ u32x4 bf16x8_to_f16x8(u32x4 v) {
     r[i] = pack_f16x2(__builtin_bit_cast(float, v[i] << 16), __builtin_bit_cast(float, v[i] & 0xffff0000u));
   return r;
 }
-// Eight e4m3fn codes (two dwords) to eight fp16 values; exact.
-__device__ __forceinline__ u32x4 fp8x8_to_f16x8(unsigned lo, unsigned hi) {
-  u32x4 r;
-  r[0] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, false));
-  r[1] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 1.0f, true));
-  r[2] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, false));
-  r[3] = __builtin_bit_cast(unsigned, (f16x2)__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 1.0f, true));
-  return r;
-}
-
-template <bool ALIBI, bool FP8>
+// F16: queries, rows and output are fp16 instead of bf16 (rows may still be e4m3fn codes).  S runs on the fp16
+// MFMA and V needs no conversion on its way into LDS; nothing can leave the fp16 range, so there is no second pass.
+template <bool ALIBI, bool FP8, bool F16 = false>
 __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kStageBytes];
   const int lane = threadIdx.x & 63;
@@ -140,7 +132,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;
 
   // ---- this wave's columns: block nb, column n -> (token, head); unused columns get q = 0
-  bf16x8 qop[kNB][4];
+  u32x4 qop[kNB][4];
   int limit[kNB];       // rows below this are visible to the lane's column
   int col_tok[kNB], col_head[kNB];
   float slope_log2[kNB];
@@ -158,7 +150,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     for (int ks = 0; ks < 4; ++ks) {
       u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + ks * 32 + g * 8);
       if (!valid) raw = (u32x4){0, 0, 0, 0};
-      qop[nb][ks] = __builtin_bit_cast(bf16x8, raw);
+      qop[nb][ks] = raw;
     }
   }
   // rows this wave needs: up to the limit of its last used column; its first column's limit says from
@@ -228,13 +220,13 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     for (int j = 0; j < kLd; ++j) {
       if constexpr (FP8) {
         // pieces 2p and 2p+1 of a row sit 16 bytes apart before the swizzle, which flips bit 4 or leaves it
-        *reinterpret_cast<u32x4 *>(base + st_k[j]) = fp8x8_to_bf16x8(kst[j][0], kst[j][1]);
-        *reinterpret_cast<u32x4 *>(base + (st_k[j] ^ 16)) = fp8x8_to_bf16x8(kst[j][2], kst[j][3]);
+        *reinterpret_cast<u32x4 *>(base + st_k[j]) = fp8x8_widen<F16>(kst[j][0], kst[j][1]);
+        *reinterpret_cast<u32x4 *>(base + (st_k[j] ^ 16)) = fp8x8_widen<F16>(kst[j][2], kst[j][3]);
         *reinterpret_cast<u32x4 *>(base + st_v[j]) = fp8x8_to_f16x8(vst[j][0], vst[j][1]);
         *reinterpret_cast<u32x4 *>(base + (st_v[j] ^ 16)) = fp8x8_to_f16x8(vst[j][2], vst[j][3]);
       } else {
         *reinterpret_cast<u32x4 *>(base + st_k[j]) = kst[j];
-        *reinterpret_cast<u32x4 *>(base + st_v[j]) = WIDE ? vst[j] : bf16x8_to_f16x8(vst[j]);
+        *reinterpret_cast<u32x4 *>(base + st_v[j]) = (WIDE || F16) ? vst[j] : bf16x8_to_f16x8(vst[j]);
       }
     }
   };
@@ -283,8 +275,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
           sacc[nb][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int ks = 0; ks < 4; ++ks)
-            sacc[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ka[t][ks]), qop[nb][ks],
-                                                                  sacc[nb][t], 0, 0, 0);
+            sacc[nb][t] = mfma_16x16x32<F16>(ka[t][ks], qop[nb][ks], sacc[nb][t]);
         }
       // reduction slot (g, j) of the K=32 P.V MFMA stands for row 4g+j of the first tile (j < 4) and row
       // 4g+j-4 of the second (j >= 4), so a lane's A operand is its transposed quad of the first tile
@@ -395,7 +386,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     }
   };
   run(std::false_type{});
-  if constexpr (!FP8) {
+  if constexpr (!FP8 && !F16) {
     // A V value beyond the fp16 range went into LDS as infinity and has made some accumulator of the workgroup
     // infinite or NaN (a weight of exactly zero gives NaN).  Then the whole unit is computed again with V in
     // bf16; e4m3fn codes always fit fp16.  Inputs that are themselves non-finite take the second pass too and
@@ -427,7 +418,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
       if (p.out_f32) {
         *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.out) + o0 + db * 16) = r;
       } else {
-        u32x2 w = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+        u32x2 w = {pack_16x2<F16>(r[0], r[1]), pack_16x2<F16>(r[2], r[3])};
         *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(p.out) + o0 + db * 16) = w;
       }
     }
@@ -455,10 +446,10 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   VTKV_REQUIRE(num_units >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
   VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
-  VTKV_REQUIRE(q_dtype == VTKV_BF16, "q_dtype must be BF16");
-  VTKV_REQUIRE(out_dtype == VTKV_BF16 || out_dtype == VTKV_F32, "out_dtype must be BF16 or F32");
+  VTKV_REQUIRE(q_dtype == VTKV_BF16 || q_dtype == VTKV_F16, "q_dtype must be BF16 or F16");
+  VTKV_REQUIRE(out_dtype == q_dtype || out_dtype == VTKV_F32, "out_dtype must be q_dtype or F32");
   VTKV_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
-  VTKV_REQUIRE(kv_dtype == VTKV_BF16 || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be BF16 or FP8_E4M3");
+  VTKV_REQUIRE(kv_dtype == q_dtype || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be q_dtype or FP8_E4M3");
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   if (fp8) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
   const int group = num_heads / num_kv_heads;
@@ -488,14 +479,13 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   p.v_scale = fp8 ? v_scale : 1.f;
   const dim3 grid((unsigned)((int64_t)num_units * num_kv_heads)), block(kThreads);
   hipStream_t st = (hipStream_t)stream;
-  if (alibi_slopes && fp8)
-    hipLaunchKernelGGL((prefill_attn_kernel<true, true>), grid, block, 0, st, p);
-  else if (alibi_slopes)
-    hipLaunchKernelGGL((prefill_attn_kernel<true, false>), grid, block, 0, st, p);
-  else if (fp8)
-    hipLaunchKernelGGL((prefill_attn_kernel<false, true>), grid, block, 0, st, p);
-  else
-    hipLaunchKernelGGL((prefill_attn_kernel<false, false>), grid, block, 0, st, p);
+  static void (*const kKernels[8])(PrefillParams) = {
+      prefill_attn_kernel<false, false, false>, prefill_attn_kernel<true, false, false>,
+      prefill_attn_kernel<false, true, false>,  prefill_attn_kernel<true, true, false>,
+      prefill_attn_kernel<false, false, true>,  prefill_attn_kernel<true, false, true>,
+      prefill_attn_kernel<false, true, true>,   prefill_attn_kernel<true, true, true>,
+  };
+  hipLaunchKernelGGL(kKernels[(q_dtype == VTKV_F16 ? 4 : 0) + (fp8 ? 2 : 0) + (alibi_slopes ? 1 : 0)], grid, block, 0, st, p);
   VTKV_HIP(hipGetLastError());
   return VTKV_OK;
 }

@@ -351,8 +351,10 @@ int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
  *            consecutive query tokens of one sequence that share one pass over its rows; every query
  *            token belongs to exactly one unit; longest units first balances the load best
  *   max_seq_len  host upper bound of position + 1 over all query tokens
- * No scratch is needed.  Other arguments as for vtkv_decode_attention (kv_dtype VTKV_BF16 or
- * VTKV_FP8_E4M3 with k_scale / v_scale). */
+ * No scratch is needed.  Other arguments as for vtkv_decode_attention.  Supported: head_size 128, q_dtype
+ * VTKV_BF16 or VTKV_F16, kv_dtype = q_dtype or VTKV_FP8_E4M3 with k_scale / v_scale, out_dtype = q_dtype or
+ * VTKV_F32; the longest-units-first order inside each sequence, sequence by sequence, lets every row be fetched
+ * from HBM once. */
 int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                            const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
                            int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,

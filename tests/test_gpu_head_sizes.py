@@ -132,38 +132,62 @@ def test_long_context_on_a_small_head_and_a_large_one(gpu_pool):
     run_case(gpu_pool, 8, [30000, 100], 16, 4, 256, "bf16")
 
 
-@pytest.mark.parametrize("d,dtype", [(64, "f16"), (80, "bf16"), (128, "f16"), (256, "bf16")])
-def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype):
-    """The prompt kernel is built for bf16 and head size 128; every other shape runs a prompt as one decode step
-    per query token.  Plain prompts and prompts behind cached rows, against the prompt oracle."""
+@pytest.mark.parametrize("d,dtype,fp8,alibi", [(64, "f16", False, False), (80, "bf16", False, False),
+                                               (128, "f16", False, False), (128, "f16", True, False),
+                                               (128, "f16", False, True), (128, "f16", True, True),
+                                               (256, "bf16", False, False)])
+def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype, fp8, alibi):
+    """The prompt kernel is built for head size 128 (bf16 and fp16, either with an fp8 cache); every other head
+    size runs a prompt as one decode step per query token.  Plain prompts and prompts behind cached rows, against
+    the prompt oracle."""
     import torch
 
     from glake_amd import _custom_ops as ops
     from glake_amd.attention.backends.vtensor import VTensorBackend
 
     VTensorBackend.get_impl_cls()(32, d, d ** -0.5, 8, None, None, "auto")     # the backend takes the head size
-    rng = np.random.default_rng(d)
+    rng = np.random.default_rng(d + 7 * fp8 + 13 * alibi)
     hq, hkv = 32, 8
     seq_lens, query_lens = [700, 33, 1, 1300], [700, 20, 1, 400]
     b = len(seq_lens)
     tdt = torch.float16 if dtype == "f16" else torch.bfloat16
-    pairs_k = [to_model(rng.standard_normal((n, hkv, d)).astype(np.float32), dtype) for n in seq_lens]
-    pairs_v = [to_model(rng.standard_normal((n, hkv, d)).astype(np.float32), dtype) for n in seq_lens]
+    k_scale, v_scale = (0.021, 0.033) if fp8 else (1.0, 1.0)
+
+    def rows(n, sc):  # (what the cache holds, the same values in fp32)
+        x = rng.standard_normal((n, hkv, d)).astype(np.float32)
+        if fp8:
+            codes = O.fp8_encode(x, sc)
+            return codes, O.fp8_decode(codes, sc)
+        return to_model(x, dtype)
+
+    pairs_k = [rows(n, k_scale) for n in seq_lens]
+    pairs_v = [rows(n, v_scale) for n in seq_lens]
     n_tok = sum(query_lens)
     q_bits, q32 = to_model(rng.standard_normal((n_tok, hq, d)).astype(np.float32), dtype)
-    gpu = GpuSeqs(gpu_pool, b, hkv, d, 2, max(seq_lens), value_skew=256)
+    slopes = (rng.standard_normal(hq) * 0.3).astype(np.float32) if alibi else None
+    gpu = GpuSeqs(gpu_pool, b, hkv, d, 1 if fp8 else 2, max(seq_lens), value_skew=256)
     for i in range(b):
         gpu.upload(i, pairs_k[i][0], pairs_v[i][0])
     kt, vt = gpu.table_tensors()
     out = torch.empty(n_tok, hq, d, dtype=torch.float32, device="cuda")
     ops.prefill_attention(out, torch.from_numpy(q_bits.view(np.int16).copy()).view(tdt).cuda(), kt, vt, hkv, d ** -0.5,
-                          query_lens, seq_lens, torch.arange(b, dtype=torch.int64, device="cuda"))
+                          query_lens, seq_lens, torch.arange(b, dtype=torch.int64, device="cuda"),
+                          None if slopes is None else torch.from_numpy(slopes).cuda(), "fp8" if fp8 else "auto",
+                          k_scale, v_scale)
+    out16 = torch.empty(n_tok, hq, d, dtype=tdt, device="cuda")
+    ops.prefill_attention(out16, torch.from_numpy(q_bits.view(np.int16).copy()).view(tdt).cuda(), kt, vt, hkv, d ** -0.5,
+                          query_lens, seq_lens, torch.arange(b, dtype=torch.int64, device="cuda"),
+                          None if slopes is None else torch.from_numpy(slopes).cuda(), "fp8" if fp8 else "auto",
+                          k_scale, v_scale)
     torch.cuda.synchronize()
     gpu.close()
     want = O.prefill_attention(q32, O.VTensorCache([p[1] for p in pairs_k], [p[1] for p in pairs_v], np.arange(b), hkv, d),
-                               d ** -0.5, query_lens, seq_lens)
-    err = np.abs(out.cpu().numpy() - want)
+                               d ** -0.5, query_lens, seq_lens, slopes)
+    got = out.cpu().numpy()
+    err = np.abs(got - want)
     assert bool(np.all(err <= 2e-3 + 2e-3 * np.abs(want))), f"max err {err.max():.3e}"
+    # the output in the model's type is the fp32 result rounded once
+    assert torch.equal(out16.cpu(), torch.from_numpy(got).to(tdt))
 
 
 def test_workspace_is_sized_for_the_padded_head_size(gpu_pool):
