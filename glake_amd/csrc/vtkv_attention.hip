@@ -175,7 +175,7 @@ __global__ void __launch_bounds__(kThreads)
     __attribute__((amdgpu_waves_per_eu(D > 128 ? 1 : (FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES))))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
   static_assert(D % 16 == 0 && D >= 64 && D <= 256, "head sizes are multiples of 16 from 64 to 256");
-  static_assert(!APPEND || (D == 128 && !F16), "the fused append is built for bf16 rows of 128 only");
+  static_assert(!APPEND || D == 128, "the fused append is built for head size 128 only");
   constexpr int kHD = FP8 ? (D + 63) / 64 * 64 : (D + 31) / 32 * 32;  // head size as held in LDS and registers
   constexpr int kKSteps = kHD / 32;                                  // MFMA steps of S^T = K.Q^T
   constexpr int kDBlocks = kHD / 16;                                 // 16-row blocks of O^T
@@ -453,7 +453,7 @@ __global__ void __launch_bounds__(kThreads)
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
                 const uint32_t pair = src[(2 * w + e / 2) & 3];
-                const float x = __builtin_bit_cast(float, (e & 1) ? (pair & 0xffff0000u) : (pair << 16));
+                const float x = unpack_16<F16>(pair, e & 1);
                 word |= (uint32_t)vtkv::fp8_e4m3fn_encode(x / sc) << (8 * e);
               }
               c[w] = word;
@@ -990,7 +990,8 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16 + 24;  // instantiations of the streaming kernel: 16 of the tuned shape, 24 others
+constexpr int kVariants = 16 + 24 + 2;  // instantiations of the streaming kernel: 16 of the tuned shape, 24 others,
+                                        // and the fused append for fp16 at head size 128 (fp16 rows, fp8 rows)
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
 int head_size_index(int head_size) {
@@ -1102,7 +1103,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
                "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
   if (append) {
     VTKV_REQUIRE(new_value != nullptr, "null argument");
-    VTKV_REQUIRE(tuned, "the fused append needs bf16 queries and head size 128");
+    VTKV_REQUIRE(head_size == 128, "the fused append needs head size 128");
     const int64_t row = (int64_t)num_kv_heads * head_size;
     VTKV_REQUIRE(key_stride >= row && value_stride >= row && key_stride % 8 == 0 && value_stride % 8 == 0 &&
                      (uintptr_t)new_key % 16 == 0 && (uintptr_t)new_value % 16 == 0,
@@ -1124,8 +1125,9 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   const int seg_heads = pair ? 2 : 1;
   // kernel variant of the tuned shape: bit 0 alibi, bit 1 fused append, bit 2 paired kv heads, bit 3 fp8; the
   // other head sizes and fp16 have one variant per (head size, type, cache type), ALiBi decided at run time
-  const int variant = tuned ? (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0)
-                            : 16 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
+  const int variant = tuned    ? (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0)
+                      : append ? 40 + (fp8 ? 1 : 0)
+                               : 16 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
 #define VTKV_ROW(F8, H)                                                                                      \
   decode_attn_stream_kernel<false, F8, false, H>, decode_attn_stream_kernel<true, F8, false, H>,             \
       decode_attn_stream_kernel<false, F8, true, H>, decode_attn_stream_kernel<true, F8, true, H>
@@ -1135,6 +1137,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   static void (*const kKernels[kVariants])(AttnParams, InlineLens) = {
       VTKV_ROW(false, 1), VTKV_ROW(false, 2), VTKV_ROW(true, 1), VTKV_ROW(true, 2),
       VTKV_SIZE(64), VTKV_SIZE(80), VTKV_SIZE(96), VTKV_SIZE(112), VTKV_SIZE(128), VTKV_SIZE(256),
+      decode_attn_stream_kernel<true, false, true, 1, 128, true>, decode_attn_stream_kernel<true, true, true, 1, 128, true>,
   };
 #undef VTKV_ROW
 #undef VTKV_SIZE

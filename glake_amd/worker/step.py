@@ -156,8 +156,7 @@ class DecodeStepPlan:
         self._ws = torch.zeros(max(int(need), 1 << 20), dtype=torch.uint8, device=self.device)
         self._ws_p, self._ws_n = C.c_void_p(self._ws.data_ptr()), self._ws.numel()
         self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
-        self.fused = (bool(fused) and self._src_dt == _C.BF16 and self.head_size == 128
-                      and self._kv_dt in (_C.BF16, _C.FP8_E4M3))
+        self.fused = (bool(fused) and self.head_size == 128 and self._kv_dt in (self._src_dt, _C.FP8_E4M3))
         self._inline = self.fused and n <= 512
         self._host_lens_p = [C.c_void_p(self._stage[i].data_ptr() + 8 * n) for i in range(ring)]
 

@@ -363,13 +363,14 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
 
 /* reshape_and_cache (decode form: one new row per sequence) fused into the attention launch; replaces
  * the pair of calls at vllm/attention/backends/xformers.py:310-312 and :357-371 for a decode step.
- * seq_lens[b] counts the new token: key[b] / value[b] ([num_seqs, num_kv_heads, head_size] bf16, row strides
+ * seq_lens[b] counts the new token: key[b] / value[b] ([num_seqs, num_kv_heads, head_size] of q_dtype, row strides
  * in elements) are appended at row seq_lens[b]-1 of sequence b's ranges, which must be mapped that far, and
  * attention runs over all seq_lens[b] rows.  The cache contents and the result are those of
  * vtkv_reshape_and_cache followed by vtkv_decode_attention (the result up to fp32 summation order).
  * Lengths come either from the device (seq_lens) or from the host (host_seq_lens: copied into the kernel
  * arguments during the call, 512 per launch, so no upload is needed and the array may be reused at once);
- * pass NULL for the other.  kv_dtype is VTKV_BF16, or VTKV_FP8_E4M3 with k_scale / v_scale: the new
+ * pass NULL for the other.  Head size 128 only; q_dtype VTKV_BF16 or VTKV_F16 (the paired-head variants for
+ * very many short sequences exist for bf16 only).  kv_dtype is q_dtype, or VTKV_FP8_E4M3 with k_scale / v_scale: the new
  * rows are then stored as e4m3fn(x / scale), bit for bit as vtkv_reshape_and_cache stores them, and attended
  * to in that form.  Other arguments as for vtkv_decode_attention. */
 int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,

@@ -190,6 +190,68 @@ def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype, fp8, alibi):
     assert torch.equal(out16.cpu(), torch.from_numpy(got).to(tdt))
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("lens_from", ["host", "device"])
+def test_fused_append_for_fp16_models(gpu_pool, fp8, lens_from):
+    """vtkv_decode_append_attention with fp16 queries and new rows (head size 128): the new row lands in the cache
+    as reshape_and_cache stores it (the fp16 bits, or the e4m3fn codes of value / scale), attention over all
+    rows against the oracle; lengths around tile and chunk boundaries, ALiBi, lengths from either side."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(90 + fp8)
+    hq, hkv, d = 32, 8, 128
+    eb = 1 if fp8 else 2
+    row = hkv * d * eb
+    per = (2 << 20) // row
+    lens = [1, 2, 16, 17, 18, 33, 257, per - 1, per, per + 1, 2500]      # they count the new token
+    b = len(lens)
+    k_scale, v_scale = (0.021, 0.033) if fp8 else (1.0, 1.0)
+
+    def stored(x32, sc):  # (bits in the cache, the values they stand for)
+        if fp8:
+            codes = O.fp8_encode(x32, sc)
+            return codes, O.fp8_decode(codes, sc)
+        return to_model(x32, "f16")
+
+    gpu = GpuSeqs(gpu_pool, b, hkv, d, eb, max(lens) + 1, value_skew=256)
+    k_bits, v_bits, k32, v32 = [], [], [], []
+    for i, t in enumerate(lens):
+        kb, kf = stored(rng.standard_normal((t - 1, hkv, d)).astype(np.float32), k_scale)
+        vb, vf = stored(rng.standard_normal((t - 1, hkv, d)).astype(np.float32), v_scale)
+        gpu.upload(i, kb, vb)
+        k_bits.append(kb), v_bits.append(vb), k32.append(kf), v32.append(vf)
+    used = gpu_pool.extend_kv_cache_batch(None, None, list(range(b)), [row] * b, gpu.segs, [0] * b, row, True)
+    assert used == [(t - 1) * row for t in lens]
+    q16, q32 = to_model(rng.standard_normal((b, hq, d)).astype(np.float32), "f16")
+    nk16, nk32 = to_model(rng.standard_normal((b, hkv, d)).astype(np.float32), "f16")
+    nv16, nv32 = to_model(rng.standard_normal((b, hkv, d)).astype(np.float32), "f16")
+    slopes = (rng.standard_normal(hq) * 0.1).astype(np.float32)
+    kt, vt = gpu.table_tensors()
+    dev = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16).cuda()
+    out = torch.empty(b, hq, d, dtype=torch.float32, device="cuda")
+    lens_arg = list(lens) if lens_from == "host" else torch.tensor(lens, dtype=torch.int32, device="cuda")
+    ops.decode_append_attention(out, dev(q16), dev(nk16).view(b, hkv * d), dev(nv16).view(b, hkv * d), kt, vt, hkv,
+                                d ** -0.5, lens_arg, max(lens), torch.from_numpy(slopes).cuda(),
+                                torch.arange(b, dtype=torch.int64, device="cuda"),
+                                kv_cache_dtype="fp8" if fp8 else "auto", kv_scale=k_scale, v_scale=v_scale)
+    torch.cuda.synchronize()
+    # the appended rows, bit for bit, and nothing before them disturbed
+    for i, t in enumerate(lens):
+        nkb, nkf = stored(nk32[i:i + 1], k_scale)
+        nvb, nvf = stored(nv32[i:i + 1], v_scale)
+        want_k = np.concatenate([k_bits[i], nkb]).reshape(-1).view(np.uint8)
+        want_v = np.concatenate([v_bits[i], nvb]).reshape(-1).view(np.uint8)
+        assert np.array_equal(gpu.download(i, t * row, which="k"), want_k), ("k rows", i)
+        assert np.array_equal(gpu.download(i, t * row, which="v"), want_v), ("v rows", i)
+        k32[i], v32[i] = np.concatenate([k32[i], nkf]), np.concatenate([v32[i], nvf])
+    gpu.close()
+    want = O.paged_attention_v1(q32, O.VTensorCache(k32, v32, np.arange(b), hkv, d), d ** -0.5, lens, slopes)
+    err = np.abs(out.cpu().numpy() - want)
+    assert bool(np.all(err <= 2e-3 + 2e-3 * np.abs(want))), f"max err {err.max():.3e}"
+
+
 def test_workspace_is_sized_for_the_padded_head_size(gpu_pool):
     """A head size of 112 is held as 128 (fp8 rows pad to 64 elements): the workspace the library asks for must
     be sized for that, also through the split-K interface, where the grid and with it the scratch is exact."""
