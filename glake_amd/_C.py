@@ -95,6 +95,7 @@ SIGNATURES = {
     "vtkv_decode_append_attention": (_i, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f,
                                            _i, _p, _i, _i, _i, _f, _f, _p, _i64, _i, _p]),
     "vtkv_prefill_unit_tokens": (_i, [_i, _i, _i]),
+    "vtkv_prefill_unit_tokens_for": (_i, [_i, _i, _i, _i]),
     "vtkv_prefill_attention": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f, _i, _p, _i, _i, _i, _f, _f, _p]),
     "vtkv_set_fused_merge": (_i, [_i]),
     "vtkv_set_head_major": (_i, [_i]),

@@ -247,14 +247,9 @@ def prefill_attention(
     qd = _dt(query)
     kvd = _kv_dtype(kv_cache_dtype, qd)
     lib = _C.lib()
-    if head_size != 128:
-        # the prompt kernel is built for head size 128 (bf16 or fp16); the other head sizes take the
-        # general route: every query token is one decode step over the rows up to its own
-        return _prefill_through_decode(out, query, key_cache, value_cache, num_kv_heads, scale, query_lens, seq_lens,
-                                       slot_mapping, alibi_slopes, kv_cache_dtype, kv_scale, v_scale)
-    per_unit = lib.vtkv_prefill_unit_tokens(num_heads, num_kv_heads, kvd)
+    per_unit = lib.vtkv_prefill_unit_tokens_for(num_heads, num_kv_heads, head_size, kvd)
     if per_unit <= 0:
-        raise _C.VtkvError(_C.EINVAL, f"unsupported head counts {num_heads}/{num_kv_heads}")
+        raise _C.VtkvError(_C.EINVAL, f"unsupported head counts {num_heads}/{num_kv_heads} or head size {head_size}")
     units = prefill_units(query_lens, seq_lens, per_unit)
     if len(units) == 0:
         return
@@ -267,31 +262,6 @@ def prefill_attention(
         _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping), _ptr(units_t), len(units),
         num_heads, num_kv_heads, head_size, query.stride(0), float(scale), int(max(seq_lens)), _ptr(alibi_slopes), qd,
         _dt(out), kvd, float(kv_scale), float(kv_scale if v_scale is None else v_scale), _stream()))
-
-
-def _prefill_through_decode(out, query, key_cache, value_cache, num_kv_heads, scale, query_lens, seq_lens,
-                            slot_mapping, alibi_slopes, kv_cache_dtype, kv_scale, v_scale) -> None:
-    """Causal prompt attention as one decode step per query token (the token at position t attends to rows
-    0..t of its sequence), at most 1024 tokens per launch.  Reads a prompt's rows once per token: correct for
-    every shape the decode kernel serves, and slow for long prompts."""
-    import numpy as np
-
-    lens, owner = [], []
-    for b, (ql, sl) in enumerate(zip(query_lens, seq_lens)):
-        if ql < 0 or sl < ql:
-            raise _C.VtkvError(_C.EINVAL, f"sequence {b}: {ql} query tokens but {sl} rows")
-        lens.append(np.arange(sl - ql + 1, sl + 1, dtype=np.int32))
-        owner.append(np.full(ql, b, np.int64))
-    lens_np = np.concatenate(lens) if lens else np.empty(0, np.int32)
-    if lens_np.size == 0:
-        return
-    dev = query.device
-    lens_t = torch.from_numpy(lens_np).pin_memory().to(dev, non_blocking=True)
-    slot_tok = slot_mapping[torch.from_numpy(np.concatenate(owner)).pin_memory().to(dev, non_blocking=True)]
-    for i in range(0, lens_np.size, 1024):
-        j = min(i + 1024, lens_np.size)
-        paged_attention_v1(out[i:j], query[i:j], key_cache, value_cache, num_kv_heads, scale, lens_t[i:j], 1,
-                           int(lens_np[i:j].max()), alibi_slopes, kv_cache_dtype, kv_scale, slot_tok[i:j], v_scale)
 
 
 def paged_attention_v2(

@@ -44,10 +44,10 @@ constexpr int kThreads = kWaves * 64;
 #define VTKV_PREFILL_NB 2
 #endif
 
-constexpr int kNB = VTKV_PREFILL_NB;          // column blocks of 16 per wave
-constexpr int kCols = kWaves * kNB * 16;      // columns per workgroup
+constexpr int kNB = VTKV_PREFILL_NB;          // column blocks of 16 per wave (one for head sizes above 128)
 constexpr int kKeyBlock = 32;                 // rows per LDS stage = rows of one P.V reduction (two 16-row tiles)
-constexpr int kStageBytes = 2 * kKeyBlock * kRowBytes;  // K then V
+constexpr int col_blocks(int head_size) { return head_size > 128 ? 1 : kNB; }
+constexpr int cols_per_group(int head_size) { return kWaves * col_blocks(head_size) * 16; }  // columns per workgroup
 
 struct PrefillParams {
   const uint16_t *q;
@@ -108,8 +108,21 @@ __device__ __forceinline__ u32x4 bf16x8_to_f16x8(u32x4 v) {
 }
 // F16: queries, rows and output are fp16 instead of bf16 (rows may still be e4m3fn codes).  S runs on the fp16
 // MFMA and V needs no conversion on its way into LDS; nothing can leave the fp16 range, so there is no second pass.
-template <bool ALIBI, bool FP8, bool F16 = false>
+// HS: the head size, 64, 80, 96, 112, 128 or 256.  The kernel was shaped for 128, where every constant below has
+// the value it always had.  K rows are held in LDS padded to the MFMA depth of 32 (80 as 96, 112 as 128; the pad
+// is cleared once and q is zero there); V and the output need no padding, every size being a multiple of 16.
+// Above 128 a wave owns one block of 16 columns instead of two.
+template <bool ALIBI, bool FP8, bool F16 = false, int HS = 128>
 __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p) {
+  constexpr int kD = HS;                              // (shadows the library-wide 128 inside this kernel)
+  constexpr int kHD = (HS + 31) / 32 * 32;            // K row as held in LDS
+  constexpr int kRowBytes = kHD * 2 < 256 ? 256 : kHD * 2;  // LDS pitch of a row (16-bit elements)
+  constexpr int kKS = kHD / 32;                       // MFMA steps over d of S
+  constexpr int kDB = HS / 16;                        // blocks of 16 output columns
+  constexpr int kNB = col_blocks(HS);
+  constexpr int kStageBytes = 2 * kKeyBlock * kRowBytes;  // K then V
+  auto k_lds_offset = [](int row, int piece16) { return row * kRowBytes + ((piece16 ^ (row & 15)) << 4); };
+  auto v_lds_offset = [](int row, int piece16) { return row * kRowBytes + ((piece16 ^ ((row & 7) << 1)) << 4); };
   __shared__ __attribute__((aligned(16))) char smem[2 * kStageBytes];
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
@@ -126,13 +139,13 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   typedef const __attribute__((address_space(1))) char *gptr;
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
   const int64_t slot = p.slot_ids[u_seq];
-  constexpr int kKvRowBytes = FP8 ? kD : kRowBytes;  // bytes of one head row in the cache
+  constexpr int kKvRowBytes = FP8 ? kD : 2 * kD;  // bytes of one head row in the cache
   gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
   gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
   const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;
 
   // ---- this wave's columns: block nb, column n -> (token, head); unused columns get q = 0
-  u32x4 qop[kNB][4];
+  u32x4 qop[kNB][kKS];
   int limit[kNB];       // rows below this are visible to the lane's column
   int col_tok[kNB], col_head[kNB];
   float slope_log2[kNB];
@@ -144,11 +157,12 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     col_tok[nb] = valid ? tok : -1;
     col_head[nb] = head;
     limit[nb] = valid ? u_pos0 + tok + 1 : 0x7fffffff;
-    slope_log2[nb] = ALIBI && valid ? p.alibi_slopes[kvh * G + head] * kLog2e : 0.f;
+    slope_log2[nb] = ALIBI && valid && p.alibi_slopes ? p.alibi_slopes[kvh * G + head] * kLog2e : 0.f;
     const uint16_t *qrow = p.q + (int64_t)(u_row0 + (valid ? tok : 0)) * p.q_stride + (int64_t)(kvh * G + head) * kD;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      u32x4 raw = *reinterpret_cast<const u32x4 *>(qrow + ks * 32 + g * 8);
+    for (int ks = 0; ks < kKS; ++ks) {
+      u32x4 raw = (u32x4){0, 0, 0, 0};
+      if (kHD == kD || ks * 32 + g * 8 < kD) raw = *reinterpret_cast<const u32x4 *>(qrow + ks * 32 + g * 8);
       if (!valid) raw = (u32x4){0, 0, 0, 0};
       qop[nb][ks] = raw;
     }
@@ -159,7 +173,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   const int wave_end = tok_lo < u_ntok ? u_pos0 + min(tok_hi, u_ntok - 1) + 1 : 0;  // 0: no column in use
   const int wave_first_limit = u_pos0 + tok_lo + 1;
 
-  f32x4 acc[kNB][8];
+  f32x4 acc[kNB][kDB];
   float m_run[kNB], l_run[kNB];
   auto reset = [&]() {
 #pragma unroll
@@ -167,49 +181,67 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
       m_run[nb] = -INFINITY;
       l_run[nb] = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[nb][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < kDB; ++i) acc[nb][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
   };
   reset();
 
-  // ---- cooperative stage loads of a block of kKeyBlock rows.  bf16 rows: thread t takes piece t%16 of
-  // rows t/16 + 16j.  fp8 rows have 8 pieces of 16 codes: thread t takes piece t%8 of rows t/8 + 32j and
-  // widens it to two 16-bit pieces on the way into LDS.  A thread's byte offset into the K range is also
-  // its offset into the V range; it advances by 32 rows per stage and is clamped to the same piece of the
-  // last row (rows past the end are masked for every column in use, so any finite in-bounds data will do).
-  constexpr int kLd = FP8 ? kKeyBlock / 32 : kKeyBlock / 16;
-  const int ld_piece = FP8 ? threadIdx.x & 7 : threadIdx.x & 15, ld_row = FP8 ? threadIdx.x >> 3 : threadIdx.x >> 4;
+  // ---- cooperative stage loads of a block of kKeyBlock rows.  The 16-byte pieces of the block (kGp per row:
+  // 16 for a bf16 row of 128, 8 for its fp8 codes) are dealt to the threads in order, piece 256 j + t to load j
+  // of thread t; an fp8 piece carries 16 codes and is widened to two 16-bit pieces on the way into LDS.  A
+  // thread's byte offset into the K range is also its offset into the V range; it advances by 32 rows per
+  // stage and is clamped to the same piece of the last row (rows past the end are masked for every column in
+  // use, so any finite in-bounds data will do).  Where the pieces do not fill the last load, its idle threads
+  // fetch a piece again and store nothing.
+  constexpr int kGp = FP8 ? kD / 16 : kD / 8;
+  constexpr int kStagePieces = kKeyBlock * kGp;
+  constexpr int kLd = (kStagePieces + kThreads - 1) / kThreads;
+  constexpr bool kEvenLd = kStagePieces % kThreads == 0;
+  int ld_row[kLd], ld_piece[kLd];
+  bool ld_live[kLd];
+#pragma unroll
+  for (int j = 0; j < kLd; ++j) {
+    const int idx = j * kThreads + (int)threadIdx.x;
+    ld_live[j] = kEvenLd || idx < kStagePieces;
+    ld_row[j] = ld_live[j] ? idx / kGp : 0;
+    ld_piece[j] = ld_live[j] ? idx % kGp : 0;
+  }
   const int nblocks = (kv_len + kKeyBlock - 1) / kKeyBlock;
-  const uint32_t last_off = (uint32_t)(kv_len - 1) * row_stride + ld_piece * 16;
   const uint32_t stage_step = kKeyBlock * row_stride;
-  uint32_t ld_off[kLd];
+  uint32_t ld_off[kLd], last_off[kLd];
+#pragma unroll
+  for (int j = 0; j < kLd; ++j) last_off[j] = (uint32_t)(kv_len - 1) * row_stride + ld_piece[j] * 16;
   auto rewind = [&]() {
 #pragma unroll
-    for (int j = 0; j < kLd; ++j) ld_off[j] = (uint32_t)(j * (kKeyBlock / kLd) + ld_row) * row_stride + ld_piece * 16;
+    for (int j = 0; j < kLd; ++j) ld_off[j] = (uint32_t)ld_row[j] * row_stride + ld_piece[j] * 16;
   };
   rewind();
   u32x4 kst[kLd], vst[kLd];
   auto gload = [&]() {  // loads the next stage's rows and moves on
 #pragma unroll
     for (int j = 0; j < kLd; ++j) {
-      const uint32_t off = min(ld_off[j], last_off);
+      const uint32_t off = min(ld_off[j], last_off[j]);
       kst[j] = *(gvec)(k_base + off);
       vst[j] = *(gvec)(v_base + off);
       ld_off[j] += stage_step;
     }
   };
+  if constexpr (kHD != kD) {
+    // the pad pieces of the K rows of both stages: cleared once, no load ever writes them
+    constexpr int kPad = (kHD - kD) / 8;
+    for (int i = threadIdx.x; i < 2 * kKeyBlock * kPad; i += kThreads) {
+      const int buf = i / (kKeyBlock * kPad), rem = i % (kKeyBlock * kPad), row = rem / kPad, pp = kD / 8 + rem % kPad;
+      *reinterpret_cast<u32x4 *>(smem + buf * kStageBytes + (row >> 4) * kTile * kRowBytes + k_lds_offset(row & 15, pp)) =
+          (u32x4){0, 0, 0, 0};
+    }
+  }
   // LDS byte offsets that do not depend on the stage, so that the stage's buffer and tile add as immediates
   int st_k[kLd], st_v[kLd];  // where lstore puts this thread's pieces (fp8: the first of each pair)
 #pragma unroll
   for (int j = 0; j < kLd; ++j) {
-    if constexpr (FP8) {
-      const int row = j * 32 + ld_row, tile = row >> 4, r = row & 15;
-      st_k[j] = tile * kTile * kRowBytes + k_lds_offset(r, 2 * ld_piece);
-      st_v[j] = kKeyBlock * kRowBytes + tile * kTile * kRowBytes + v_lds_offset(r, 2 * ld_piece);
-    } else {
-      st_k[j] = j * kTile * kRowBytes + k_lds_offset(ld_row, ld_piece);
-      st_v[j] = kKeyBlock * kRowBytes + j * kTile * kRowBytes + v_lds_offset(ld_row, ld_piece);
-    }
+    const int tile = ld_row[j] >> 4, r = ld_row[j] & 15, lp = FP8 ? 2 * ld_piece[j] : ld_piece[j];
+    st_k[j] = tile * kTile * kRowBytes + k_lds_offset(r, lp);
+    st_v[j] = kKeyBlock * kRowBytes + tile * kTile * kRowBytes + v_lds_offset(r, lp);
   }
   // WIDE (bf16 rows only): V stays bf16 in LDS and P.V runs on the bf16 MFMA with P as a bf16 head plus a bf16
   // tail, the decode kernel's arithmetic: twice the P.V MFMAs, no limit on |V|.  Used for a unit's second pass.
@@ -218,6 +250,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     char *base = smem + decltype(bufc)::value * kStageBytes;
 #pragma unroll
     for (int j = 0; j < kLd; ++j) {
+      if (!ld_live[j]) continue;
       if constexpr (FP8) {
         // pieces 2p and 2p+1 of a row sit 16 bytes apart before the swizzle, which flips bit 4 or leaves it
         *reinterpret_cast<u32x4 *>(base + st_k[j]) = fp8x8_widen<F16>(kst[j][0], kst[j][1]);
@@ -231,17 +264,17 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     }
   };
   // A operands of S^T = K.Q^T: lane (n, g) takes row n, bytes [16g, +16) of each 64-byte quarter c
-  int ka_off[4];
+  int ka_off[kKS];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) ka_off[c] = k_lds_offset(n, 4 * c + g);
+  for (int c = 0; c < kKS; ++c) ka_off[c] = k_lds_offset(n, 4 * c + g);
   // A operands of O^T += V^T.P^T: the lane's transposed quad of dims [16db, +16)
-  int vq_off[8];
+  int vq_off[kDB];
   {
     const int row = 4 * g + (n >> 2);
     const int base = kKeyBlock * kRowBytes + row * kRowBytes + ((n & 1) << 3);
     const int swz = (row & 7) << 1;
 #pragma unroll
-    for (int db = 0; db < 8; ++db) vq_off[db] = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
+    for (int db = 0; db < kDB; ++db) vq_off[db] = base + (((2 * db + ((n >> 1) & 1)) ^ swz) << 4);
   }
   const float sl = p.scale_log2;
   // The reference point of the exponentials only follows the running maximum when that has grown by more
@@ -258,11 +291,11 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     const char *st = smem + buf * kStageBytes;
     const int t0 = kb * kKeyBlock;
     if (t0 < wave_end) {  // wave-uniform: else nothing this wave's columns may see
-      u32x4 ka[2][4];
+      u32x4 ka[2][kKS];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
+        for (int c = 0; c < kKS; ++c)
           ka[t][c] = *reinterpret_cast<const u32x4 *>(st + t * kTile * kRowBytes + ka_off[c]);
       const bool masked = t0 + kKeyBlock > wave_first_limit;  // wave-uniform: the stage reaches some column's limit
       // all S MFMAs first, then per column block its softmax followed by its P.V MFMAs, so that the matrix
@@ -274,15 +307,15 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
         for (int t = 0; t < 2; ++t) {
           sacc[nb][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks)
+          for (int ks = 0; ks < kKS; ++ks)
             sacc[nb][t] = mfma_16x16x32<F16>(ka[t][ks], qop[nb][ks], sacc[nb][t]);
         }
       // reduction slot (g, j) of the K=32 P.V MFMA stands for row 4g+j of the first tile (j < 4) and row
       // 4g+j-4 of the second (j >= 4), so a lane's A operand is its transposed quad of the first tile
       // followed by that of the second; read once for both column blocks
-      u32x4 vop[8];
+      u32x4 vop[kDB];
 #pragma unroll
-      for (int db = 0; db < 8; ++db) {
+      for (int db = 0; db < kDB; ++db) {
         const u32x2 qa = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                                                        (__attribute__((address_space(3))) s16x4 *)(st + vq_off[db])));
         const u32x2 qb = __builtin_bit_cast(
@@ -321,7 +354,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
           m_run[nb] = m_new;
           l_run[nb] *= alpha;
 #pragma unroll
-          for (int d = 0; d < 8; ++d) acc[nb][d] *= alpha;
+          for (int d = 0; d < kDB; ++d) acc[nb][d] *= alpha;
         }
         // (a column can have everything so far masked; the reference point 0 keeps exp2(-inf - ref) = 0)
         const float m_ref = m_run[nb] == -INFINITY ? 0.f : m_run[nb];
@@ -349,7 +382,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
           for (int r = 0; r < 8; ++r) l += pr[r];
           l_run[nb] = l;
 #pragma unroll
-          for (int db = 0; db < 8; ++db) {
+          for (int db = 0; db < kDB; ++db) {
             acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[db]),
                                                                   __builtin_bit_cast(bf16x8, ph), acc[nb][db], 0, 0, 0);
             acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[db]),
@@ -365,7 +398,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
           l_run[nb] = l;
           const f16x8 pop = __builtin_bit_cast(f16x8, pb);
 #pragma unroll
-          for (int db = 0; db < 8; ++db)
+          for (int db = 0; db < kDB; ++db)
             acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, vop[db]), pop, acc[nb][db], 0,
                                                                  0, 0);
         }
@@ -395,10 +428,19 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
-      for (int db = 0; db < 8; ++db)
+      for (int db = 0; db < kDB; ++db)
 #pragma unroll
         for (int i = 0; i < 4; ++i) expo = max(expo, __builtin_bit_cast(unsigned, acc[nb][db][i]) & 0x7f800000u);
-    if (__syncthreads_or(expo == 0x7f800000u)) {
+    // (one flag at the start of the stage memory, which nobody reads any more: every wave has passed the last
+    // stage's barrier; the second pass may only overwrite it once all have read it)
+    int *flag = reinterpret_cast<int *>(smem);
+    if (threadIdx.x == 0) *flag = 0;
+    __syncthreads();
+    if (__builtin_amdgcn_ballot_w64(expo == 0x7f800000u) != 0 && lane == 0) *flag = 1;
+    __syncthreads();
+    const bool again = uniform(*flag) != 0;
+    __syncthreads();
+    if (again) {
       reset();
       rewind();
       run(std::true_type{});
@@ -413,7 +455,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     const float inv = p.v_scale / l;
     const int64_t o0 = ((int64_t)(u_row0 + col_tok[nb]) * p.num_heads + kvh * G + col_head[nb]) * kD + 4 * g;
 #pragma unroll
-    for (int db = 0; db < 8; ++db) {
+    for (int db = 0; db < kDB; ++db) {
       const f32x4 r = acc[nb][db] * inv;
       if (p.out_f32) {
         *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.out) + o0 + db * 16) = r;
@@ -425,16 +467,33 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   }
 }
 
+// 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
+int size_index(int head_size) {
+  switch (head_size) {
+    case 64: return 0;
+    case 80: return 1;
+    case 96: return 2;
+    case 112: return 3;
+    case 128: return 4;
+    case 256: return 5;
+    default: return -1;
+  }
+}
+
 }  // namespace
 
 extern "C" {
 
-int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype) {
+int vtkv_prefill_unit_tokens_for(int num_heads, int num_kv_heads, int head_size, int kv_dtype) {
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return 0;
   const int group = num_heads / num_kv_heads;
-  if (group > 16) return 0;
-  (void)kv_dtype;  // the same kernel serves both cache types
-  return kCols / group;
+  if (group > 16 || size_index(head_size) < 0) return 0;
+  (void)kv_dtype;  // the same kernels serve both cache types
+  return cols_per_group(head_size) / group;
+}
+
+int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype) {
+  return vtkv_prefill_unit_tokens_for(num_heads, num_kv_heads, 128, kv_dtype);
 }
 
 int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
@@ -445,7 +504,8 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   VTKV_REQUIRE(out && q && k_ptrs && v_ptrs && slot_ids && units, "null argument");
   VTKV_REQUIRE(num_units >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
-  VTKV_REQUIRE(head_size == kD, "head_size %d is not supported (only 128)", head_size);
+  const int d_index = size_index(head_size);
+  VTKV_REQUIRE(d_index >= 0, "head_size %d is not supported (64, 80, 96, 112, 128, 256)", head_size);
   VTKV_REQUIRE(q_dtype == VTKV_BF16 || q_dtype == VTKV_F16, "q_dtype must be BF16 or F16");
   VTKV_REQUIRE(out_dtype == q_dtype || out_dtype == VTKV_F32, "out_dtype must be q_dtype or F32");
   VTKV_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
@@ -479,13 +539,25 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   p.v_scale = fp8 ? v_scale : 1.f;
   const dim3 grid((unsigned)((int64_t)num_units * num_kv_heads)), block(kThreads);
   hipStream_t st = (hipStream_t)stream;
+  // head size 128: one kernel per (type, cache type, ALiBi); the other sizes decide ALiBi at run time
   static void (*const kKernels[8])(PrefillParams) = {
       prefill_attn_kernel<false, false, false>, prefill_attn_kernel<true, false, false>,
       prefill_attn_kernel<false, true, false>,  prefill_attn_kernel<true, true, false>,
       prefill_attn_kernel<false, false, true>,  prefill_attn_kernel<true, false, true>,
       prefill_attn_kernel<false, true, true>,   prefill_attn_kernel<true, true, true>,
   };
-  hipLaunchKernelGGL(kKernels[(q_dtype == VTKV_F16 ? 4 : 0) + (fp8 ? 2 : 0) + (alibi_slopes ? 1 : 0)], grid, block, 0, st, p);
+#define VTKV_PREFILL_SIZE(HS)                                                                        \
+  prefill_attn_kernel<true, false, false, HS>, prefill_attn_kernel<true, true, false, HS>,           \
+      prefill_attn_kernel<true, false, true, HS>, prefill_attn_kernel<true, true, true, HS>
+  static void (*const kOthers[6][4])(PrefillParams) = {
+      {VTKV_PREFILL_SIZE(64)}, {VTKV_PREFILL_SIZE(80)},  {VTKV_PREFILL_SIZE(96)},
+      {VTKV_PREFILL_SIZE(112)}, {VTKV_PREFILL_SIZE(128)}, {VTKV_PREFILL_SIZE(256)},
+  };
+#undef VTKV_PREFILL_SIZE
+  const bool f16 = q_dtype == VTKV_F16;
+  void (*kernel)(PrefillParams) = head_size == 128 ? kKernels[(f16 ? 4 : 0) + (fp8 ? 2 : 0) + (alibi_slopes ? 1 : 0)]
+                                                   : kOthers[d_index][(f16 ? 2 : 0) + (fp8 ? 1 : 0)];
+  hipLaunchKernelGGL(kernel, grid, block, 0, st, p);
   VTKV_HIP(hipGetLastError());
   return VTKV_OK;
 }

@@ -336,8 +336,10 @@ int vtkv_decode_attention_v2(void *out, float *exp_sums, float *max_logits, void
                              const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
                              float v_scale, void *workspace, int64_t workspace_bytes, void *stream);
 
-/* Query tokens one unit may hold: 128 / (num_heads/num_kv_heads) (one workgroup per unit and kv head).
- * 0 for unsupported shapes. */
+/* Query tokens one unit may hold (one workgroup per unit and kv head): 128 / (num_heads/num_kv_heads) for head
+ * sizes up to 128, 64 / (num_heads/num_kv_heads) for 256.  0 for unsupported shapes.  vtkv_prefill_unit_tokens is
+ * the head size 128 form. */
+int vtkv_prefill_unit_tokens_for(int num_heads, int num_kv_heads, int head_size, int kv_dtype);
 int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
 
 /* Causal attention of prompt (or chunked-prefill) tokens over the contiguous ranges, which already hold
@@ -347,11 +349,12 @@ int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
  * function of the cache contents).  The query token at position t of its sequence attends to rows 0..t.
  *   q, out   [num_query_tokens, num_heads, head_size]: the query tokens of all sequences, packed
  *   units    device int32[num_units][4] = {sequence index into slot_ids, first query row, number of query
- *            tokens (1 .. vtkv_prefill_unit_tokens(...)), position of the first of them in its sequence}:
+ *            tokens (1 .. vtkv_prefill_unit_tokens_for(...)), position of the first of them in its sequence}:
  *            consecutive query tokens of one sequence that share one pass over its rows; every query
  *            token belongs to exactly one unit; longest units first balances the load best
  *   max_seq_len  host upper bound of position + 1 over all query tokens
- * No scratch is needed.  Other arguments as for vtkv_decode_attention.  Supported: head_size 128, q_dtype
+ * No scratch is needed.  Other arguments as for vtkv_decode_attention.  Supported: head_size 64, 80, 96, 112, 128
+ * or 256 (the kernel is tuned for 128; units hold vtkv_prefill_unit_tokens_for(...) tokens), q_dtype
  * VTKV_BF16 or VTKV_F16, kv_dtype = q_dtype or VTKV_FP8_E4M3 with k_scale / v_scale, out_dtype = q_dtype or
  * VTKV_F32; the longest-units-first order inside each sequence, sequence by sequence, lets every row be fetched
  * from HBM once. */

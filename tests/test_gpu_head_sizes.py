@@ -132,14 +132,18 @@ def test_long_context_on_a_small_head_and_a_large_one(gpu_pool):
     run_case(gpu_pool, 8, [30000, 100], 16, 4, 256, "bf16")
 
 
-@pytest.mark.parametrize("d,dtype,fp8,alibi", [(64, "f16", False, False), (80, "bf16", False, False),
+@pytest.mark.parametrize("d,dtype,fp8,alibi", [(64, "f16", False, False), (64, "bf16", True, True),
+                                               (80, "bf16", False, False), (80, "f16", True, False),
+                                               (96, "bf16", True, False), (96, "f16", False, True),
+                                               (112, "f16", False, True), (112, "bf16", False, False),
                                                (128, "f16", False, False), (128, "f16", True, False),
                                                (128, "f16", False, True), (128, "f16", True, True),
-                                               (256, "bf16", False, False)])
+                                               (256, "bf16", False, False), (256, "f16", True, True),
+                                               (256, "bf16", True, False), (256, "f16", False, False)])
 def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype, fp8, alibi):
-    """The prompt kernel is built for head size 128 (bf16 and fp16, either with an fp8 cache); every other head
-    size runs a prompt as one decode step per query token.  Plain prompts and prompts behind cached rows, against
-    the prompt oracle."""
+    """The prompt kernel on every head size of the reference's list, bf16 and fp16 models, 16-bit and fp8 caches,
+    with and without ALiBi (shaped for bf16 at 128, which tests/test_gpu_prefill_attention.py covers).  Plain
+    prompts and prompts behind cached rows, against the prompt oracle."""
     import torch
 
     from glake_amd import _custom_ops as ops
