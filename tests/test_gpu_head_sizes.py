@@ -144,15 +144,20 @@ def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype, fp8, alibi):
     """The prompt kernel on every head size of the reference's list, bf16 and fp16 models, 16-bit and fp8 caches,
     with and without ALiBi (shaped for bf16 at 128, which tests/test_gpu_prefill_attention.py covers).  Plain
     prompts and prompts behind cached rows, against the prompt oracle."""
-    import torch
-
-    from glake_amd import _custom_ops as ops
     from glake_amd.attention.backends.vtensor import VTensorBackend
 
     VTensorBackend.get_impl_cls()(32, d, d ** -0.5, 8, None, None, "auto")     # the backend takes the head size
-    rng = np.random.default_rng(d + 7 * fp8 + 13 * alibi)
-    hq, hkv = 32, 8
-    seq_lens, query_lens = [700, 33, 1, 1300], [700, 20, 1, 400]
+    run_prompt_case(gpu_pool, d + 7 * fp8 + 13 * alibi, [700, 20, 1, 400], [700, 33, 1, 1300], 32, 8, d, dtype, fp8, alibi)
+
+
+def run_prompt_case(vmm, seed, query_lens, seq_lens, hq, hkv, d, dtype, fp8=False, alibi=False):
+    """Prompts of query_lens tokens behind seq_lens - query_lens cached rows: fp32 output against the prompt oracle,
+    and the output in the model's type equal to the fp32 one rounded once."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(seed)
     b = len(seq_lens)
     tdt = torch.float16 if dtype == "f16" else torch.bfloat16
     k_scale, v_scale = (0.021, 0.033) if fp8 else (1.0, 1.0)
@@ -169,20 +174,17 @@ def test_prompt_attention_on_other_head_sizes(gpu_pool, d, dtype, fp8, alibi):
     n_tok = sum(query_lens)
     q_bits, q32 = to_model(rng.standard_normal((n_tok, hq, d)).astype(np.float32), dtype)
     slopes = (rng.standard_normal(hq) * 0.3).astype(np.float32) if alibi else None
-    gpu = GpuSeqs(gpu_pool, b, hkv, d, 1 if fp8 else 2, max(seq_lens), value_skew=256)
+    gpu = GpuSeqs(vmm, b, hkv, d, 1 if fp8 else 2, max(seq_lens), value_skew=256)
     for i in range(b):
         gpu.upload(i, pairs_k[i][0], pairs_v[i][0])
     kt, vt = gpu.table_tensors()
     out = torch.empty(n_tok, hq, d, dtype=torch.float32, device="cuda")
-    ops.prefill_attention(out, torch.from_numpy(q_bits.view(np.int16).copy()).view(tdt).cuda(), kt, vt, hkv, d ** -0.5,
-                          query_lens, seq_lens, torch.arange(b, dtype=torch.int64, device="cuda"),
-                          None if slopes is None else torch.from_numpy(slopes).cuda(), "fp8" if fp8 else "auto",
-                          k_scale, v_scale)
     out16 = torch.empty(n_tok, hq, d, dtype=tdt, device="cuda")
-    ops.prefill_attention(out16, torch.from_numpy(q_bits.view(np.int16).copy()).view(tdt).cuda(), kt, vt, hkv, d ** -0.5,
-                          query_lens, seq_lens, torch.arange(b, dtype=torch.int64, device="cuda"),
-                          None if slopes is None else torch.from_numpy(slopes).cuda(), "fp8" if fp8 else "auto",
-                          k_scale, v_scale)
+    for o in (out, out16):
+        ops.prefill_attention(o, torch.from_numpy(q_bits.view(np.int16).copy()).view(tdt).cuda(), kt, vt, hkv, d ** -0.5,
+                              query_lens, seq_lens, torch.arange(b, dtype=torch.int64, device="cuda"),
+                              None if slopes is None else torch.from_numpy(slopes).cuda(), "fp8" if fp8 else "auto",
+                              k_scale, v_scale)
     torch.cuda.synchronize()
     gpu.close()
     want = O.prefill_attention(q32, O.VTensorCache([p[1] for p in pairs_k], [p[1] for p in pairs_v], np.arange(b), hkv, d),

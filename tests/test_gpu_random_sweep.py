@@ -98,7 +98,8 @@ def test_random_sweep_fp8_decode(gpu_pool, seed):
 @pytest.mark.parametrize("seed", [606, 707])
 def test_random_sweep_over_head_sizes_and_types(gpu_pool, seed):
     """The same sweep over the other head sizes (64, 80, 96, 112, 256, and 128 in fp16), fp16 and bf16, plain and
-    fp8 caches, the plain entry point with stream-K or fixed partitions and the split-K interface."""
+    fp8 caches, the plain entry point with stream-K or fixed partitions and the split-K interface; for half of
+    the cases also a batch of prompts (some behind cached rows) through the prompt kernel of that shape."""
     import test_gpu_head_sizes as H
     from glake_amd import _C
 
@@ -127,5 +128,12 @@ def test_random_sweep_over_head_sizes_and_types(gpu_pool, seed):
             print(f"case {case}: seed {sub} heads {hq}/{hkv} d {d} {dtype} fp8 {fp8} lens {lens} {version} partition {pt} "
                   f"alibi {alibi} merge {merge}", flush=True)
             H.run_case(gpu_pool, sub, lens, hq, hkv, d, dtype, fp8=fp8, alibi=alibi, version=version, partition_tokens=pt)
+            if rng.integers(2) == 0:
+                seq = [int(x) for x in rng.integers(1, 700, int(rng.integers(1, 6)))]
+                ql = [int(rng.integers(1, s + 1)) if rng.integers(2) else s for s in seq]
+                pf8, pal = bool(rng.integers(3) == 0), bool(rng.integers(3) == 0)
+                print(f"prompt case {case}: seed {sub} heads {hq}/{hkv} d {d} {dtype} queries {ql} rows {seq} fp8 {pf8} "
+                      f"alibi {pal}", flush=True)
+                H.run_prompt_case(gpu_pool, sub, ql, seq, hq, hkv, d, dtype, fp8=pf8, alibi=pal)
     finally:
         _C.check(lib.vtkv_set_fused_merge(-1))
