@@ -990,8 +990,9 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16 + 24 + 2;  // instantiations of the streaming kernel: 16 of the tuned shape, 24 others,
-                                        // and the fused append for fp16 at head size 128 (fp16 rows, fp8 rows)
+constexpr int kVariants = 16 + 24 + 2 + 18;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
+                                             // others, the fused append for fp16 at head size 128 (fp16 rows, fp8
+                                             // rows), 18 that stream several kv heads per segment at other shapes
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
 int head_size_index(int head_size) {
@@ -1122,12 +1123,25 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   // groups up to 8.
   const bool many_short = (int64_t)num_seqs * num_kv_heads >= 4096;
   const bool pair = tuned && (fp8 ? VTKV_ATTN_FP8_PAIR != 0 : many_short) && num_kv_heads % 2 == 0 && group <= 8;
-  const int seg_heads = pair ? 2 : 1;
+  int seg_heads = pair ? 2 : 1;
   // kernel variant of the tuned shape: bit 0 alibi, bit 1 fused append, bit 2 paired kv heads, bit 3 fp8; the
   // other head sizes and fp16 have one variant per (head size, type, cache type), ALiBi decided at run time
-  const int variant = tuned    ? (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0)
-                      : append ? 40 + (fp8 ? 1 : 0)
-                               : 16 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
+  int variant = tuned    ? (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0)
+                : append ? 40 + (fp8 ? 1 : 0)
+                         : 16 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
+  if (!tuned) {
+    // A head row that is no whole number of 128-byte lines (160, 192, 224 bytes; 64 to 112 bytes of fp8 codes)
+    // drags its neighbours' bytes along with every fetch, and a lone line streams slower than a pair (see the
+    // kernel): where the head counts allow it, a segment then holds 2 or 4 adjacent kv heads, so that a workgroup
+    // reads 256 to 896 contiguous bytes per token.  64 sequences of 512..4096 rows, 8 kv heads, share of the
+    // HBM peak with one head per segment: head size 80 0.51, 96 0.60, 112 0.53, 64 0.72; fp8 rows 0.29 to 0.40.
+    static const int kHeads16[6] = {2, 4, 2, 4, 1, 1}, kHeads8[6] = {4, 4, 4, 4, 2, 1};
+    const int want = fp8 ? kHeads8[d_index] : kHeads16[d_index];
+    if (want > 1 && num_kv_heads % want == 0 && group * want <= 16) {
+      seg_heads = want;
+      variant = head_size == 128 ? 58 + (append ? 1 : 0) : 42 + d_index * 4 + (f16 ? 2 : 0) + (fp8 ? 1 : 0);
+    }
+  }
 #define VTKV_ROW(F8, H)                                                                                      \
   decode_attn_stream_kernel<false, F8, false, H>, decode_attn_stream_kernel<true, F8, false, H>,             \
       decode_attn_stream_kernel<false, F8, true, H>, decode_attn_stream_kernel<true, F8, true, H>
@@ -1138,6 +1152,12 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
       VTKV_ROW(false, 1), VTKV_ROW(false, 2), VTKV_ROW(true, 1), VTKV_ROW(true, 2),
       VTKV_SIZE(64), VTKV_SIZE(80), VTKV_SIZE(96), VTKV_SIZE(112), VTKV_SIZE(128), VTKV_SIZE(256),
       decode_attn_stream_kernel<true, false, true, 1, 128, true>, decode_attn_stream_kernel<true, true, true, 1, 128, true>,
+#define VTKV_GROUPED(DD, H16, H8)                                                                                  \
+  decode_attn_stream_kernel<true, false, false, H16, DD, false>, decode_attn_stream_kernel<true, true, false, H8, DD, false>, \
+      decode_attn_stream_kernel<true, false, false, H16, DD, true>, decode_attn_stream_kernel<true, true, false, H8, DD, true>
+      VTKV_GROUPED(64, 2, 4), VTKV_GROUPED(80, 4, 4), VTKV_GROUPED(96, 2, 4), VTKV_GROUPED(112, 4, 4),
+#undef VTKV_GROUPED
+      decode_attn_stream_kernel<true, true, false, 2, 128, true>, decode_attn_stream_kernel<true, true, true, 2, 128, true>,
   };
 #undef VTKV_ROW
 #undef VTKV_SIZE
