@@ -164,7 +164,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=32, help="layers of a step with --host-path backend")
     ap.add_argument("--repeats", type=int, default=0,
                     help="timed regions of exactly --steps steps each, synchronised on both sides; the median one is "
-                         "reported (0 = 11 for regions of up to 50 steps, else 3)")
+                         "reported (0 = 21 for regions of up to 50 steps, else 3)")
     ap.add_argument("--unfused", action="store_true",
                     help="plan path: separate reshape_and_cache and attention launches instead of the fused one")
     ap.add_argument("--merge", default="auto", choices=["auto", "fused", "separate"],
@@ -195,7 +195,7 @@ def main() -> int:
     _C.check(_C.lib().vtkv_set_head_major({"auto": -1, "on": 1, "off": 0}[args.head_major]))
     B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
     K, W = args.steps, args.warmup
-    R = args.repeats if args.repeats > 0 else (11 if K <= 50 else 3)
+    R = args.repeats if args.repeats > 0 else (21 if K <= 50 else 3)
     backend_path = args.host_path == "backend"
     L = args.layers if backend_path else 1
     torch.cuda.set_device(0)
