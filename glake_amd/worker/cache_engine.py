@@ -164,6 +164,24 @@ class CacheEngine:
         for key in keys:
             if key not in self._swapped:
                 raise _C.VtkvError(_C.ESTATE, f"sequence {key} is not swapped out")
+        try:
+            total = self._swap_in_copies(slots, keys)
+        except Exception:
+            # (the pool ran dry part of the way, most likely) the sequences stay swapped out, whole: copies already
+            # queued finish, and every slot of this call gives back what was mapped for it
+            torch.cuda.current_stream().synchronize()
+            for slot in slots:
+                self.vmm_kvcache_segment[slot].preempt_seq(slot)
+            raise
+        torch.cuda.current_stream().synchronize()  # the arena space is reused after this
+        for key in keys:
+            off, used = self._swapped.pop(key)
+            if used:
+                self._arena.release(off, 2 * self.num_layers * used)
+        return total
+
+    def _swap_in_copies(self, slots: Sequence[int], keys: Sequence) -> int:
+        total = 0
         src, dst, nbytes, queued = [], [], [], 0
         step = max(1, self.swap_in_map_bytes // self.chunk_bytes)   # chunks per range mapped between two rounds of copies
         for slot, key in zip(slots, keys):
@@ -201,11 +219,6 @@ class CacheEngine:
             seg.set_used_size(used)
         if src:
             ops.swap_ranges(src, dst, nbytes, "in")
-        torch.cuda.current_stream().synchronize()  # the arena space is reused after this
-        for key in keys:
-            off, used = self._swapped.pop(key)
-            if used:
-                self._arena.release(off, 2 * self.num_layers * used)
         return total
 
     # ------------------------------------------------------------------ block-wise API of the reference

@@ -165,3 +165,55 @@ def test_swap_out_into_a_full_arena_changes_nothing(gpu_pool):
         eng.swap_in([slot])
     resident_bytes_intact()
     eng.close()
+
+
+def test_swap_in_that_finds_the_pool_empty_leaves_the_sequences_swapped_out(gpu_pool):
+    """Two sequences are swapped out and somebody else takes the chunks in between: swapping both in fails part
+    of the way, both stay in host memory and their slots hold nothing, and once the chunks are back the same call
+    succeeds with every byte in place."""
+    import torch
+
+    from glake_amd import _C
+    from glake_amd.worker.cache_engine import CacheEngine
+
+    vmm = gpu_pool
+    vmm.trim()
+    free0 = vmm.showFreeBlocks()
+    hkv, d, layers = 8, 128, 2
+    row = hkv * d * 2
+    tokens = {0: 2500, 1: 1800}                            # 3 and 2 chunks per range
+    eng = CacheEngine(num_layers=layers, num_kv_heads=hkv, head_size=d, dtype=torch.bfloat16, max_num_seqs=2,
+                      max_num_batched_tokens=3000, swap_space_bytes=64 << 20)
+    rng = np.random.default_rng(4)
+    data = {}
+    for slot, n in tokens.items():
+        seg = eng.vmm_kvcache_segment[slot]
+        seg.ensure_mapped(n * row)
+        seg.set_used_size(n * row)
+        for l in range(layers):
+            for which, base in (("k", seg.getKeyDevicePtr(l)), ("v", seg.getValueDevicePtr(l))):
+                buf = rng.integers(0, 256, n * row, dtype=np.uint8)
+                _C.check(_C.lib().vtkv_memcpy_h2d(base, buf.ctypes.data, buf.nbytes))
+                data[(slot, l, which)] = buf
+    eng.swap_out([0, 1])
+    assert vmm.showFreeBlocks() == free0
+    # a hog leaves enough for the first sequence (3 chunks x 2 ranges x 2 layers) but not for the second
+    spare = vmm.showFreeBlocks()
+    hog = vmm.KVcacheSegment(1, (spare // 2 + 2) * CHUNK, 0, False)
+    hog.expandMultiSegment((spare - 14) // 2)
+    with pytest.raises(_C.VtkvOutOfChunks):
+        eng.swap_in([0, 1])
+    assert sorted(eng._swapped) == [0, 1]
+    assert [s.actual_size for s in eng.vmm_kvcache_segment] == [0, 0] and [s.used_size for s in eng.vmm_kvcache_segment] == [0, 0]
+    hog.destroy()
+    eng.swap_in([0, 1])
+    assert eng._swapped == {}
+    for (slot, l, which), buf in data.items():
+        seg = eng.vmm_kvcache_segment[slot]
+        base = seg.getKeyDevicePtr(l) if which == "k" else seg.getValueDevicePtr(l)
+        back = np.empty_like(buf)
+        _C.check(_C.lib().vtkv_memcpy_d2h(back.ctypes.data, base, buf.nbytes))
+        assert np.array_equal(back, buf), (slot, l, which)
+    eng.close()
+    vmm.trim()
+    assert vmm.showFreeBlocks() == free0
