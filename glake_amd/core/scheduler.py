@@ -8,9 +8,15 @@ last sequence of the queue -> ``append_slots`` fills ``extend_list``), ``:726-76
 ``can_allocate`` / ``allocate`` give a prompt its slot), ``:781-873`` (``_schedule_default``: prompts first, and
 no decodes in a step that runs prompts), ``:1160-1225`` (preemption by recompute or by swap), and the engine's
 bookkeeping around a step, ``vllm/engine/llm_engine.py:607-618`` (release the slots of finished sequences) and
-``:686-701`` (unmap the preempted slots before the model runs).  Sequence groups, LoRA, beam search, chunked
-prefill and the prefix-cache branch are left out: one sequence per request, prompts and decodes in separate
-steps, as the fork runs.
+``:686-701`` (unmap the preempted slots before the model runs).  Sequence groups, LoRA, beam search and chunked
+prefill are left out: one sequence per request, prompts and decodes in separate steps, as the fork runs.
+
+The prefix-cache branch of ``_schedule_prefills`` (``scheduler.py:726-766``) is there in the form the reference
+sketches and switches off (it looks up the empty prompt, ``:728``, and never inserts, ``:1097``): with a
+``prefix_lookup`` a prompt that begins with a cached prefix is admitted with ``prefix_rows`` of its rows already
+in place -- at least one token is left to run (``:757-766``) -- and the step computes only the rest.  Here the
+prompt still gets a slot of its own, which the step loop starts from the cached prefix by mapping the prefix's
+chunks a second time; the reference would hand the cached slot itself to the new sequence (``set_slot``).
 
 The objects here only count; the GPU side (``CacheEngine``, ``prepare_step``, the attention backend) is driven
 from their output by :class:`glake_amd.worker.step_loop.StepLoop`.
@@ -20,7 +26,7 @@ from __future__ import annotations
 import enum
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, List, Optional
+from typing import Callable, Deque, List, Optional, Sequence, Tuple
 
 from .chunk_manager import AllocStatus, ChunkSpaceManager, SequenceChunks
 
@@ -51,6 +57,8 @@ class Request:
     preemptions: int = 0
     swap_slot: int = -1     # swapped out in this step: the slot its rows are still in
     final_slot: int = -1    # finished: the slot to release
+    token_ids: Optional[Sequence[int]] = None  # the prompt's tokens, for the prefix lookup (None: never looked up)
+    prefix_rows: int = 0    # rows of the coming prompt run that a cached prefix provides (set at admission)
 
     @property
     def total_len(self) -> int:
@@ -75,6 +83,8 @@ class SchedulerOutputs:
     swapped_in: List[Request] = field(default_factory=list)    # brought back before the step (they also decode)
     ignored: List[Request] = field(default_factory=list)
     recompute: List[Request] = field(default_factory=list)     # preempted by recompute: back at the head of waiting
+    # prompts of this step that start from a cached prefix: (request, holder of the prefix, rows)
+    prefix_hits: List[Tuple[Request, object, int]] = field(default_factory=list)
     num_batched_tokens: int = 0
 
     def is_empty(self) -> bool:
@@ -86,11 +96,13 @@ class StepScheduler:
 
     ``token_size``: bytes of one token row of one range; ``value_skew``: what the engine sets the V rows off
     by (claimed with the first rows, as ``SequenceChunks`` does); ``preemption``: what happens to a sequence
-    that loses its chunks."""
+    that loses its chunks; ``prefix_lookup(tokens) -> (holder, rows)``: the longest cached prefix of a prompt
+    (``(None, 0)`` if none), e.g. ``PrefixStore.lookup``."""
 
     def __init__(self, manager: ChunkSpaceManager, token_size: int, max_num_seqs: int, max_num_batched_tokens: int,
                  chunk_bytes: int = 2 << 20, value_skew: int = 0,
-                 preemption: PreemptionMode = PreemptionMode.RECOMPUTE, max_model_len: Optional[int] = None):
+                 preemption: PreemptionMode = PreemptionMode.RECOMPUTE, max_model_len: Optional[int] = None,
+                 prefix_lookup: Optional[Callable[[Sequence[int]], Tuple[object, int]]] = None):
         self.block_manager = manager
         self.token_size = int(token_size)
         self.max_num_seqs = int(max_num_seqs)
@@ -98,6 +110,7 @@ class StepScheduler:
         self.chunk_bytes = int(chunk_bytes)
         self.value_skew = int(value_skew)
         self.preemption = preemption
+        self.prefix_lookup = prefix_lookup
         # scheduler.py:297-303: a prompt longer than this is ignored
         self.prompt_limit = min(max_model_len or max_num_batched_tokens, max_num_batched_tokens)
         self.waiting: Deque[Request] = deque()
@@ -108,10 +121,12 @@ class StepScheduler:
         self._next_id = 0
 
     # ------------------------------------------------------------------ requests
-    def add_request(self, prompt_len: int, max_new_tokens: int) -> Request:
+    def add_request(self, prompt_len: int, max_new_tokens: int, token_ids: Optional[Sequence[int]] = None) -> Request:
         if prompt_len <= 0 or max_new_tokens <= 0:
             raise ValueError("a request needs at least one prompt token and one token to generate")
-        req = Request(self._next_id, int(prompt_len), int(max_new_tokens))
+        if token_ids is not None and len(token_ids) != prompt_len:
+            raise ValueError("token_ids must hold the prompt's tokens")
+        req = Request(self._next_id, int(prompt_len), int(max_new_tokens), token_ids=token_ids)
         self._next_id += 1
         self.waiting.append(req)
         return req
@@ -135,10 +150,19 @@ class StepScheduler:
                 out.ignored.append(req)
                 self.waiting.popleft()
                 continue
+            if num_curr_seqs + 1 > self.max_num_seqs:
+                break
+            # scheduler.py:726-766: rows a cached prefix provides need not be run; one token always is
+            # (the lookup may cut a holder for the matched length: only asked once a slot could be had)
+            holder, rows = None, 0
+            if self.prefix_lookup is not None and req.token_ids is not None:
+                holder, rows = self.prefix_lookup(req.token_ids)
+                rows = min(int(rows), req.total_len - 1) if holder is not None else 0
+            num_new_tokens -= rows
             if (out.num_batched_tokens + num_new_tokens > self.max_num_batched_tokens
                     or num_curr_seqs + 1 > self.max_num_seqs):
                 break
-            chunks = self._new_chunks(num_new_tokens)
+            chunks = self._new_chunks(req.total_len)  # (a shared prefix is claimed in full: an upper bound)
             can = self.block_manager.can_allocate(chunks, self.preempted_flag)
             if can is AllocStatus.LATER:
                 break
@@ -152,6 +176,9 @@ class StepScheduler:
             req.chunks = chunks
             req.status = SeqStatus.RUNNING
             req.num_cached = 0
+            req.prefix_rows = rows
+            if rows:
+                out.prefix_hits.append((req, holder, rows))
             self.waiting.popleft()
             out.prompts.append(req)
             out.num_batched_tokens += num_new_tokens

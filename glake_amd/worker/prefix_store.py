@@ -9,7 +9,7 @@ at its end is copied.  A chunk returns to the pool when the last slot that maps 
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence, Tuple
+from typing import Callable, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -19,28 +19,55 @@ from .cache_engine import CacheEngine
 
 class PrefixStore:
     """``cache_slots``: the slots of ``engine`` that hold cached prefixes (the scheduler must not hand them to
-    running sequences)."""
+    running sequences).  ``room() -> int``: physical chunks the store may still take from the pool (below zero:
+    it holds chunks that running sequences have been promised); None: whatever the pool has.  A new holder takes
+    chunks only for the partly filled end of its prefix; the store evicts least recently used prefixes to stay
+    within ``room``, and a prefix that cannot be had that way is not cached (``keep``) or not found (``lookup``)."""
 
-    def __init__(self, engine: CacheEngine, cache_slots: Sequence[int]):
+    def __init__(self, engine: CacheEngine, cache_slots: Sequence[int], room: Optional[Callable[[], int]] = None):
         self.engine = engine
+        self.room = room
         self.token_size = engine.token_size
         self.free_slots: List[int] = list(cache_slots)
         self.rows = {}                                   # cache slot -> rows it holds
         self.tree = RadixCache(self.token_size, self._split)
+        self.evicted_rows = 0                            # rows of all holders evicted so far
+        self._pinned = []                                # nodes looked up in this step: not evicted before end_step
 
     def _stream(self) -> int:
         return torch.cuda.current_stream().cuda_stream
 
-    def _take_slot(self) -> int:
+    def _own_chunks(self, nbytes: int) -> int:
+        """Chunks a holder of ``nbytes`` bytes per range takes from the pool: what lies behind the prefix's whole
+        chunks, up to the end of its V rows, in every K and V range."""
+        gran = self.engine.chunk_bytes
+        tail = nbytes + self.engine.value_skew - (nbytes // gran) * gran if nbytes else 0
+        return 2 * self.engine.num_layers * ((tail + gran - 1) // gran)
+
+    def _take_slot(self, nbytes: int) -> int:
         if not self.free_slots:
             self.evict(1)                                # the least recently used prefix nobody refers to
         if not self.free_slots:
             raise RuntimeError("no slot left for a cached prefix: every cached prefix is in use")
+        need = self._own_chunks(nbytes)
+        while self.room is not None and self.room() < need:
+            if self.evict(1) == 0:
+                raise RuntimeError("no chunks left for a cached prefix")
         return self.free_slots.pop()
+
+    def make_room(self) -> int:
+        """Evict until ``room()`` is not negative (or nothing is left to evict).  Returns the rows evicted."""
+        gone = 0
+        while self.room is not None and self.room() < 0:
+            rows = self.evict(1)
+            if rows == 0:
+                break
+            gone += rows
+        return gone
 
     def _split(self, slot: int, nbytes: int) -> int:
         """The holder of the first ``nbytes`` bytes of what ``slot`` holds (radix_cache.py:184)."""
-        new = self._take_slot()
+        new = self._take_slot(nbytes)
         segs = self.engine.vmm_kvcache_segment
         segs[new].share_prefix(segs[slot], nbytes, self._stream())
         self.rows[new] = nbytes // self.token_size
@@ -50,10 +77,22 @@ class PrefixStore:
     def lookup(self, tokens: Sequence[int]) -> Tuple[Optional[int], int]:
         """(cache slot, rows) of the longest cached prefix of ``tokens`` that leaves at least one token to
         run (scheduler.py:757-766 runs ``prefix_len - 1`` cached tokens when the whole prompt is cached)."""
-        slot, n = self.tree.match_prefix(tokens)
-        if slot is None:
+        try:
+            node = self.tree.match_node(tokens)          # (cuts a holder when the match ends inside an edge)
+        except RuntimeError:                             # no slot or no chunks for the cut: the tree is as it was
             return None, 0
-        return slot, min(n, len(tokens) - 1)
+        if node is self.tree.root_node:
+            return None, 0
+        # a later lookup of the same step may have to evict for room: not what this one has just handed out
+        self.tree.inc_ref_counter(node)
+        self._pinned.append(node)
+        return node.value[0], min(node.prefix_len, len(tokens) - 1)
+
+    def end_step(self) -> None:
+        """The step has started its sequences from what the lookups handed out: those holders may go again."""
+        for node in self._pinned:
+            self.tree.dec_ref_counter(node)
+        self._pinned = []
 
     def start_from(self, run_slot: int, cache_slot: int, rows: int) -> None:
         """Begin the (empty) running slot with ``rows`` cached rows of ``cache_slot``."""
@@ -65,7 +104,7 @@ class PrefixStore:
         how many leading tokens the tree had already."""
         if len(tokens) == 0:
             return 0
-        new = self._take_slot()
+        new = self._take_slot(len(tokens) * self.token_size)
         segs = self.engine.vmm_kvcache_segment
         segs[new].share_prefix(segs[run_slot], len(tokens) * self.token_size, self._stream())
         self.rows[new] = len(tokens)
@@ -87,4 +126,6 @@ class PrefixStore:
 
     def evict(self, num_tokens: int) -> int:
         """Free cached prefixes, least recently used first, until ``num_tokens`` rows' worth is gone."""
-        return self.tree.evict(num_tokens, lambda value: self._drop(value[0]))
+        rows = self.tree.evict(num_tokens, lambda value: self._drop(value[0]))
+        self.evicted_rows += rows
+        return rows

@@ -11,6 +11,14 @@
 4. every scheduled sequence gets its sampled token accounted, and finished sequences release their slots
    (``release_seq``).
 
+With a ``PrefixStore`` the loop also runs the prefix-cache branch that the reference sketches
+(``vllm/core/scheduler.py:726-766``, ``vmm_allocator/radix_cache.py``): the scheduler looks every new prompt up,
+a prompt that begins with a cached prefix has its slot started from the prefix's holder before the model runs
+(whole chunks mapped a second time) and computes only the remaining rows, and a finished request's prompt rows
+are kept as a new holder.  Holders take physical chunks that the manager does not count, so the loop tells the
+store how many it may take (what the pool has beyond everything the manager has handed out or may still hand
+out) and has it evict when a release leaves it above that.
+
 The model itself (projections, sampling) is not part of this package: ``run_model(metadata, outputs)`` is the
 caller's, and it calls ``VTensorImpl.forward`` once per layer with ``engine.gpu_cache[layer]``.
 """
@@ -21,9 +29,11 @@ from typing import Callable, List, Optional
 
 import torch
 
+from .. import vmm_allocator as vmm
 from ..attention.backends.vtensor import VTensorBackend, VTensorMetadata
 from ..core.scheduler import Request, SchedulerOutputs, StepScheduler
 from .cache_engine import CacheEngine
+from .prefix_store import PrefixStore
 from .step import prepare_step
 
 
@@ -35,10 +45,44 @@ class StepResult:
 
 
 class StepLoop:
-    def __init__(self, engine: CacheEngine, scheduler: StepScheduler, device: Optional[torch.device] = None):
+    """``prefix_store``: cached prefixes in slots of ``engine`` beyond the manager's ``max_seqs`` (requests need
+    ``token_ids`` to take part).  ``pool_chunks``: physical chunks (all layers, K and V) that the engine and the
+    store may take from the pool from now on; by default all that is free now."""
+
+    def __init__(self, engine: CacheEngine, scheduler: StepScheduler, device: Optional[torch.device] = None,
+                 prefix_store: Optional[PrefixStore] = None, pool_chunks: Optional[int] = None):
         self.engine = engine
         self.scheduler = scheduler
         self.device = torch.device("cuda", engine.device) if device is None else device
+        self.prefix_store = prefix_store
+        if prefix_store is not None:
+            mgr = scheduler.block_manager
+            if mgr.cache_token:
+                raise ValueError("a prompt that starts from a cached prefix needs an empty slot: no pre-mapped slots")
+            if any(s < mgr.max_seqs for s in prefix_store.free_slots):
+                raise ValueError("the prefix store's slots must lie beyond the slots the manager hands out")
+            free = vmm.showFreeBlocks()
+            pool_chunks = free if pool_chunks is None else int(pool_chunks)
+            if pool_chunks > free or pool_chunks < engine.num_layers * mgr.get_num_free_gpu_blocks():
+                raise ValueError("pool_chunks must cover the manager's chunks in every layer and be free in the pool")
+            self._pool_floor = free - pool_chunks       # free chunks of the pool that are not this loop's
+            prefix_store.room = self.prefix_room
+            if scheduler.prefix_lookup is None:
+                scheduler.prefix_lookup = prefix_store.lookup
+
+    def prefix_room(self) -> int:
+        """Physical chunks the prefix store may still take: what the pool has free (counting what slots that no
+        sequence owns any more are about to give back), less what the manager may still hand out and what it has
+        handed out to slots that have not mapped it yet."""
+        eng, mgr = self.engine, self.scheduler.block_manager
+        owed = mgr.get_num_free_gpu_blocks()
+        for slot in range(mgr.max_seqs):
+            mapped = 2 * (eng.vmm_kvcache_segment[slot].actual_size // eng.chunk_bytes)
+            if mgr.kv_cache_slot[slot]:
+                owed += max(0, mgr.block_tables[slot] - mapped)
+            else:
+                owed -= mapped
+        return vmm.showFreeBlocks() - self._pool_floor - eng.num_layers * owed
 
     def build_metadata(self, out: SchedulerOutputs) -> VTensorMetadata:
         """model_runner.py:595-622: prompts first, then decodes; per-sequence slot ids; ``extend_seq_list``
@@ -49,17 +93,22 @@ class StepLoop:
         seq_lens = [r.total_len for r in seqs]
         n_pre = len(out.prompts)
         grow = set(out.extend_list)
+        # a prompt behind a cached prefix runs the rows after it (scheduler.py:757-766)
+        cached = [r.prefix_rows for r in out.prompts] + [0] * len(out.decodes)
+        query_lens = [n - c for n, c in zip(seq_lens[:n_pre], cached)]
         meta = VTensorBackend.make_metadata(
-            num_prefills=n_pre, num_prefill_tokens=sum(seq_lens[:n_pre]), num_decode_tokens=len(out.decodes),
+            num_prefills=n_pre, num_prefill_tokens=sum(query_lens), num_decode_tokens=len(out.decodes),
             slot_mapping=torch.tensor(slots, dtype=torch.int64, device=dev), seq_lens=seq_lens,
             seq_lens_tensor=torch.tensor(seq_lens, dtype=torch.int32, device=dev),
-            max_query_len=max(seq_lens[:n_pre]) if n_pre else None,
+            max_query_len=max(query_lens) if n_pre else None,
             max_prefill_seq_len=max(seq_lens[:n_pre]) if n_pre else 0,
             max_decode_seq_len=max(seq_lens[n_pre:]) if out.decodes else 0, query_start_loc=None, seq_start_loc=None,
             context_lens_tensor=None, block_tables=None, is_extend=int(bool(grow)), kv_batch_stride=eng.kv_batch_stride,
             kv_num_heads=eng.num_kv_heads, kv_head_size=eng.head_size, max_seq_len=max(seq_lens),
-            slot_mapping_list=slots, set_used_size=[0] * len(slots),
+            slot_mapping_list=slots, set_used_size=cached if any(cached) else [0] * len(slots),
             extend_seq_list=[s if s in grow else -1 for s in slots], use_cuda_graph=False)
+        if any(cached):
+            meta.query_lens = query_lens
         meta.k_cache_segment_ptr_list = eng.k_cache_ptr          # model_runner.py:749-755
         meta.v_cache_segment_ptr_list = eng.v_cache_ptr
         meta.kvcache_segment = [eng.vmm_kvcache_segment[s] for s in slots]
@@ -77,6 +126,13 @@ class StepLoop:
                 eng.vmm_kvcache_segment[slot].preempt_seq(slot)
         if out.swapped_out:                                               # worker.py:213-225
             eng.swap_out([r.swap_slot for r in out.swapped_out], keys=[("req", r.request_id) for r in out.swapped_out])
+        store = self.prefix_store
+        if store is not None:
+            for req, holder, rows in out.prefix_hits:                     # the slot begins as the prefix
+                store.start_from(req.slot, holder, rows)
+            store.end_step()
+            if out.recompute or out.swapped_out:
+                store.make_room()      # a slot that shared a holder's chunks gave the pool less than its claim
         if out.swapped_in:
             eng.swap_in([r.slot for r in out.swapped_in], keys=[("req", r.request_id) for r in out.swapped_in])
         meta = None
@@ -88,5 +144,12 @@ class StepLoop:
         if finished:                                                      # llm_engine.py:607-618
             stream.synchronize()                                          # the step's kernels have read the ranges
             for req in finished:
+                if store is not None and req.token_ids is not None:
+                    try:                                                  # the prompt's rows stay as a cached prefix
+                        store.keep(req.token_ids, req.final_slot)
+                    except RuntimeError:                                  # no slot or no chunks for it: not cached
+                        pass
                 eng.vmm_kvcache_segment[req.final_slot].release_seq(req.final_slot)
+            if store is not None:
+                store.make_room()
         return StepResult(out, meta, finished)

@@ -58,6 +58,7 @@ def test_three_prompts_with_nested_shared_prefixes(gpu_pool):
         assert cached == expect_cached
         if cached:
             store.start_from(run_slot, cache_slot, cached)
+        store.end_step()                                  # (a lookup keeps its holder from eviction until then)
         n, nq = len(tokens), len(tokens) - cached
         meta = VTensorBackend.make_metadata(
             num_prefills=1, num_prefill_tokens=nq, num_decode_tokens=0,
@@ -128,8 +129,11 @@ def test_three_prompts_with_nested_shared_prefixes(gpu_pool):
     # a fourth lookup of a cached prompt in full runs its last token only
     slot, n = store.lookup(tok_a)
     assert n == len(tok_a) - 1 and store.rows[slot] == len(tok_a)
+    # B's and C's holders go; not the one the lookup handed out, nor the cuts that lead to it
+    assert store.evict(10 ** 9) == 3000 + 1324
+    store.end_step()
     # eviction frees every holder; shared chunks go back with their last user
-    assert store.evict(10 ** 9) == 3000 + 2500 + 3000 + 1024 + 1324
+    assert store.evict(10 ** 9) == 3000 + 2500 + 1024
     assert vmm.sharedBlocks() == 0 and sorted(store.free_slots) == [3, 4, 5, 6, 7]
     eng.close()
     assert vmm.showFreeBlocks() == free0

@@ -154,3 +154,68 @@ def test_random_traffic_conserves_chunks_and_finishes_everything(mode, seed):
         if r.status is SeqStatus.FINISHED:
             assert r.generated == r.max_new_tokens
     assert mgr.get_num_free_gpu_blocks() == 20
+
+
+def test_a_prompt_behind_a_cached_prefix_is_charged_for_the_rest_only():
+    """scheduler.py:726-766: the token budget counts the rows that still have to run, at least one token runs,
+    the chunks of the whole prompt are claimed, and the lookup is not asked when no slot is free."""
+    cached = {tuple(range(600)): ("holder-a", 600)}
+    asked = []
+
+    def lookup(tokens):
+        asked.append(len(tokens))
+        for key, (holder, rows) in cached.items():
+            if tuple(tokens[:len(key)]) == key:
+                return holder, min(rows, len(tokens) - 1)
+        return None, 0
+
+    mgr = ChunkSpaceManager(3, 40, watermark=0.0)
+    s = StepScheduler(mgr, ROW, 3, 1000, prefix_lookup=lookup)
+    a = s.add_request(900, 3, token_ids=list(range(900)))            # 600 cached: 300 rows to run
+    b = s.add_request(600, 3, token_ids=list(range(600)))            # cached in full: its last token runs
+    c = s.add_request(650, 3, token_ids=list(range(5000, 5650)))     # nothing cached
+    d = s.add_request(500, 3)                                         # no tokens given: never looked up
+    out = s.schedule()
+    # 300 + 1 + 650 = 951 of 1000 tokens; the fourth prompt finds no slot and is not looked up
+    assert [r.request_id for r in out.prompts] == [0, 1, 2] and out.num_batched_tokens == 951
+    assert [(r.request_id, h, n) for r, h, n in out.prefix_hits] == [(0, "holder-a", 600), (1, "holder-a", 599)]
+    assert (a.prefix_rows, b.prefix_rows, c.prefix_rows) == (600, 599, 0) and asked == [900, 600, 650]
+    # the claim is for the whole prompt: 900 + 100 rows of slack -> one chunk pair, as without a prefix
+    assert a.chunks.get_logical_block_num() == 2 and mgr.block_tables[a.slot] == 2
+    s.on_step_done(out)
+    assert (a.num_cached, b.num_cached) == (900, 600)
+    for _ in range(2):
+        s.on_step_done(s.schedule())
+    out = s.schedule()
+    assert [r.request_id for r in out.prompts] == [3] and not out.prefix_hits and asked == [900, 600, 650]
+    # without the prefix the first two prompts alone pass the budget of 1000 tokens
+    s2 = StepScheduler(ChunkSpaceManager(3, 40, watermark=0.0), ROW, 3, 1000)
+    s2.add_request(900, 3, token_ids=list(range(900)))
+    s2.add_request(600, 3, token_ids=list(range(600)))
+    assert [r.request_id for r in s2.schedule().prompts] == [0]
+
+
+def test_a_recomputed_sequence_is_looked_up_again_with_its_prompt():
+    rows = {"n": 0}
+
+    def lookup(tokens):
+        return ("h", min(rows["n"], len(tokens) - 1)) if rows["n"] else (None, 0)
+
+    mgr = ChunkSpaceManager(2, 4, watermark=0.0)
+    s = StepScheduler(mgr, ROW, 2, 4096, prefix_lookup=lookup)
+    a = s.add_request(900, 400, token_ids=list(range(900)))
+    b = s.add_request(900, 400, token_ids=list(range(1000, 1900)))
+    s.on_step_done(s.schedule())
+    rows["n"] = 900                                        # from now on every prompt is cached in full
+    for _ in range(400):
+        out = s.schedule()
+        s.on_step_done(out)
+        if out.recompute:
+            break
+    assert out.recompute == [b] and b.generated > 0        # both outgrew their chunk; the pool has no third pair
+    while b.status is not SeqStatus.RUNNING:
+        out = s.schedule()
+        s.on_step_done(out)
+    # its prompt's 900 tokens are cached, the tokens it had generated are run again behind them
+    assert out.prompts == [b] and b.prefix_rows == 899 and out.prefix_hits == [(b, "h", 899)]
+    assert out.num_batched_tokens == b.num_cached - 899
