@@ -108,7 +108,8 @@ struct AttnParams {
   void *out;           // [B,Hq,D] bf16, or fp32 when out_f32
   int out_f32;
   int64_t q_stride;
-  int num_seqs, num_heads, num_kv_heads, group;  // B, Hq, Hkv, G
+  int num_seqs, num_heads, num_kv_heads, group;  // B, Hq, Hkv, G (kv heads and heads of each as the kernels see them)
+  int kv_split, group_real;  // see first_head_of: > 1 when a kv head has more than 16 query heads
   int head_size;    // D as the caller's tensors have it (the kernels hold it padded to their tile sizes)
   int out_f16;      // 16-bit outputs are fp16 (else bf16)
   int span_tiles;   // tiles per workgroup; 0 = all tiles / gridDim.x
@@ -170,12 +171,16 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 // size that is no multiple of the MFMA depth is held padded (80 as 96, 112 as 128; with fp8 rows, whose pieces
 // carry 16 elements, 80, 96 and 112 as 128): the padding of the K and V tiles in LDS is cleared once and q is
 // zero there, so padded columns add nothing to the logits and yield output columns that are never stored.
-template <bool ALIBI, bool FP8, bool APPEND, int HPS, int D = 128, bool F16 = false>
+//
+// SPLIT: some kv head has more than 16 query heads and is served in parts (see first_head_of); the variants
+// without it index heads as kv head * group and carry none of that arithmetic.
+template <bool ALIBI, bool FP8, bool APPEND, int HPS, int D = 128, bool F16 = false, bool SPLIT = false>
 __global__ void __launch_bounds__(kThreads)
     __attribute__((amdgpu_waves_per_eu(D > 128 ? 1 : (FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES))))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
   static_assert(D % 16 == 0 && D >= 64 && D <= 256, "head sizes are multiples of 16 from 64 to 256");
   static_assert(!APPEND || D == 128, "the fused append is built for head size 128 only");
+  static_assert(!SPLIT || HPS == 1, "a segment of several kv heads is never one of split kv heads");
   constexpr int kHD = FP8 ? (D + 63) / 64 * 64 : (D + 31) / 32 * 32;  // head size as held in LDS and registers
   constexpr int kKSteps = kHD / 32;                                  // MFMA steps of S^T = K.Q^T
   constexpr int kDBlocks = kHD / 16;                                 // 16-row blocks of O^T
@@ -316,7 +321,7 @@ __global__ void __launch_bounds__(kThreads)
   constexpr int kLoads = (kTilePieces + 63) / 64;    // load j of lane l takes piece 64 j + l, i.e. row (64 j + l) / kPieces
   constexpr bool kEvenLoads = kTilePieces % 64 == 0; // every load of every lane carries a piece of the tile
   constexpr int kKa = FP8 ? kHD / 64 : kKSteps;      // 16-byte A-operand pieces a lane reads back per K tile
-  const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;  // bytes between consecutive tokens
+  const uint32_t row_stride = (uint32_t)(SPLIT ? Hkv / p.kv_split : Hkv) * kKvRowBytes;  // bytes between consecutive tokens
   char *v_tile = smem + wave * kTileBytes;
   char *k_tile = smem + kWaves * kTileBytes + 1024 + wave * kTileBytes;
   // tile layouts in LDS (see vtkv_attn_common.h for the swizzles), with this head size's row pitch
@@ -350,12 +355,22 @@ __global__ void __launch_bounds__(kThreads)
     // the tables hold plain integers: say explicitly that they are global-memory addresses, otherwise
     // the loads become flat loads that also count on the LDS wait counter and defeat the prefetch
     const int64_t slot = p.slot_ids[b];
-    gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
-    gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
+    // (virtual kv heads of one kv head read the same rows; with the fused append each of them stores the new
+    // row, the same bytes at the same place)
+    // this wave's kv head in memory and its query heads [head0, head0 + n_heads)
+    int kv_real = kvh, head0 = kvh * G, n_heads = G;
+    if constexpr (SPLIT) {
+      kv_real = kvh / p.kv_split;
+      const int part = kvh - kv_real * p.kv_split;
+      head0 = kv_real * p.group_real + part * G;
+      n_heads = min(G, p.group_real - part * G);
+    }
+    gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kv_real * kKvRowBytes;
+    gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kv_real * kKvRowBytes;
     gptr nk_base = k_base, nv_base = v_base;
     if (APPEND) {
-      nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kvh * (2 * D);
-      nv_base = (gptr)(uintptr_t)p.new_v + (int64_t)b * p.new_v_stride + kvh * (2 * D);
+      nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kv_real * (2 * D);
+      nv_base = (gptr)(uintptr_t)p.new_v + (int64_t)b * p.new_v_stride + kv_real * (2 * D);
     }
 
     // B operand of S^T = K.Q^T: for MFMA step ks lane (n, g) holds the eight q[head n][d] whose K
@@ -364,18 +379,18 @@ __global__ void __launch_bounds__(kThreads)
     // padded heads.
     u32x4 qop[kKSteps];
     {
-      const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(kvh * G + (n < G ? n : 0)) * D;
+      const uint16_t *qrow = p.q + (int64_t)b * p.q_stride + (int64_t)(head0 + (n < n_heads ? n : 0)) * D;
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
         const int d0 = FP8 ? (ks >> 1) * 64 + g * 16 + (ks & 1) * 8 : ks * 32 + g * 8;
         u32x4 raw = (u32x4){0, 0, 0, 0};
         if (kHD == D || d0 < D) raw = *reinterpret_cast<const u32x4 *>(qrow + d0);  // (pieces are all in or all out)
-        if (n >= G) raw = (u32x4){0, 0, 0, 0};
+        if (n >= n_heads) raw = (u32x4){0, 0, 0, 0};
         qop[ks] = raw;
       }
     }
     float slope_log2 = 0.f;
-    if (ALIBI) slope_log2 = (n < G && p.alibi_slopes) ? p.alibi_slopes[kvh * G + n] * kLog2e : 0.f;
+    if (ALIBI) slope_log2 = (n < n_heads && p.alibi_slopes) ? p.alibi_slopes[head0 + n] * kLog2e : 0.f;
 
     f32x4 acc[kDBlocks];
 #pragma unroll
@@ -647,7 +662,7 @@ __global__ void __launch_bounds__(kThreads)
     const int w0 = first_tile / span, w1 = (first_tile + nt_b - 1) / span;
     const bool whole = p.fused_merge && w0 == w1;  // no other workgroup: the result is final
     auto store_out = [&](int kv_head, int head, int d, float r) {
-      const int64_t oi = ((int64_t)b * p.num_heads + kv_head * G + head) * D + d;
+      const int64_t oi = ((int64_t)b * p.num_heads + (SPLIT ? head0 : kv_head * G) + head) * D + d;
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
@@ -672,6 +687,7 @@ __global__ void __launch_bounds__(kThreads)
         if (kHD != D && d >= D) continue;  // a padded column
         const int head = h0 + hh;
         const int kv_head = kvg * kHps + sd;
+        const bool real_head = !SPLIT || head < n_heads;  // (the last part of a split kv head may have fewer)
         const float mw = head_max(sd, head);
         float lsum = 0.f, o = 0.f;
 #pragma unroll
@@ -681,10 +697,10 @@ __global__ void __launch_bounds__(kThreads)
           o += sm_o[(w * 8 + hh) * kHD + d];
         }
         const float o_norm = o / lsum;
-        if (aligned && p.v2_tmp_out) {
+        if (aligned && p.v2_tmp_out && real_head) {
           // the reference's per-partition outputs: max logit in natural units, sum of exponentials, and the
           // partition's normalised result in the model's dtype (csrc/attention/attention_kernels.cu:404-419)
-          const int64_t vi = ((int64_t)b * p.num_heads + kv_head * G + head) * aligned + v2_part;
+          const int64_t vi = ((int64_t)b * p.num_heads + (SPLIT ? head0 : kv_head * G) + head) * aligned + v2_part;
           p.v2_tmp_out[vi * D + d] = f32_to_16<F16>(o_norm * p.v_scale);
           if (d == 0) {
             p.v2_max_logits[vi] = mw * 0.6931471805599453f;
@@ -692,7 +708,7 @@ __global__ void __launch_bounds__(kThreads)
           }
         }
         if (whole) {
-          store_out(kv_head, head, d, o_norm * p.v_scale);
+          if (real_head) store_out(kv_head, head, d, o_norm * p.v_scale);
           continue;
         }
         // (head-major order: (segment's kv heads, sequence, head inside the segment) is what grows along it)
@@ -815,7 +831,12 @@ __global__ void __launch_bounds__(kThreads)
       }
       const float r = o / wsum * p.v_scale;
       // segment = sequence * Hkv + kv head, so (segment * G + head) is (sequence * Hq + query head)
-      const int64_t oi = (seg * G + head) * D + d;
+      int64_t oi = (seg * G + head) * D + d;
+      if constexpr (SPLIT) {
+        const int bb = (int)seg / Hkv, kv_head = (int)seg - bb * Hkv;
+        if (head >= heads_of(p, kv_head)) continue;
+        oi = ((int64_t)bb * p.num_heads + first_head_of(p, kv_head) + head) * D + d;
+      }
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
@@ -838,7 +859,7 @@ __global__ void __launch_bounds__(kThreads)
 // four at a time in turn, so a group of eight heads is merged in one pass instead of two.
 // HD: the head size as the stream kernel pads it (the row length of a partial result); thread d handles
 // column d and stores it if it is a real one (d < p.head_size).
-template <int GROUPS, int HSETS, int HD = 128>
+template <int GROUPS, int HSETS, int HD = 128, bool SPLIT = false>
 __global__ void __launch_bounds__(HD * GROUPS * HSETS) decode_attn_reduce_kernel(AttnParams p) {
   static_assert(GROUPS == 1 || HSETS == 1, "head sets only without piece groups");
   constexpr int kD = HD;  // (shadows the library-wide 128 inside this kernel)
@@ -920,10 +941,10 @@ __global__ void __launch_bounds__(HD * GROUPS * HSETS) decode_attn_reduce_kernel
     if (grp != 0) continue;
 #pragma unroll
     for (int hh = 0; hh < 4; ++hh) {
-      if (h0 + hh >= G) break;
+      if (h0 + hh >= (SPLIT ? heads_of(p, kvh) : G)) break;
       if (d >= p.head_size) break;  // a padded column
       const float r = o[hh] / wsum[hh] * p.v_scale;
-      const int64_t oi = ((int64_t)b * p.num_heads + kvh * G + h0 + hh) * p.head_size + d;
+      const int64_t oi = ((int64_t)b * p.num_heads + (SPLIT ? first_head_of(p, kvh) : kvh * G) + h0 + hh) * p.head_size + d;
       if (p.out_f32)
         reinterpret_cast<float *>(p.out)[oi] = r;
       else
@@ -990,9 +1011,10 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16 + 24 + 2 + 18;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
-                                             // others, the fused append for fp16 at head size 128 (fp16 rows, fp8
-                                             // rows), 18 that stream several kv heads per segment at other shapes
+constexpr int kVariants = 16 + 24 + 2 + 18 + 28;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
+                                                  // others, the fused append for fp16 at head size 128 (fp16 rows,
+                                                  // fp8 rows), 18 that stream several kv heads per segment at other
+                                                  // shapes, 28 for kv heads of more than 16 query heads (SPLIT)
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
 int head_size_index(int head_size) {
@@ -1091,21 +1113,27 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   const bool f16 = q_dtype == VTKV_F16;
   const bool tuned = head_size == 128 && !f16;  // the shape the kernel was built around, with all its variants
   if (kv_dtype == VTKV_FP8_E4M3) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
-  const int group = num_heads / num_kv_heads;
-  VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
-  VTKV_REQUIRE(num_kv_heads <= kMaxKvHeads, "num_kv_heads %d exceeds %d", num_kv_heads, kMaxKvHeads);
+  // More than 16 query heads per kv head: the kernels see every kv head as kv_split virtual ones over the same
+  // rows, each with at most 16 of its query heads (see first_head_of).  From here on num_kv_heads and group are
+  // what the kernels see; kv_heads_real is what the rows in memory hold.
+  const int kv_heads_real = num_kv_heads, group_real = num_heads / num_kv_heads;
+  const int kv_split = vtkv_kv_split(group_real);
+  const int group = (group_real + kv_split - 1) / kv_split;
+  num_kv_heads = kv_heads_real * kv_split;
+  VTKV_REQUIRE(num_kv_heads <= kMaxKvHeads, "%d kv heads (as %d of at most 16 query heads each) exceed %d", kv_heads_real,
+               num_kv_heads, kMaxKvHeads);
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0,
                "q rows must be 16-byte aligned and at least num_heads*head_size apart");
   VTKV_REQUIRE(max_seq_len > 0, "max_seq_len must be > 0");
   // the kernel addresses rows of a range with 32-bit byte offsets
-  VTKV_REQUIRE((int64_t)max_seq_len * num_kv_heads * head_size * vtkv::elem_bytes(kv_dtype) < (1ll << 31),
+  VTKV_REQUIRE((int64_t)max_seq_len * kv_heads_real * head_size * vtkv::elem_bytes(kv_dtype) < (1ll << 31),
                "a sequence range of %d rows exceeds 2 GiB", max_seq_len);
   VTKV_REQUIRE(partition_tokens == 0 || (partition_tokens >= kWaves * kTile && partition_tokens % kTile == 0),
                "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
   if (append) {
     VTKV_REQUIRE(new_value != nullptr, "null argument");
     VTKV_REQUIRE(head_size == 128, "the fused append needs head size 128");
-    const int64_t row = (int64_t)num_kv_heads * head_size;
+    const int64_t row = (int64_t)kv_heads_real * head_size;
     VTKV_REQUIRE(key_stride >= row && value_stride >= row && key_stride % 8 == 0 && value_stride % 8 == 0 &&
                      (uintptr_t)new_key % 16 == 0 && (uintptr_t)new_value % 16 == 0,
                  "key/value rows must be 16-byte aligned and at least num_kv_heads*head_size apart");
@@ -1122,7 +1150,8 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   // num_seqs * num_kv_heads of `group` heads each, which the workspace (16 heads per workgroup) holds for
   // groups up to 8.
   const bool many_short = (int64_t)num_seqs * num_kv_heads >= 4096;
-  const bool pair = tuned && (fp8 ? VTKV_ATTN_FP8_PAIR != 0 : many_short) && num_kv_heads % 2 == 0 && group <= 8;
+  const bool pair = tuned && kv_split == 1 && (fp8 ? VTKV_ATTN_FP8_PAIR != 0 : many_short) && num_kv_heads % 2 == 0 &&
+                    group <= 8;
   int seg_heads = pair ? 2 : 1;
   // kernel variant of the tuned shape: bit 0 alibi, bit 1 fused append, bit 2 paired kv heads, bit 3 fp8; the
   // other head sizes and fp16 have one variant per (head size, type, cache type), ALiBi decided at run time
@@ -1137,11 +1166,14 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
     // HBM peak with one head per segment: head size 80 0.51, 96 0.60, 112 0.53, 64 0.72; fp8 rows 0.29 to 0.40.
     static const int kHeads16[6] = {2, 4, 2, 4, 1, 1}, kHeads8[6] = {4, 4, 4, 4, 2, 1};
     const int want = fp8 ? kHeads8[d_index] : kHeads16[d_index];
-    if (want > 1 && num_kv_heads % want == 0 && group * want <= 16) {
+    if (want > 1 && kv_split == 1 && num_kv_heads % want == 0 && group * want <= 16) {
       seg_heads = want;
       variant = head_size == 128 ? 58 + (append ? 1 : 0) : 42 + d_index * 4 + (f16 ? 2 : 0) + (fp8 ? 1 : 0);
     }
   }
+  // kv heads of more than 16 query heads: one variant per (head size, type, cache type), the fused append at 128
+  if (kv_split > 1)
+    variant = append ? 84 + (f16 ? 2 : 0) + (fp8 ? 1 : 0) : 60 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
 #define VTKV_ROW(F8, H)                                                                                      \
   decode_attn_stream_kernel<false, F8, false, H>, decode_attn_stream_kernel<true, F8, false, H>,             \
       decode_attn_stream_kernel<false, F8, true, H>, decode_attn_stream_kernel<true, F8, true, H>
@@ -1158,6 +1190,12 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
       VTKV_GROUPED(64, 2, 4), VTKV_GROUPED(80, 4, 4), VTKV_GROUPED(96, 2, 4), VTKV_GROUPED(112, 4, 4),
 #undef VTKV_GROUPED
       decode_attn_stream_kernel<true, true, false, 2, 128, true>, decode_attn_stream_kernel<true, true, true, 2, 128, true>,
+#define VTKV_SPLIT(DD, APP)                                                                                               \
+  decode_attn_stream_kernel<true, false, APP, 1, DD, false, true>, decode_attn_stream_kernel<true, true, APP, 1, DD, false, true>, \
+      decode_attn_stream_kernel<true, false, APP, 1, DD, true, true>, decode_attn_stream_kernel<true, true, APP, 1, DD, true, true>
+      VTKV_SPLIT(64, false), VTKV_SPLIT(80, false), VTKV_SPLIT(96, false), VTKV_SPLIT(112, false), VTKV_SPLIT(128, false),
+      VTKV_SPLIT(256, false), VTKV_SPLIT(128, true),
+#undef VTKV_SPLIT
   };
 #undef VTKV_ROW
 #undef VTKV_SIZE
@@ -1177,7 +1215,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
     if (g <= 0) return vtkv::fail(VTKV_EHIP, "cannot query the kernel's occupancy");
     grid = g;
   }
-  const int64_t n_float = scratch_floats(grid, num_seqs, num_heads, hd);
+  const int64_t n_float = scratch_floats(grid, num_seqs, num_kv_heads * group, hd);
   const int64_t count_bytes = counter_bytes(num_seqs, num_heads);
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
   const int64_t need = n_float * (int64_t)sizeof(float) + cum_bytes + count_bytes;
@@ -1197,7 +1235,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   p.slot_ids = slot_ids;
   p.seq_lens = seq_lens;
   p.alibi_slopes = alibi_slopes;
-  const int64_t n_stat = grid * 16 + (int64_t)num_seqs * num_heads;  // (slot, head) pairs
+  const int64_t n_stat = grid * 16 + (int64_t)num_seqs * num_kv_heads * group;  // (slot, head) pairs
   // the counters come first, at a place that does not depend on the sizes of a call
   p.seg_count = (uint32_t *)workspace;
   // Merging inside the streaming kernel saves the second launch, but the workgroup that arrives last
@@ -1234,6 +1272,8 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   p.num_heads = num_heads;
   p.num_kv_heads = num_kv_heads;
   p.group = group;
+  p.kv_split = kv_split;
+  p.group_real = group_real;
   p.span_tiles = partition_tokens > 0 ? partition_tokens / kTile : 0;
   p.grid = (int)grid;
   // Head-major tile order (see the kernel) where it lines the kv heads up with the XCDs: a contiguous eighth
@@ -1288,13 +1328,20 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   if (!p.fused_merge) {
     // segments of at least four pieces on average: four sets of threads share a segment's pieces
     const dim3 rgrid(num_kv_heads, num_seqs);
-#define VTKV_REDUCE_LAUNCH(G, S, HD)                                                                          \
+#define VTKV_REDUCE_LAUNCH_(G, S, HD, SP)                                                                     \
   do {                                                                                                        \
     if (timed)                                                                                                \
-      hipExtLaunchKernelGGL((decode_attn_reduce_kernel<G, S, HD>), rgrid, dim3(G * S * HD), 0, st, ev[2],     \
+      hipExtLaunchKernelGGL((decode_attn_reduce_kernel<G, S, HD, SP>), rgrid, dim3(G * S * HD), 0, st, ev[2], \
                             ev[3], 0, p);                                                                     \
     else                                                                                                      \
-      hipLaunchKernelGGL((decode_attn_reduce_kernel<G, S, HD>), rgrid, dim3(G * S * HD), 0, st, p);           \
+      hipLaunchKernelGGL((decode_attn_reduce_kernel<G, S, HD, SP>), rgrid, dim3(G * S * HD), 0, st, p);       \
+  } while (0)
+#define VTKV_REDUCE_LAUNCH(G, S, HD)                                                                          \
+  do {                                                                                                        \
+    if (kv_split > 1)                                                                                         \
+      VTKV_REDUCE_LAUNCH_(G, S, HD, true);                                                                    \
+    else                                                                                                      \
+      VTKV_REDUCE_LAUNCH_(G, S, HD, false);                                                                   \
   } while (0)
 #define VTKV_REDUCE(HD)                                                                                       \
   do {                                                                                                        \
@@ -1313,6 +1360,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
     }
 #undef VTKV_REDUCE
 #undef VTKV_REDUCE_LAUNCH
+#undef VTKV_REDUCE_LAUNCH_
   }
   if (timed) {
     g_timer.merged.resize(g_timer.calls + 1);
@@ -1375,8 +1423,10 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
                            : kDefaultMaxGrid;
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
   // (the kernels hold a head size padded to 32 elements, to 64 for fp8 rows: sized for the larger)
-  return scratch_floats(grid, num_seqs, num_heads, (head_size + 63) / 64 * 64) * (int64_t)sizeof(float) + cum_bytes +
-         counter_bytes(num_seqs, num_heads);
+  // (kv heads with more than 16 query heads are served in parts that may leave some of their 16 places empty:
+  // at most one sixteenth more places than heads)
+  return scratch_floats(grid, num_seqs, num_heads + num_heads / 16, (head_size + 63) / 64 * 64) * (int64_t)sizeof(float) +
+         cum_bytes + counter_bytes(num_seqs, num_heads);
 }
 
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
@@ -1396,8 +1446,8 @@ int64_t vtkv_decode_attention_v2_workspace_bytes(int num_seqs, int num_heads, in
   const int64_t grid = (int64_t)num_seqs * num_heads * max_num_partitions;  // at most one workgroup per head
   const int64_t cum_bytes = ((int64_t)(num_seqs + 1) * 4 + 15) / 16 * 16;
   // (the kernels hold a head size padded to 32 elements, to 64 for fp8 rows: sized for the larger)
-  return scratch_floats(grid, num_seqs, num_heads, (head_size + 63) / 64 * 64) * (int64_t)sizeof(float) + cum_bytes +
-         counter_bytes(num_seqs, num_heads);
+  return scratch_floats(grid, num_seqs, num_heads + num_heads / 16, (head_size + 63) / 64 * 64) * (int64_t)sizeof(float) +
+         cum_bytes + counter_bytes(num_seqs, num_heads);
 }
 
 int vtkv_decode_attention_v2(void *out, float *exp_sums, float *max_logits, void *tmp_out, const void *q,

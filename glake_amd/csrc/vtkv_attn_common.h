@@ -159,4 +159,27 @@ __device__ __forceinline__ float load_device_coherent(const float *p) {
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
+// More than 16 query heads per kv head (multi-query models).  The MFMA layouts hold a group's heads in 16
+// columns, so such a kv head is served as kv_split virtual kv heads that read the same K and V rows: the
+// kernels' num_kv_heads counts the virtual heads and `group` is the heads of each, virtual head v stands for
+// kv head v / kv_split and for the query heads [first_head_of(v), + heads_of(v)); the last virtual head of a
+// kv head has fewer heads than `group` when group_real is no multiple of it.  kv_split == 1: nothing changes.
+template <class Params>
+__device__ __forceinline__ int first_head_of(const Params &p, int kvh) {
+  if (p.kv_split == 1) return kvh * p.group;
+  return (kvh / p.kv_split) * p.group_real + (kvh % p.kv_split) * p.group;
+}
+template <class Params>
+__device__ __forceinline__ int real_kv_head(const Params &p, int kvh) {
+  return p.kv_split == 1 ? kvh : kvh / p.kv_split;
+}
+template <class Params>
+__device__ __forceinline__ int heads_of(const Params &p, int kvh) {
+  if (p.kv_split == 1) return p.group;
+  return min(p.group, p.group_real - (kvh % p.kv_split) * p.group);
+}
+
 }  // namespace vtkv_attn
+
+// Host side of the same rule: how many virtual kv heads a kv head with `group_real` query heads becomes.
+inline int vtkv_kv_split(int group_real) { return (group_real + 15) / 16; }

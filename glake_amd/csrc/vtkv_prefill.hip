@@ -57,7 +57,8 @@ struct PrefillParams {
   void *out;
   int out_f32;
   int64_t q_stride;
-  int num_heads, num_kv_heads, group;
+  int num_heads, num_kv_heads, group;  // (kv heads and heads of each as the kernel sees them: see first_head_of)
+  int kv_split, group_real;
   float scale_log2;  // scale * log2(e) [* k_scale for an fp8 cache]
   float v_scale;     // 1 for a bf16 cache
 };
@@ -140,9 +141,11 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   typedef const __attribute__((address_space(1))) u32x4 *gvec;
   const int64_t slot = p.slot_ids[u_seq];
   constexpr int kKvRowBytes = FP8 ? kD : 2 * kD;  // bytes of one head row in the cache
-  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kvh * kKvRowBytes;
-  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kvh * kKvRowBytes;
-  const uint32_t row_stride = (uint32_t)Hkv * kKvRowBytes;
+  const int kv_real = real_kv_head(p, kvh);  // whose rows this workgroup reads
+  gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kv_real * kKvRowBytes;
+  gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kv_real * kKvRowBytes;
+  const uint32_t row_stride = (uint32_t)(Hkv / p.kv_split) * kKvRowBytes;
+  const int head0 = first_head_of(p, kvh), n_heads = heads_of(p, kvh);
 
   // ---- this wave's columns: block nb, column n -> (token, head); unused columns get q = 0
   u32x4 qop[kNB][kKS];
@@ -153,12 +156,13 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   for (int nb = 0; nb < kNB; ++nb) {
     const int c = (wave * kNB + nb) * 16 + n;
     const int tok = c / G, head = c % G;
-    const bool valid = tok < u_ntok;
+    const bool valid = tok < u_ntok && head < n_heads;
     col_tok[nb] = valid ? tok : -1;
     col_head[nb] = head;
     limit[nb] = valid ? u_pos0 + tok + 1 : 0x7fffffff;
-    slope_log2[nb] = ALIBI && valid && p.alibi_slopes ? p.alibi_slopes[kvh * G + head] * kLog2e : 0.f;
-    const uint16_t *qrow = p.q + (int64_t)(u_row0 + (valid ? tok : 0)) * p.q_stride + (int64_t)(kvh * G + head) * kD;
+    slope_log2[nb] = ALIBI && valid && p.alibi_slopes ? p.alibi_slopes[head0 + head] * kLog2e : 0.f;
+    const uint16_t *qrow =
+        p.q + (int64_t)(u_row0 + (valid ? tok : 0)) * p.q_stride + (int64_t)(head0 + (valid ? head : 0)) * kD;
 #pragma unroll
     for (int ks = 0; ks < kKS; ++ks) {
       u32x4 raw = (u32x4){0, 0, 0, 0};
@@ -453,7 +457,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     const float l = sum_over_row_groups(l_run[nb]);
     if (col_tok[nb] < 0) continue;
     const float inv = p.v_scale / l;
-    const int64_t o0 = ((int64_t)(u_row0 + col_tok[nb]) * p.num_heads + kvh * G + col_head[nb]) * kD + 4 * g;
+    const int64_t o0 = ((int64_t)(u_row0 + col_tok[nb]) * p.num_heads + head0 + col_head[nb]) * kD + 4 * g;
 #pragma unroll
     for (int db = 0; db < kDB; ++db) {
       const f32x4 r = acc[nb][db] * inv;
@@ -486,10 +490,10 @@ extern "C" {
 
 int vtkv_prefill_unit_tokens_for(int num_heads, int num_kv_heads, int head_size, int kv_dtype) {
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return 0;
-  const int group = num_heads / num_kv_heads;
-  if (group > 16 || size_index(head_size) < 0) return 0;
+  const int group_real = num_heads / num_kv_heads, split = vtkv_kv_split(group_real);
+  if (size_index(head_size) < 0) return 0;
   (void)kv_dtype;  // the same kernels serve both cache types
-  return cols_per_group(head_size) / group;
+  return cols_per_group(head_size) / ((group_real + split - 1) / split);
 }
 
 int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype) {
@@ -512,15 +516,16 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   VTKV_REQUIRE(kv_dtype == q_dtype || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be q_dtype or FP8_E4M3");
   const bool fp8 = kv_dtype == VTKV_FP8_E4M3;
   if (fp8) VTKV_REQUIRE(k_scale > 0.f && v_scale > 0.f, "fp8 scales must be positive");
-  const int group = num_heads / num_kv_heads;
-  VTKV_REQUIRE(group <= 16, "num_heads/num_kv_heads = %d exceeds 16", group);
+  // more than 16 query heads per kv head: several virtual kv heads over the same rows (see first_head_of)
+  const int group_real = num_heads / num_kv_heads, split = vtkv_kv_split(group_real);
+  const int group = (group_real + split - 1) / split, kv_virtual = num_kv_heads * split;
   VTKV_REQUIRE(q_stride >= (int64_t)num_heads * head_size && q_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                    (uintptr_t)out % 16 == 0,
                "q rows must be 16-byte aligned and at least num_heads*head_size apart");
   // (the kernel addresses a sequence's rows with 32-bit byte offsets)
   VTKV_REQUIRE(max_seq_len > 0 && ((int64_t)max_seq_len + 64) * num_kv_heads * head_size * 2 < (1ll << 31),
                "max_seq_len %d: a sequence's K or V range must stay below 2 GiB", max_seq_len);
-  VTKV_REQUIRE((int64_t)num_units * num_kv_heads < (1ll << 31), "too many units");
+  VTKV_REQUIRE((int64_t)num_units * kv_virtual < (1ll << 31), "too many units");
   if (num_units == 0) return VTKV_OK;
   PrefillParams p;
   p.q = (const uint16_t *)q;
@@ -533,11 +538,13 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   p.out_f32 = out_dtype == VTKV_F32;
   p.q_stride = q_stride;
   p.num_heads = num_heads;
-  p.num_kv_heads = num_kv_heads;
+  p.num_kv_heads = kv_virtual;
   p.group = group;
+  p.kv_split = split;
+  p.group_real = group_real;
   p.scale_log2 = scale * kLog2e * (fp8 ? k_scale : 1.f);
   p.v_scale = fp8 ? v_scale : 1.f;
-  const dim3 grid((unsigned)((int64_t)num_units * num_kv_heads)), block(kThreads);
+  const dim3 grid((unsigned)((int64_t)num_units * kv_virtual)), block(kThreads);
   hipStream_t st = (hipStream_t)stream;
   // head size 128: one kernel per (type, cache type, ALiBi); the other sizes decide ALiBi at run time
   static void (*const kKernels[8])(PrefillParams) = {

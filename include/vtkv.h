@@ -289,8 +289,10 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  * A launch takes up to 1024 sequences; a larger batch runs as consecutive launches of 1024 on `stream` within
  * the one call.
  * Supported: q_dtype VTKV_BF16 or VTKV_F16, kv_dtype = q_dtype or VTKV_FP8_E4M3, head_size 64, 80, 96, 112, 128 or
- * 256 (the reference's list, vllm/attention/ops/paged_attn.py:33-34), num_heads/num_kv_heads in 1..16.  The kernel
- * is tuned for bf16 and head size 128; the other shapes run the same code with their own tile constants. */
+ * 256 (the reference's list, vllm/attention/ops/paged_attn.py:33-34), any whole num_heads/num_kv_heads.  The kernel
+ * is tuned for bf16 and head size 128; the other shapes run the same code with their own tile constants.  A kv head
+ * with more than 16 query heads (multi-query models) is served in ceil(n/16) parts of equal size (the last may be
+ * smaller) that each read the kv head's rows: the parts count as kv heads towards the limit of 64 per call. */
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                           const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
@@ -336,9 +338,10 @@ int vtkv_decode_attention_v2(void *out, float *exp_sums, float *max_logits, void
                              const float *alibi_slopes, int q_dtype, int out_dtype, int kv_dtype, float k_scale,
                              float v_scale, void *workspace, int64_t workspace_bytes, void *stream);
 
-/* Query tokens one unit may hold (one workgroup per unit and kv head): 128 / (num_heads/num_kv_heads) for head
- * sizes up to 128, 64 / (num_heads/num_kv_heads) for 256.  0 for unsupported shapes.  vtkv_prefill_unit_tokens is
- * the head size 128 form. */
+/* Query tokens one unit may hold (one workgroup per unit and kv head): 128 / g for head sizes up to 128, 64 / g for
+ * 256, where g = num_heads/num_kv_heads, or, beyond 16, the heads of one of the ceil(g/16) parts a kv head is then
+ * served in (71 heads: parts of 15).  0 for unsupported shapes.  vtkv_prefill_unit_tokens is the head size 128
+ * form. */
 int vtkv_prefill_unit_tokens_for(int num_heads, int num_kv_heads, int head_size, int kv_dtype);
 int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
 

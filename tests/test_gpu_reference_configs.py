@@ -240,7 +240,7 @@ def test_config4_full_size_through_the_step_plan(gpu_pool):
     eng.close()
 
 
-@pytest.mark.parametrize("hq,hkv,fp8", [(32, 8, False), (64, 8, True), (8, 8, False)])
+@pytest.mark.parametrize("hq,hkv,fp8", [(32, 8, False), (64, 8, True), (8, 8, False), (71, 1, False), (48, 2, True)])
 def test_split_k_interface_fills_the_callers_partition_buffers(gpu_pool, hq, hkv, fp8):
     """paged_attention_v2 with exp_sums / max_logits / tmp_out (csrc/attention/attention_kernels.cu:451-583):
     partition j of a sequence is rows [512 j, 512 j + 512).  Its entries are checked against values derived
