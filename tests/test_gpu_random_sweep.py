@@ -100,16 +100,30 @@ def test_random_sweep_over_head_sizes_and_types(gpu_pool, seed):
     """The same sweep over the other head sizes (64, 80, 96, 112, 256, and 128 in fp16), fp16 and bf16, plain and
     fp8 caches, the plain entry point with stream-K or fixed partitions and the split-K interface; for half of
     the cases also a batch of prompts (some behind cached rows) through the prompt kernel of that shape."""
+    sweep_head_sizes(gpu_pool, seed, HEADS, 40, always_f16_at_128=True)
+
+
+# more than 16 query heads per kv head: served in parts of 16, 15 + 11, 10, 9 + 8, 12, 13 + 12, 16 heads
+HEADS_MANY = [(64, 1), (48, 1), (71, 1), (40, 2), (17, 1), (96, 4), (100, 4), (128, 2)]
+
+
+@pytest.mark.parametrize("seed", [808])
+def test_random_sweep_with_many_query_heads_per_kv_head(gpu_pool, seed):
+    """The sweep over head sizes and types on multi-query shapes (head size 128 in bf16 included)."""
+    sweep_head_sizes(gpu_pool, seed, HEADS_MANY, 40, always_f16_at_128=False)
+
+
+def sweep_head_sizes(gpu_pool, seed, heads, cases, always_f16_at_128):
     import test_gpu_head_sizes as H
     from glake_amd import _C
 
     lib = _C.lib()
     rng = np.random.default_rng(seed)
     try:
-        for case in range(40):
-            hq, hkv = HEADS[rng.integers(len(HEADS))]
+        for case in range(cases):
+            hq, hkv = heads[rng.integers(len(heads))]
             d = int(rng.choice(H.HEAD_SIZES))
-            dtype = "f16" if (d == 128 or rng.integers(2)) else "bf16"
+            dtype = "f16" if ((d == 128 and always_f16_at_128) or rng.integers(2)) else "bf16"
             b = int(rng.integers(1, 16))
             kind = rng.integers(3)
             if kind == 0:
