@@ -68,10 +68,19 @@ class PrefixStore:
     def _split(self, slot: int, nbytes: int) -> int:
         """The holder of the first ``nbytes`` bytes of what ``slot`` holds (radix_cache.py:184)."""
         new = self._take_slot(nbytes)
-        segs = self.engine.vmm_kvcache_segment
-        segs[new].share_prefix(segs[slot], nbytes, self._stream())
+        self._share(new, slot, nbytes)
         self.rows[new] = nbytes // self.token_size
         return new
+
+    def _share(self, new: int, src: int, nbytes: int) -> None:
+        """Start the free holder ``new`` from the first ``nbytes`` bytes of slot ``src``; the holder goes back to
+        the free ones if that fails (the pool can still run dry under a map-ahead request)."""
+        segs = self.engine.vmm_kvcache_segment
+        try:
+            segs[new].share_prefix(segs[src], nbytes, self._stream())
+        except Exception:
+            self.free_slots.append(new)
+            raise
 
     # ------------------------------------------------------------------ the engine's calls
     def lookup(self, tokens: Sequence[int]) -> Tuple[Optional[int], int]:
@@ -105,8 +114,7 @@ class PrefixStore:
         if len(tokens) == 0:
             return 0
         new = self._take_slot(len(tokens) * self.token_size)
-        segs = self.engine.vmm_kvcache_segment
-        segs[new].share_prefix(segs[run_slot], len(tokens) * self.token_size, self._stream())
+        self._share(new, run_slot, len(tokens) * self.token_size)
         self.rows[new] = len(tokens)
         try:
             known = self.tree.insert(tokens, new)

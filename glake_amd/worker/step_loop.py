@@ -129,7 +129,10 @@ class StepLoop:
         store = self.prefix_store
         if store is not None:
             for req, holder, rows in out.prefix_hits:                     # the slot begins as the prefix
-                store.start_from(req.slot, holder, rows)
+                try:
+                    store.start_from(req.slot, holder, rows)
+                except RuntimeError:       # the pool ran dry under a map-ahead request: the prompt runs in full
+                    req.prefix_rows = 0    # (its chunks were claimed for all of its rows)
             store.end_step()
             if out.recompute or out.swapped_out:
                 store.make_room()      # a slot that shared a holder's chunks gave the pool less than its claim
