@@ -97,7 +97,9 @@ class DecodeStepPlan:
     travel in one asynchronous copy.  With ``fused=True`` (bf16 or fp8 cache) the append and the attention
     are one launch (``vtkv_decode_append_attention``) and, up to 512 sequences, the lengths travel with the
     kernel arguments, so a step is two kernels (attention and its merge) and no copy.  Build a new plan
-    when the set of running sequences changes.
+    when the set of running sequences changes.  ``run`` does host-side bookkeeping every step and hands the lengths
+    over by value: it is not something to record into a HIP graph (a captured step calls the separate
+    operators with device-side lengths).
     """
 
     def __init__(self, segments: Sequence, slot_ids: Sequence[int], key_cache, value_cache, num_heads: int,

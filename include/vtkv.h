@@ -374,7 +374,8 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
  * attention runs over all seq_lens[b] rows.  The cache contents and the result are those of
  * vtkv_reshape_and_cache followed by vtkv_decode_attention (the result up to fp32 summation order).
  * Lengths come either from the device (seq_lens) or from the host (host_seq_lens: copied into the kernel
- * arguments during the call, 512 per launch, so no upload is needed and the array may be reused at once);
+ * arguments during the call, 512 per launch, so no upload is needed and the array may be reused at once; a call
+ * recorded into a HIP graph keeps the lengths it was recorded with, so a captured step passes device lengths);
  * pass NULL for the other.  Head size 128 only; q_dtype VTKV_BF16 or VTKV_F16 (the paired-head variants for
  * very many short sequences exist for bf16 only).  kv_dtype is q_dtype, or VTKV_FP8_E4M3 with k_scale / v_scale: the new
  * rows are then stored as e4m3fn(x / scale), bit for bit as vtkv_reshape_and_cache stores them, and attended
