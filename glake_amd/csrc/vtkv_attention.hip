@@ -1255,7 +1255,10 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   const int knob_hm = g_head_major.load(std::memory_order_relaxed);
   const int segs_per_seq = num_kv_heads / seg_heads;
   const int64_t segs = (int64_t)num_seqs * segs_per_seq;
-  const bool hm_fits = partition_tokens == 0 && grid % 8 == 0 && (segs_per_seq % 8 == 0 || 8 % segs_per_seq == 0);
+  // (the parts of a split kv head read the same rows: head-major only if every XCD then holds whole kv heads, else
+  // each part would fetch the rows into another L2; one kv head of 64 query heads, 64 sequences: 58 us against 67)
+  const bool hm_fits = partition_tokens == 0 && grid % 8 == 0 && (segs_per_seq % 8 == 0 || 8 % segs_per_seq == 0) &&
+                       (kv_split == 1 || (segs_per_seq % 8 == 0 && (segs_per_seq / 8) % kv_split == 0));
   const bool hm_auto = knob_hm != 0 && hm_fits;  // the head-major order is open to this call
   p.fused_merge = !v2 && (knob_merge == 1 || (knob_merge < 0 && (hm_auto ? segs >= 2 * grid : 2 * segs >= 5 * grid)));
   p.heads_per_seg = seg_heads;
