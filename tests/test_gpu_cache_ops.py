@@ -46,6 +46,78 @@ def test_vtensor_scatter_decode_bit_exact(gpu_pool, hkv, d):
     gpu.close()
 
 
+@pytest.mark.parametrize("eb", [2, 4])
+@pytest.mark.parametrize("d", [64, 80, 96, 112, 128, 256])
+def test_vtensor_scatter_over_the_reference_matrix(gpu_pool, d, eb):
+    """tests/kernels/test_cache.py:10-18: 42 tokens, 8 heads, head sizes 64..256, half / bfloat16 (any 16-bit
+    pattern is moved as it is) and float; one new row per sequence, rows taken from a fused qkv tensor."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(d + eb)
+    b, hkv = 42, 8
+    row = hkv * d * eb
+    np_t, t_t = (np.uint16, torch.bfloat16) if eb == 2 else (np.uint32, torch.float32)
+    gpu = GpuSeqs(gpu_pool, b, hkv, d, eb, 1024)
+    gpu.map_zeroed(300 * row)
+    fused = rng.integers(0, 1 << (8 * eb), (b, 3, hkv, d), dtype=np.uint64).astype(np_t)
+    if eb == 4:                                           # keep the patterns finite floats: NaN payloads need not survive a .cuda()
+        fused &= np.uint32(0xBF7FFFFF)
+    slot_ids = rng.permutation(b).astype(np.int64)
+    slot_m = (rng.integers(0, 299, b) * row).astype(np.int64)
+    ks, vs, kp, vp = host_ranges(b, 300 * row)
+    O.reshape_and_cache_vtensor(fused[:, 1], fused[:, 2], kp, vp, slot_m, slot_ids, np.ones(b), np.zeros(b), 1, hkv, d)
+    f_t = torch.from_numpy(fused.view(np.int16 if eb == 2 else np.int32)).cuda().view(t_t)
+    kt, vt = gpu.table_tensors()
+    ops.reshape_and_cache(f_t[:, 1], f_t[:, 2], kt, vt, torch.from_numpy(slot_m).cuda(),
+                          torch.from_numpy(slot_ids).cuda(), None, None, 1, hkv, d)
+    torch.cuda.synchronize()
+    for s_ in range(b):
+        assert np.array_equal(gpu.download(s_, 300 * row, which="k"), ks[s_])
+        assert np.array_equal(gpu.download(s_, 300 * row, which="v"), vs[s_])
+    gpu.close()
+
+
+@pytest.mark.parametrize("d,src", [(64, "f16"), (80, "bf16"), (96, "f32"), (112, "f16"), (256, "bf16"), (128, "f16")])
+def test_vtensor_scatter_fp8_over_head_sizes_and_source_types(gpu_pool, d, src):
+    """kv_cache_dtype fp8 of the same matrix (test_cache.py:24): codes e4m3fn(x / scale) from half, bfloat16 and
+    float rows; an fp16 value is exact in fp32, so the oracle is given the fp32 values."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(3 * d)
+    b, hkv = 42, 8
+    row = hkv * d
+    x_k = (rng.standard_normal((b, hkv, d)) * 2.0).astype(np.float32)
+    x_v = (rng.standard_normal((b, hkv, d)) * 2.0).astype(np.float32)
+    k_scale, v_scale = float(np.abs(x_k).max() / 448), 0.0171
+    if src == "bf16":
+        hk, hv = O.f32_to_bf16(x_k), O.f32_to_bf16(x_v)
+        tk, tv = torch_bf16_from_bits(hk), torch_bf16_from_bits(hv)
+    elif src == "f16":
+        hk, hv = x_k.astype(np.float16).astype(np.float32), x_v.astype(np.float16).astype(np.float32)
+        tk, tv = torch.from_numpy(hk).cuda().to(torch.float16), torch.from_numpy(hv).cuda().to(torch.float16)
+    else:
+        hk, hv = x_k, x_v
+        tk, tv = torch.from_numpy(x_k).cuda(), torch.from_numpy(x_v).cuda()
+    gpu = GpuSeqs(gpu_pool, b, hkv, d, 1, 2048)
+    gpu.map_zeroed(500 * row)
+    slot_ids = rng.permutation(b).astype(np.int64)
+    slot_m = (rng.integers(0, 499, b) * row).astype(np.int64)
+    ks, vs, kp, vp = host_ranges(b, 500 * row)
+    O.reshape_and_cache_vtensor_fp8(hk, hv, kp, vp, slot_m, slot_ids, hkv, d, k_scale, v_scale)
+    kt, vt = gpu.table_tensors()
+    ops.reshape_and_cache(tk, tv, kt, vt, torch.from_numpy(slot_m).cuda(), torch.from_numpy(slot_ids).cuda(), None,
+                          None, 1, hkv, d, "fp8", k_scale, v_scale)
+    torch.cuda.synchronize()
+    for s_ in range(b):
+        assert np.array_equal(gpu.download(s_, 500 * row, which="k"), ks[s_])
+        assert np.array_equal(gpu.download(s_, 500 * row, which="v"), vs[s_])
+    gpu.close()
+
+
 def test_vtensor_scatter_prefill_form_bit_exact(gpu_pool):
     """grid (batch, max_query_len): rows cache_seq_lens[b]+t of the packed prompt go to consecutive rows."""
     import torch
