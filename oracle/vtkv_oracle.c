@@ -25,9 +25,15 @@
  *   oracle_copy_blocks              : compiled reference CPU twin, identity.
  *   oracle_reshape_and_cache_vtensor: brute-force address formula; equals the paged
  *       variant at block_size 1 up to the [T,Hkv,D] collapse.
- *   oracle_fp8_e4m3fn_*             : torch.float8_e4m3fn casts (library routine),
- *       exhaustive over the 256 codes and all 65536 bf16 inputs.
- *   oracle_swap_blocks              : identity / exact equality.
+ *   oracle_fp8_e4m3fn_*, oracle_convert_to_fp8 : torch.float8_e4m3fn casts (library routine),
+ *       exhaustive over the 256 codes and all 65536 bf16 inputs at scale 1, and with a
+ *       scale (torch's cast of the IEEE quotient x / scale) over all bf16 inputs for each of
+ *       the 112 scales of the reference's tests/fp8_kv/.../kv_cache_scales.json and eight
+ *       others, random fp32 inputs and inputs whose quotient is an exact tie.
+ *   oracle_reshape_and_cache_vtensor_fp8 : the same cast plus the address formula of
+ *       csrc/cache_kernels.cu:176-199 in numpy, skipped rows and strided sources included.
+ *   oracle_swap_blocks              : want[dst] = src[src] by numpy indexing on the block
+ *       pairs of the reference's tests/worker/test_swap.py:57-89 and on random pairs.
  */
 #include <math.h>
 #include <stdint.h>

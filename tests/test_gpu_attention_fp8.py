@@ -16,7 +16,7 @@ from kvharness import GpuSeqs, bf16_randn, bits_from_torch_bf16, torch_bf16_from
 pytestmark = pytest.mark.gpu
 
 
-def run_case(vmm, seed, seq_lens, hq, hkv, d=128, alibi=False, spread=1.0, partition_tokens=0):
+def run_case(vmm, seed, seq_lens, hq, hkv, d=128, alibi=False, spread=1.0, partition_tokens=0, scales=None):
     import torch
 
     from glake_amd import _custom_ops as ops
@@ -28,6 +28,8 @@ def run_case(vmm, seed, seq_lens, hq, hkv, d=128, alibi=False, spread=1.0, parti
     v_f = [rng.standard_normal((t, hkv, d)).astype(np.float32) * spread for t in seq_lens]
     k_scale = float(max(np.abs(k).max() for k in k_f) / 448.0)
     v_scale = float(max(np.abs(v).max() for v in v_f) / 448.0)
+    if scales is not None:  # given scales instead of amax / 448: values beyond 448 * scale saturate
+        k_scale, v_scale = scales
     gpu = GpuSeqs(vmm, b + 2, hkv, d, 1, max(seq_lens))
     empty8 = np.zeros((1, hkv, d), np.uint8)
     k_codes, v_codes = [empty8] * (b + 2), [empty8] * (b + 2)
@@ -76,6 +78,21 @@ def test_fp8_config4_shape_llama70b_layer(gpu_pool):
     # BASELINE config 4 at reduced batch: Hq 64, Hkv 8 (GQA 8), ctx uniform in [1024, 8192]
     rng = np.random.default_rng(1003)
     run_case(gpu_pool, 1003, rng.integers(1024, 8193, 6).tolist(), 64, 8)
+
+
+def test_fp8_with_the_reference_models_layer_scales(gpu_pool):
+    """The per-layer scales of the reference's llama2-7b and llama2-70b fp8 checkpoints
+    (tests/fp8_kv/*/kv_cache_scales.json) through the loader, one scale for K and V of a layer as the model passes
+    it (llama.py:484-505; no doubling: this cache is OCP e4m3fn like the file, not FNUZ)."""
+    import os
+
+    from glake_amd.worker.kv_scales import layer_scales
+
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fp8_kv")
+    s7 = layer_scales(os.path.join(golden, "llama2-7b_kv_cache_scales.json"), 32, model_type="llama")
+    s70 = layer_scales(os.path.join(golden, "llama2-70b_kv_cache_scales.json"), 80, model_type="llama")
+    for seed, (s, hq, hkv) in enumerate([(s7[0], 32, 32), (s7[31], 32, 8), (s70[0], 64, 8), (max(s70), 64, 8)]):
+        run_case(gpu_pool, 40 + seed, [17, 300, 1111], hq, hkv, scales=(s, s))
 
 
 def test_fp8_alibi_and_wide_values(gpu_pool):
