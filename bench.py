@@ -29,23 +29,24 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes moved per launch of the dominant kernel relative to its algorithmic bytes, measured with
 # rocprofv3 (FETCH_SIZE and WRITE_SIZE in separate runs, each scaled by what the counter reads for the
 # calibration copy of known size that this script runs before timing).  Counters cannot be read from
-# inside this process, so the measured ratios are kept in a small table beside the profile summaries.
-TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_decode_attn_stream_kernel.txt")
+# inside this process: the ratios below were measured once per workload with the commands given in the
+# named summaries, and `roofline.traffic` is the launch's algorithmic bytes times that stored ratio (the
+# JSON says so: "traffic_replayed_from_profile").
+# workload: (fetch bytes, write bytes, algorithmic bytes of the profiled launches, MFMA-busy share, summary)
+MEASURED_TRAFFIC = {
+    "c2": (634797463, 2403448, 635113472, 0.0663, "profiles/decode_attn_stream_kernel_c2_llama3_8b_decode.md"),
+    "c3": (926249383, 1144900, 926629888, 0.0681, "profiles/decode_attn_stream_kernel_c3_c4_c5.md"),
+    "c4": (1212193147, 10957685, 1213501440, 0.1253, "profiles/decode_attn_stream_kernel_c3_c4_c5.md"),
+    "c5": (1236069922, 5777604, 1235329024, 0.0651, "profiles/decode_attn_stream_kernel_c3_c4_c5.md"),
+}
 
 
 def measured_traffic(config: str):
-    """(traffic / algorithmic bytes, MFMA-busy fraction or None, source) for `config`, or (None, None, None)."""
-    try:
-        with open(TRAFFIC_TABLE) as f:
-            for line in f:
-                cols = line.split()
-                if len(cols) >= 6 and cols[0] == config:
-                    fetch, write, algo = float(cols[1]), float(cols[2]), float(cols[3])
-                    mfma = None if cols[4] == "-" else float(cols[4])
-                    return (fetch + write) / algo, mfma, cols[5]
-    except OSError:
-        pass
-    return None, None, None
+    """(traffic / algorithmic bytes, MFMA-busy fraction, source) for `config`, or (None, None, None)."""
+    if config not in MEASURED_TRAFFIC:
+        return None, None, None
+    fetch, write, algo, mfma, source = MEASURED_TRAFFIC[config]
+    return (fetch + write) / algo, mfma, source
 
 
 CONFIGS = {
@@ -58,7 +59,8 @@ CONFIGS = {
     # configs[3]: fp8-e4m3 KV at the Llama-3-70B per-layer shape
     "c4": dict(name="llama3-70b-layer-decode-fp8kv B=128 Hq=64 Hkv=8 D=128 ctx~U[1024,8192]", batch=128, hq=64,
                hkv=8, d=128, lo=1024, hi=8192, seed=1003, kv="fp8"),
-    # configs[4] without its swap events: 256 sequences
+    # configs[4]: 256 sequences that grow; as a plain workload (--config c5) without its swap events, with them
+    # in growth_and_swap_protocol()
     "c5": dict(name="growth-bf16 B=256 Hq=32 Hkv=8 D=128 ctx~U[256,2048]", batch=256, hq=32, hkv=8, d=128, lo=256,
                hi=2048, seed=1004, kv="bf16"),
     # outside BASELINE.json: very many short sequences (every workgroup meets many segment starts and ends)
@@ -174,6 +176,10 @@ def main() -> int:
     ap.add_argument("--head-major", default="auto", choices=["auto", "on", "off"],
                     help="tile order of the decode kernel: (kv head, sequence, rows) or (sequence, kv head, rows)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", action="store_true",
+                    help="with --config c2: leave out the other BASELINE configurations (c3, c4 and the growth-and-swap "
+                         "protocol) that the default run appends under \"configs\"")
+    ap.add_argument("--other-repeats", type=int, default=7, help="timed regions of each of those other configurations")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -181,21 +187,43 @@ def main() -> int:
               "use --gpus 1", file=sys.stderr)
         return 2
 
-    import torch
-
-    from glake_amd import _C, _custom_ops as ops, vmm_allocator as vmm
-    from glake_amd.worker.cache_engine import CacheEngine
-
     cfg = CONFIGS[args.config]
     if cfg.get("prefill"):
         if args.steps == 200 and args.warmup == 20:
             args.steps, args.warmup = 20, 3
         return prompt_run(args, cfg)
+    from glake_amd import _C
+
     _C.check(_C.lib().vtkv_set_fused_merge({"auto": -1, "fused": 1, "separate": 0}[args.merge]))
     _C.check(_C.lib().vtkv_set_head_major({"auto": -1, "on": 1, "off": 0}[args.head_major]))
+    R = args.repeats if args.repeats > 0 else (21 if args.steps <= 50 else 3)
+    result = decode_run(args, args.config, R, with_swap=args.host_path != "backend", with_cpu=not args.no_cpu_baseline)
+    # The other BASELINE configurations in the same line (the headline stays configs[1]): configs[2] and [3] as
+    # plain decode workloads with fewer regions, configs[4] as BASELINE.json writes it, swap events included.
+    if args.config == "c2" and args.host_path == "plan" and args.partition_tokens == 0 and not args.only:
+        keep = ("value", "unit", "ms_per_step", "pct_of_hbm_peak", "tokens_per_s", "repeats", "regions_gbps",
+                "algorithmic_bytes_per_step", "host_issue_ms_per_step", "dtype", "roofline", "mfma_util")
+        others = {}
+        for name in ("c3", "c4"):
+            r = decode_run(args, name, args.other_repeats, with_swap=False, with_cpu=False)
+            others[name] = {"workload": r["config"]["workload"], **{k: r[k] for k in keep}}
+        others["c5"] = growth_and_swap_protocol(args)
+        result["configs"] = others
+    print(json.dumps(result))
+    return 0
+
+
+def decode_run(args, config: str, R: int, with_swap: bool, with_cpu: bool) -> dict:
+    """W warm-up steps, R timed regions of exactly K decode steps, the per-kernel event pass, optionally the swap
+    figures and the CPU baseline, for one workload of CONFIGS; returns the JSON object of that workload."""
+    import torch
+
+    from glake_amd import _C, _custom_ops as ops, vmm_allocator as vmm
+    from glake_amd.worker.cache_engine import CacheEngine
+
+    cfg = CONFIGS[config]
     B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
     K, W = args.steps, args.warmup
-    R = args.repeats if args.repeats > 0 else (21 if K <= 50 else 3)
     backend_path = args.host_path == "backend"
     L = args.layers if backend_path else 1
     torch.cuda.set_device(0)
@@ -210,7 +238,7 @@ def main() -> int:
     row = Hkv * D * eb
     max_tokens = max(ctx0) + total_steps + 1
     chunks_per_range = (max_tokens * row + args.value_skew + (2 << 20) - 1) // (2 << 20)
-    vmm.init_physical_handle(2 * L * B * chunks_per_range + 16, 0)
+    ensure_pool(2 * L * B * chunks_per_range + 16)
     engine = CacheEngine(num_layers=L, num_kv_heads=Hkv, head_size=D, dtype=torch.uint8 if fp8 else torch.bfloat16,
                          max_num_seqs=B, max_num_batched_tokens=max_tokens,
                          swap_space_bytes=0 if backend_path else 1 << 30, value_skew=args.value_skew)
@@ -350,7 +378,7 @@ def main() -> int:
     # hipMemMap and hipMemUnmap wait for all work queued on the null stream, so a chunk mapped while
     # decode steps are queued there would drain the pipeline every time a sequence crosses 2 MiB.
     torch.cuda.synchronize()
-    torch.cuda.set_stream(torch.cuda.Stream(device=dev))
+    torch.cuda.set_stream(bench_stream(dev))
 
     # ---- timed regions: each exactly K steps, synchronised on both sides.  A region of few steps carries the
     # fixed cost of its two ends (the host work before the first launch reaches the GPU, the wake-up after
@@ -368,8 +396,8 @@ def main() -> int:
         host_dt = time.perf_counter() - t0  # all K steps issued; the GPU may still be running
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        regions.append((nbytes / dt / 1e9, dt, host_dt))
-    gbps, dt, host_dt = sorted(regions)[len(regions) // 2]
+        regions.append((nbytes / dt / 1e9, dt, host_dt, nbytes))
+    gbps, dt, host_dt, region_bytes = sorted(regions)[len(regions) // 2]
     ms_per_step = dt / K * 1e3
     tokens_per_s = B * K / dt
 
@@ -390,11 +418,13 @@ def main() -> int:
     part_ms, red_ms = list(t_stream), list(t_reduce)
     avg_part_ms = float(np.mean(part_ms))
     achieved = float(np.mean(kbytes)) / (avg_part_ms * 1e-3) / 1e9
-    ratio, mfma_busy, source = measured_traffic(args.config)
+    ratio, mfma_busy, source = measured_traffic(config)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "traffic": None if ratio is None else int(ratio * float(np.mean(kbytes))),
                 "traffic_unit": "bytes per launch", "traffic_over_algorithmic": ratio, "traffic_source": source,
+                # (the ratio was measured in a separate rocprofv3 --pmc run of this workload, not in this run)
+                "traffic_replayed_from_profile": ratio is not None,
                 "kernel": "decode_attn_stream_kernel", "avg_kernel_us": round(avg_part_ms * 1e3, 2),
                 "avg_reduce_kernel_us": round(float(np.mean(red_ms)) * 1e3, 2),
                 "algorithmic_bytes_per_launch": int(np.mean(kbytes))}
@@ -405,7 +435,7 @@ def main() -> int:
     # sequence swapped back in before its chunks were needed elsewhere finds them still mapped ("warm");
     # the second round trip forces the unmapping in between ("cold": swap-in has to map every chunk).
     swap = None
-    if not backend_path:
+    if with_swap:
         nswap = max(1, B // 4)
         swap_slots = list(range(nswap))
         engine.swap_out(swap_slots)  # untimed: first use of the pinned arena and of the copy streams
@@ -443,6 +473,8 @@ def main() -> int:
                    "value_skew_bytes": engine.value_skew},
         "repeats": R,
         "regions_gbps": [round(r[0], 1) for r in regions],
+        # attention + cache-write bytes of one step of the median region (value = this / ms_per_step)
+        "algorithmic_bytes_per_step": int(region_bytes // K),
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "tokens_per_s": round(tokens_per_s, 1),
         "ms_per_layer": round(ms_per_step / L, 4),
@@ -455,14 +487,176 @@ def main() -> int:
                                                       "source": source},
     }
 
-    if not args.no_cpu_baseline:
+    if with_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg, engine, final_lens, q, scale, args.cpu_seconds, k_scale, v_scale)
         result["cpu_baseline_c1"] = cpu_baseline_c1(max(2.0, args.cpu_seconds / 3))
 
-    print(json.dumps(result))
     engine.close()
-    return 0
+    torch.cuda.synchronize()
+    return result
 
+
+_STREAM = {}
+
+
+def bench_stream(dev):
+    """The one non-blocking stream of default priority that every workload of this process runs on."""
+    import torch
+
+    if dev not in _STREAM:
+        _STREAM[dev] = torch.cuda.Stream(device=dev)
+    return _STREAM[dev]
+
+
+def ensure_pool(chunks: int) -> None:
+    """Have at least `chunks` free physical chunks in the pool (chunks of a workload that has ended are free again)."""
+    from glake_amd import vmm_allocator as vmm
+
+    have = vmm.showFreeBlocks() if vmm.totalBlocks() > 0 else 0
+    if have < chunks:
+        vmm.init_physical_handle(chunks - have, 0)
+
+
+
+
+def growth_and_swap_protocol(args) -> dict:
+    """BASELINE.json configs[4] as written: 256 sequences (bf16, Hq=32, Hkv=8, D=128, initial context
+    U[256,2048], seed 1004), 64 decode steps that append one token each and map a 2 MiB chunk where a range
+    crosses a boundary; after steps 16, 32, 48 and 64 a seeded random 25 % of the sequences is swapped out to
+    pinned host memory and back in.  Reported: attention GB/s over the decode steps (each block of 16 steps timed
+    between two synchronisations; algorithmic bytes as everywhere), host-link GB/s of every swap-out and swap-in
+    (bytes of the swapped ranges over the wall time of the call, which ends with the copies done and the chunks
+    given back or mapped), the chunks mapped while the sequences grew, and a bit-exact check: every byte of
+    every swapped range is copied aside on the device before the swap-out and again after the swap-in (outside the
+    timed calls) and the two copies are compared, and the rows appended by the 64 steps are compared with the
+    step's inputs."""
+    import torch
+
+    from glake_amd import _C, vmm_allocator as vmm
+    from glake_amd.worker.cache_engine import CacheEngine
+    from glake_amd.worker.step import DecodeStepPlan
+
+    cfg = CONFIGS["c5"]
+    B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
+    steps, every, W = 64, 16, max(args.warmup, 5)
+    dev = torch.device("cuda", 0)
+    gen = torch.Generator().manual_seed(cfg["seed"])
+    ctx0 = torch.randint(cfg["lo"], cfg["hi"] + 1, (B,), generator=gen).tolist()
+    row = Hkv * D * 2
+    chunk = vmm.chunkBytes()
+    max_tokens = max(ctx0) + steps + W + 1
+    chunks_per_range = (max_tokens * row + args.value_skew + chunk - 1) // chunk
+    ensure_pool(2 * B * chunks_per_range + 16)
+    engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.bfloat16, max_num_seqs=B,
+                         max_num_batched_tokens=max_tokens, swap_space_bytes=1 << 30, value_skew=args.value_skew)
+    segs = engine.vmm_kvcache_segment
+    from glake_amd import _custom_ops as ops
+
+    ggen = torch.Generator(device=dev).manual_seed(cfg["seed"])
+    for b in range(B):
+        nbytes = ctx0[b] * row
+        segs[b].ensure_mapped(nbytes)
+        for base in (segs[b].getKeyDevicePtr(0), segs[b].getValueDevicePtr(0)):
+            t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+            ops.swap_ranges([t.data_ptr()], [base], [nbytes], "d2d")
+            torch.cuda.synchronize()
+        segs[b].set_used_size(nbytes)
+    q = torch.randn(B, Hq, D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    new_k = torch.randn(B, Hkv * D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    new_v = torch.randn(B, Hkv * D, generator=ggen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
+    plan = DecodeStepPlan(segs, list(range(B)), engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hq, Hkv, D,
+                          float(D) ** -0.5, device=dev)
+    torch.cuda.synchronize()
+    torch.cuda.set_stream(bench_stream(dev))
+
+    def snapshot(slots):
+        """The used bytes of the K and V ranges of `slots`, gathered into one device buffer with device-to-device
+        copies (the comparison stays on the GPU: reading 0.6 GB back to the host around every event would leave the
+        GPU idle for a tenth of a second, which the next steps' clocks would show)."""
+        sizes = [segs[s_].used_size for s_ in slots]
+        buf = torch.empty(2 * sum(sizes), dtype=torch.uint8, device=dev)
+        src, dst, nb, at = [], [], [], buf.data_ptr()
+        for s_, n in zip(slots, sizes):
+            for base in (segs[s_].getKeyDevicePtr(0), segs[s_].getValueDevicePtr(0)):
+                src.append(base)
+                dst.append(at)
+                nb.append(n)
+                at += n
+        ops.swap_ranges(src, dst, nb, "d2d")
+        return buf
+
+    # warm-up steps (they append rows too), one untimed swap round trip (first use of the pinned arena and the copy
+    # streams), then the sequences are set back to their initial lengths: the 64 steps start from BASELINE's contexts
+    for _ in range(W):
+        plan.run(q, new_k, new_v, out)
+    torch.cuda.synchronize()
+    engine.swap_out([0, 1])
+    engine.swap_in([0, 1])
+    torch.cuda.synchronize()
+    for b in range(B):
+        segs[b].set_used_size(ctx0[b] * row)
+    mapped0 = sum(s.actual_size for s in segs) // chunk
+
+    blocks, events = [], []
+    bit_exact, checked = True, 0
+    step_bytes = step_time = 0.0
+    for blk in range(steps // every):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        nbytes = 0
+        for _ in range(every):
+            plan.run(q, new_k, new_v, out)
+            nbytes += int(plan.seq_lens.sum()) * 2 * row + 2 * B * Hq * D * 2 + B * 2 * row * 2
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        blocks.append(round(nbytes / dt / 1e9, 1))
+        step_bytes += nbytes
+        step_time += dt
+        # the swap event: a seeded random quarter of the sequences out and back in
+        chosen = sorted(torch.randperm(B, generator=gen)[:B // 4].tolist())
+        before = snapshot(chosen)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        moved = engine.swap_out(chosen)
+        t1 = time.perf_counter()
+        engine.swap_in(chosen)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        after = snapshot(chosen)
+        bit_exact = bit_exact and after.shape == before.shape and bool(torch.equal(after, before))
+        checked += after.numel()
+        del before, after
+        events.append({"after_step": (blk + 1) * every, "sequences": len(chosen), "bytes_per_direction": moved,
+                       "out_gbps": round(moved / (t1 - t0) / 1e9, 2), "in_gbps": round(moved / (t2 - t1) / 1e9, 2)})
+    mapped1 = sum(s.actual_size for s in segs) // chunk
+    # the rows the 64 steps appended: every sequence's last 64 K and V rows equal the step's input rows
+    nk = new_k.view(torch.int16).cpu().numpy().view(np.uint16)
+    nv = new_v.view(torch.int16).cpu().numpy().view(np.uint16)
+    appended_exact = True
+    for b in range(B):
+        appended_exact = appended_exact and segs[b].used_size == (ctx0[b] + steps) * row
+        tail = np.empty((2, steps, Hkv * D), np.uint16)
+        off = ctx0[b] * row
+        _C.check(_C.lib().vtkv_memcpy_d2h(tail[0].ctypes.data_as(C.c_void_p), segs[b].getKeyDevicePtr(0) + off, steps * row))
+        _C.check(_C.lib().vtkv_memcpy_d2h(tail[1].ctypes.data_as(C.c_void_p), segs[b].getValueDevicePtr(0) + off, steps * row))
+        appended_exact = appended_exact and bool(np.all(tail[0] == nk[b]) and np.all(tail[1] == nv[b]))
+    engine.close()
+    torch.cuda.synchronize()
+    med = lambda xs: sorted(xs)[len(xs) // 2]
+    gbps = step_bytes / step_time / 1e9
+    return {
+        "workload": "growth+swap bf16: 256 seqs Hq=32 Hkv=8 D=128 ctx0~U[256,2048], 64 steps, 25 % swapped out and in "
+                    "after steps 16/32/48/64 (BASELINE.json configs[4])",
+        "value": round(gbps, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "ms_per_step": round(step_time / steps * 1e3, 4), "tokens_per_s": round(B * steps / step_time, 1),
+        "algorithmic_bytes_per_step": int(step_bytes // steps), "steps": steps, "blocks_gbps": blocks,
+        "chunks_mapped_while_growing": int(mapped1 - mapped0),
+        "swap_events": events,
+        "swap_out_gbps": med([e["out_gbps"] for e in events]), "swap_in_gbps": med([e["in_gbps"] for e in events]),
+        "bit_exact": bool(bit_exact and appended_exact), "swapped_bytes_checked": int(checked),
+        "appended_rows_checked": B * steps * 2,
+    }
 
 def cpu_model() -> str:
     try:

@@ -82,6 +82,7 @@ SIGNATURES = {
     "vtkv_host_alloc": (_p, [_i64]),
     "vtkv_host_free": (_i, [_p]),
     "vtkv_copy_blocks": (_i, [_p, _p, _i, _p, _i, _i64, _p]),
+    "vtkv_reshape_and_cache_flash": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _i, _p]),
     "vtkv_convert_fp8": (_i, [_p, _p, _i64, _f, _i, _i, _p]),
     "vtkv_decode_attention_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
     "vtkv_decode_attention": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i64, _f, _i, _p, _i, _i, _i, _f, _f, _p,

@@ -382,6 +382,30 @@ def reshape_and_cache_paged(
         head_size, block_size, key.stride(0), value.stride(0), key.element_size(), _stream()))
 
 
+def reshape_and_cache_flash(
+    key: torch.Tensor,
+    value: torch.Tensor,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    slot_mapping: torch.Tensor,
+    kv_cache_dtype: str,
+) -> None:
+    """vllm/_custom_ops.py:255-264: K and V caches [num_blocks, block_size, H, D]; "auto" caches only
+    (csrc/cache_kernels.cu:307-310)."""
+    if kv_cache_dtype != "auto":
+        raise _C.VtkvError(_C.EINVAL, f"Unsupported data type of kv cache: {kv_cache_dtype}")
+    _require_cuda(key, value, key_cache, value_cache, slot_mapping)
+    num_tokens, num_heads, head_size = key.shape
+    if key_cache.stride(0) != value_cache.stride(0):
+        raise _C.VtkvError(_C.EINVAL, "key_cache and value_cache differ in their block stride")
+    if key.stride(1) != head_size or key.stride(2) != 1 or value.stride(1) != head_size or value.stride(2) != 1:
+        raise _C.VtkvError(_C.EINVAL, "key/value rows must be contiguous in (head, dim)")
+    _C.check(_C.lib().vtkv_reshape_and_cache_flash(
+        _ptr(key), _ptr(value), _ptr(key_cache), _ptr(value_cache), _ptr(slot_mapping), num_tokens, num_heads,
+        head_size, key_cache.shape[1], key_cache.stride(0), key.stride(0), value.stride(0), key.element_size(),
+        _stream()))
+
+
 def copy_blocks(key_caches: Sequence[torch.Tensor], value_caches: Sequence[torch.Tensor],
                 block_mapping: torch.Tensor) -> None:
     """vllm/_custom_ops.py:266-268; block_mapping is an int64 [num_pairs, 2] GPU tensor."""

@@ -76,7 +76,9 @@ class VTensorMetadata(AttentionMetadata, PagedAttentionMetadata):
     # prefix, a later chunk of a long prompt); None: every prompt is attended in full (query = all rows)
     query_lens: Optional[List[int]] = None
     query_lens_tensor: Optional[torch.Tensor] = None  # the same on the GPU (int32), made by prepare_step
-    _host_decode_lens: Optional[object] = None  # the decode sequences' lengths as a C array, made on first use
+    # the decode sequences' lengths of THIS step as a C array: made by prepare_step from seq_lens every step (never
+    # by forward, so a metadata object that is reused or changed between steps cannot carry stale lengths)
+    _host_decode_lens: Optional[object] = None
     _cached_prefill_metadata: Optional["VTensorMetadata"] = None
     _cached_decode_metadata: Optional["VTensorMetadata"] = None
 
@@ -158,6 +160,10 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
         ``slot_m``, ``seq_lens_tensor``) is ordered the same way."""
         from ... import _custom_ops as ops
 
+        if query.dtype not in (torch.bfloat16, torch.float16):
+            # the attention kernels take 16-bit queries; on the reference's vTensor path both decode branches run
+            # an external kernel that exists for fp16 and bf16 only (xformers.py:362-385,407-430)
+            raise ValueError(f"the vtensor backend runs bfloat16 and float16 models, not {query.dtype}")
         query = query.view(-1, self.num_heads, self.head_size)
         key = key.view(-1, self.num_kv_heads, self.head_size)
         value = value.view(-1, self.num_kv_heads, self.head_size)
@@ -219,11 +225,13 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
                 # reference's flow (llama.py:340: the bytes used before this step).  Where the metadata also
                 # holds the lengths on the host (model_runner.py:607 passes both), up to 512 of them travel
                 # with the kernel arguments, which spares the kernel a dependent load at its start.
-                if meta.seq_lens is not None and num_decode_tokens <= 512 and len(meta.seq_lens) == n_pre + num_decode_tokens:
-                    if meta._host_decode_lens is None:  # once per step, shared by the layers
-                        import ctypes
-                        meta._host_decode_lens = (ctypes.c_int32 * num_decode_tokens)(*meta.seq_lens[n_pre:])
-                    d_lens = meta._host_decode_lens
+                # prepare_step makes that array once per step for all layers; a step that is recorded into a graph
+                # (use_cuda_graph, or a stream that is capturing) reads the device lengths, since values passed as
+                # kernel arguments would be frozen into the recording.
+                host_lens = meta._host_decode_lens
+                if (host_lens is not None and len(host_lens) == num_decode_tokens and not meta.use_cuda_graph
+                        and not torch.cuda.is_current_stream_capturing()):
+                    d_lens = host_lens
                 ops.decode_append_attention(
                     d_out, d_query, d_key, d_value, k_table, v_table, self.num_kv_heads, self.scale, d_lens, max_len,
                     self.alibi_slopes, d_slots, kv_cache_dtype=self.kv_cache_dtype, kv_scale=kv_scale, v_scale=vs)

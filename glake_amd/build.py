@@ -23,6 +23,8 @@ HIP_FLAGS = [
     # keep MFMA accumulators in ordinary VGPRs: the softmax rescale multiplies them on the VALU and
     # the AGPR form would copy all of them back and forth every tile
     "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # only the C ABI of include/vtkv.h (declared with default visibility there) leaves the shared object
+    "-fvisibility=hidden", "-fvisibility-inlines-hidden",
     "-Wall", "-Wno-unused-function",
 ]
 
@@ -55,7 +57,8 @@ def build_library(verbose: bool = False, out_path: str = LIB_PATH, extra_flags=(
     with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     tmp = out_path + ".tmp"
-    res = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs, "-lpthread"],
+    res = subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs, "-lpthread",
+                          "-Wl,--version-script=" + os.path.join(CSRC, "vtkv.map")],
                          capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("linking libvtkv.so failed:\n" + res.stderr)

@@ -135,15 +135,48 @@ __global__ void __launch_bounds__(256) scatter_paged_kernel(const char *__restri
 }
 
 // ---------------------------------------------------------------------------------------------
+// Scatter into the flash-attention cache layout (replaces vllm::reshape_and_cache_flash_kernel,
+// csrc/cache_kernels.cu:202-236): K and V caches are both [num_blocks, block_size, H, D], so a token's row is
+// H*D contiguous elements on both sides.  grid (num_tokens); half of the lanes take K, half V, 16 bytes each.
+template <bool ALIGNED16>
+__global__ void __launch_bounds__(256) scatter_flash_kernel(const char *__restrict__ key, const char *__restrict__ value,
+                                                            char *__restrict__ k_cache, char *__restrict__ v_cache,
+                                                            const int64_t *__restrict__ slot_mapping, int block_size,
+                                                            int row_bytes, int64_t block_stride_bytes,
+                                                            int64_t key_stride_bytes, int64_t value_stride_bytes) {
+  const int64_t tok = blockIdx.x;
+  const int64_t slot = slot_mapping[tok];
+  if (slot < 0) return;  // a padded token
+  const int64_t blk = slot / block_size, off = slot % block_size;
+  const int half = blockDim.x >> 1;
+  const bool is_v = threadIdx.x >= half;
+  const int lane = is_v ? threadIdx.x - half : threadIdx.x;
+  const char *src = is_v ? value + tok * value_stride_bytes : key + tok * key_stride_bytes;
+  char *dst = (is_v ? v_cache : k_cache) + blk * block_stride_bytes + off * (int64_t)row_bytes;
+  if (ALIGNED16) {
+    for (int i = lane * 16; i < row_bytes; i += half * 16)
+      *reinterpret_cast<u32x4 *>(dst + i) = *reinterpret_cast<const u32x4 *>(src + i);
+  } else {
+    for (int i = lane * 2; i < row_bytes; i += half * 2)
+      *reinterpret_cast<uint16_t *>(dst + i) = *reinterpret_cast<const uint16_t *>(src + i);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Block copies across layers (replaces vllm::copy_blocks_kernel, csrc/cache_kernels.cu:74-100).
-// grid (num_layers, num_pairs)
-__global__ void __launch_bounds__(256) copy_blocks_kernel(const uint64_t *__restrict__ key_caches,
-                                                          const uint64_t *__restrict__ value_caches,
-                                                          const int64_t *__restrict__ mapping, int64_t block_bytes) {
+// grid (layers of this launch, num_pairs).  The layers' base addresses travel in the kernel-argument block,
+// up to kCopyLayers per launch: nothing to allocate, upload or wait for on the host (the reference builds two
+// device tensors of pointers per call, csrc/cache_kernels.cu:117-132).
+constexpr int kCopyLayers = 128;
+struct LayerTable {
+  uint64_t key[kCopyLayers], value[kCopyLayers];
+};
+__global__ void __launch_bounds__(256) copy_blocks_kernel(LayerTable layers, const int64_t *__restrict__ mapping,
+                                                          int64_t block_bytes) {
   const int layer = blockIdx.x, pair = blockIdx.y;
   const int64_t src = mapping[2 * pair] * block_bytes, dst = mapping[2 * pair + 1] * block_bytes;
-  char *kc = reinterpret_cast<char *>(key_caches[layer]);
-  char *vc = reinterpret_cast<char *>(value_caches[layer]);
+  char *kc = reinterpret_cast<char *>(layers.key[layer]);
+  char *vc = reinterpret_cast<char *>(layers.value[layer]);
   for (int64_t i = (int64_t)threadIdx.x * 16; i < block_bytes; i += (int64_t)blockDim.x * 16) {
     *reinterpret_cast<u32x4 *>(kc + dst + i) = *reinterpret_cast<const u32x4 *>(kc + src + i);
     *reinterpret_cast<u32x4 *>(vc + dst + i) = *reinterpret_cast<const u32x4 *>(vc + src + i);
@@ -347,19 +380,44 @@ int vtkv_copy_blocks(const uint64_t *key_caches, const uint64_t *value_caches, i
   VTKV_REQUIRE(block_bytes > 0 && block_bytes % 16 == 0, "block_bytes must be a positive multiple of 16");
   VTKV_REQUIRE(num_pairs <= 65535, "more than 65535 pairs in one call");
   hipStream_t st = (hipStream_t)stream;
-  // the layer base addresses travel as a small device array (stream-ordered allocation would hide
-  // a sync; the reference synchronises here as well, csrc/cache_kernels.cu:127-132)
-  uint64_t *dev = nullptr;
-  VTKV_HIP(hipMalloc((void **)&dev, (size_t)num_layers * 16));
-  VTKV_HIP(hipMemcpyAsync(dev, key_caches, (size_t)num_layers * 8, hipMemcpyHostToDevice, st));
-  VTKV_HIP(hipMemcpyAsync(dev + num_layers, value_caches, (size_t)num_layers * 8, hipMemcpyHostToDevice, st));
-  hipLaunchKernelGGL(copy_blocks_kernel, dim3(num_layers, num_pairs), dim3(256), 0, st, dev, dev + num_layers,
-                     mapping, block_bytes);
-  hipError_t e = hipGetLastError();
-  hipError_t e2 = hipStreamSynchronize(st);
-  (void)hipFree(dev);
-  VTKV_HIP(e);
-  VTKV_HIP(e2);
+  for (int at = 0; at < num_layers; at += kCopyLayers) {
+    const int n = std::min(kCopyLayers, num_layers - at);
+    LayerTable layers = {};
+    for (int l = 0; l < n; ++l) {
+      VTKV_REQUIRE(key_caches[at + l] % 16 == 0 && value_caches[at + l] % 16 == 0, "caches must be 16-byte aligned");
+      layers.key[l] = key_caches[at + l];
+      layers.value[l] = value_caches[at + l];
+    }
+    hipLaunchKernelGGL(copy_blocks_kernel, dim3(n, num_pairs), dim3(256), 0, st, layers, mapping, block_bytes);
+  }
+  VTKV_HIP(hipGetLastError());
+  return VTKV_OK;
+}
+
+int vtkv_reshape_and_cache_flash(const void *key, const void *value, void *k_cache, void *v_cache,
+                                 const int64_t *slot_mapping, int num_tokens, int num_heads, int head_size,
+                                 int block_size, int64_t block_stride, int64_t key_stride, int64_t value_stride,
+                                 int elem_bytes, void *stream) {
+  VTKV_REQUIRE(key && value && k_cache && v_cache && slot_mapping, "null argument");
+  VTKV_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "elem_bytes must be 2 or 4");
+  VTKV_REQUIRE(num_heads > 0 && head_size > 0 && block_size > 0, "bad sizes");
+  const int64_t row_elems = (int64_t)num_heads * head_size;
+  VTKV_REQUIRE(key_stride >= row_elems && value_stride >= row_elems && block_stride >= row_elems * block_size,
+               "a stride is smaller than what it steps over");
+  if (num_tokens <= 0) return VTKV_OK;
+  const int row_bytes = (int)(row_elems * elem_bytes);
+  const bool aligned = row_bytes % 16 == 0 && (key_stride * elem_bytes) % 16 == 0 && (value_stride * elem_bytes) % 16 == 0 &&
+                       (block_stride * elem_bytes) % 16 == 0 && (uintptr_t)key % 16 == 0 && (uintptr_t)value % 16 == 0 &&
+                       (uintptr_t)k_cache % 16 == 0 && (uintptr_t)v_cache % 16 == 0;
+  const int threads = aligned ? std::min(256, std::max(64, 2 * ((row_bytes / 16 + 31) / 32 * 32))) : 256;
+  hipStream_t st = (hipStream_t)stream;
+#define LAUNCH_FLASH(A)                                                                                          \
+  hipLaunchKernelGGL(scatter_flash_kernel<A>, dim3(num_tokens), dim3(threads), 0, st, (const char *)key,         \
+                     (const char *)value, (char *)k_cache, (char *)v_cache, slot_mapping, block_size, row_bytes, \
+                     block_stride * elem_bytes, key_stride * elem_bytes, value_stride * elem_bytes)
+  if (aligned) LAUNCH_FLASH(true); else LAUNCH_FLASH(false);
+#undef LAUNCH_FLASH
+  VTKV_HIP(hipGetLastError());
   return VTKV_OK;
 }
 

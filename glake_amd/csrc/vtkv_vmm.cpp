@@ -607,16 +607,17 @@ vtkv_segment *vtkv_seg_create(int layer_num, int64_t context_max_bytes, int64_t 
   if (!(s) || !g_pool.segments.count(const_cast<vtkv_segment *>(s)))                                  \
   return vtkv::fail(VTKV_ESTATE, "not a live segment")
 
-// Before a call that grows a segment: let its map-ahead requests finish, and report one that failed (also
-// when it failed a while ago and nothing is pending any more).
+// Before a call that grows a segment: let its map-ahead requests finish, and report one that failed with a
+// driver error (also when it failed a while ago and nothing is pending any more).  A request that found the
+// pool empty is advisory only: it asked for a chunk ahead of need, the pool may have chunks again by now, and
+// the call at hand maps what its own rows need and fails by itself if that cannot be had.
 #define SEG_SETTLE(s)                                                                                 \
   do {                                                                                                \
     settle(lk, (s));                                                                                  \
     if ((s)->async_error) {                                                                           \
       const int e_ = (s)->async_error;                                                                \
       (s)->async_error = 0;                                                                           \
-      return vtkv::fail(e_, "a map-ahead request of this segment failed (%s)",                        \
-                        e_ == VTKV_ENOMEM ? "chunk pool exhausted" : "driver error");                 \
+      if (e_ != VTKV_ENOMEM) return vtkv::fail(e_, "a map-ahead request of this segment failed (driver error)"); \
     }                                                                                                 \
   } while (0)
 // Before a call that shrinks a segment (preempt, release, destroy): let its map-ahead requests finish and
@@ -846,9 +847,13 @@ int vtkv_map_ahead_batch(vtkv_segment *const *segs, int n, int64_t ahead_bytes) 
   // only what the pool can serve now is asked for: a request that fails is reported by the segment's next
   // growth, and a sequence may finish before it needs the chunk
   int64_t spare = (int64_t)g_pool.free_chunks.size() + g_pool.retired;
+  // chunks that requests still in the queue will take (earlier calls, vtkv_seg_eager_extend) are spoken for;
+  // counted in full, a retired chunk a request may revive instead only makes the estimate more careful
+  for (const auto &rq : g_pool.requests) spare -= 2ll * rq.seg->layer_num * rq.chunks;
   int queued = 0;
   for (int i = 0; i < n; ++i) {
     vtkv_segment *s = segs[i];
+    if (s->async_error == VTKV_ENOMEM) s->async_error = 0;  // an earlier request found the pool empty: ask again
     if (s->pending || s->async_error || s->mapped >= s->context_max) continue;
     if (s->used + s->v_skew + ahead_bytes <= s->mapped) continue;
     const int64_t revive = s->held > s->mapped ? 1 : 0;  // a retired chunk of its own comes back without a driver call

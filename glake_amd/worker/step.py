@@ -81,6 +81,19 @@ def prepare_step(attn_metadata, kv_caches: Sequence, kv_cache_dtype: Optional[st
             raise
     attn_metadata.decode_seq_len = decode_seq_len
     attn_metadata.slot_m = torch.tensor(slot_m, dtype=torch.int64, device=device)
+    # The decode sequences' lengths for the fused append + attention launch, which takes up to 512 of them with
+    # its kernel arguments (model_runner.py:607 hands the lengths over on the host as well as on the device).
+    # Made here, once per step and for all layers, from this step's seq_lens; not for a step that is recorded
+    # into a graph, whose replays must read the lengths of their own step from the device.
+    host_lens = None
+    seq_lens = attn_metadata.seq_lens
+    if (n > n_pre and seq_lens is not None and len(seq_lens) == n and n - n_pre <= 512
+            and not getattr(attn_metadata, "use_cuda_graph", False)):
+        import ctypes
+
+        host_lens = (ctypes.c_int32 * (n - n_pre))(*seq_lens[n_pre:])
+    if hasattr(attn_metadata, "_host_decode_lens"):
+        attn_metadata._host_decode_lens = host_lens
 
 
 class DecodeStepPlan:
@@ -116,6 +129,9 @@ class DecodeStepPlan:
             raise _C.VtkvError(_C.EINVAL, "DecodeStepPlan: one slot id per segment, at least one sequence")
         if ring < 2 or ring % 2:
             raise _C.VtkvError(_C.EINVAL, "DecodeStepPlan: ring must be even and at least 2")
+        if model_dtype not in (torch.bfloat16, torch.float16):
+            raise _C.VtkvError(_C.EINVAL, f"DecodeStepPlan: the attention kernels take bfloat16 and float16 queries, "
+                                          f"not {model_dtype}")
         self._C, self._lib, self._np = _C, _C.lib(), np
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         n = self.n = len(segments)

@@ -20,6 +20,8 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the library is built with hidden visibility: what is declared here is what it exports */
+#pragma GCC visibility push(default)
 
 #define VTKV_OK 0
 #define VTKV_EINVAL (-1)   /* bad argument (shape, dtype, alignment, null pointer)      */
@@ -247,9 +249,19 @@ int vtkv_swap_ranges(const uint64_t *src, const uint64_t *dst, const int64_t *by
 void *vtkv_host_alloc(int64_t bytes);
 int vtkv_host_free(void *p);
 
+/* Scatter into the flash-attention cache layout; replaces reshape_and_cache_flash
+ * (csrc/cache_kernels.cu:202-236,299-342; bound at csrc/pybind.cpp:100).  K and V caches are both
+ * [num_blocks, block_size, H, D] with `block_stride` elements between blocks; slot_mapping device
+ * int64[num_tokens] (<0: a padded token, skipped).  Unquantised caches only, as in the reference. */
+int vtkv_reshape_and_cache_flash(const void *key, const void *value, void *k_cache, void *v_cache,
+                                 const int64_t *slot_mapping, int num_tokens, int num_heads, int head_size,
+                                 int block_size, int64_t block_stride, int64_t key_stride, int64_t value_stride,
+                                 int elem_bytes, void *stream);
+
 /* In-GPU block copies across layers; replaces copy_blocks (csrc/cache_kernels.cu:74-149).
- * key_caches/value_caches: HOST arrays of num_layers device base addresses; `mapping`: DEVICE
- * int64[num_pairs,2]; block_bytes must be a multiple of 16. */
+ * key_caches/value_caches: HOST arrays of num_layers device base addresses (16-byte aligned; read before the
+ * call returns, they travel as kernel arguments); `mapping`: DEVICE int64[num_pairs,2]; block_bytes must be a
+ * multiple of 16.  Asynchronous on `stream`: no allocation, no upload, no wait. */
 int vtkv_copy_blocks(const uint64_t *key_caches, const uint64_t *value_caches, int num_layers,
                      const int64_t *mapping, int num_pairs, int64_t block_bytes, void *stream);
 
@@ -288,7 +300,9 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  *                The result does not depend on the choice beyond fp32 summation order.
  * A launch takes up to 1024 sequences; a larger batch runs as consecutive launches of 1024 on `stream` within
  * the one call.
- * Supported: q_dtype VTKV_BF16 or VTKV_F16, kv_dtype = q_dtype or VTKV_FP8_E4M3, head_size 64, 80, 96, 112, 128 or
+ * Supported: q_dtype VTKV_BF16 or VTKV_F16 (VTKV_F32 queries are refused with VTKV_EINVAL: the reference's kernel
+ * tests also run float, tests/kernels/test_attention.py:23, but its vTensor path serves 16-bit models only, see
+ * xformers.py:362-385), kv_dtype = q_dtype or VTKV_FP8_E4M3, head_size 64, 80, 96, 112, 128 or
  * 256 (the reference's list, vllm/attention/ops/paged_attn.py:33-34), any whole num_heads/num_kv_heads.  The kernel
  * is tuned for bf16 and head size 128; the other shapes run the same code with their own tile constants.  A kv head
  * with more than 16 query heads (multi-query models) is served in ceil(n/16) parts of equal size (the last may be
@@ -309,7 +323,12 @@ int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const
  * vtkv_decode_attention with partition_tokens = 0 and gives the same result bit for bit.  Sizes whose scratch
  * does not fit (roughly num_seqs * num_heads above 45 000) are refused with VTKV_EINVAL.  All calls on one GPU
  * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race on it and must
- * be ordered by the caller; vtkv_set_kernel_timing does not apply to this entry point. */
+ * be ordered by the caller; vtkv_set_kernel_timing does not apply to this entry point.
+ * Under HIP graph capture: the first call on a device looks up the array's address and the kernels' occupancy
+ * (hipGetSymbolAddress, an occupancy query), which are not stream work and must not happen while a stream is
+ * capturing, so make one call on each device outside capture first; every later call only launches kernels (the
+ * arrival counters are cleared by a kernel, not a memset) and can be recorded and replayed, with seq_lens read
+ * from device memory at every replay. */
 int64_t vtkv_decode_attention_noalloc_max_bytes(void);
 int vtkv_decode_attention_noalloc(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                                   const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
@@ -412,6 +431,7 @@ int vtkv_set_head_major(int on);
 int vtkv_set_kernel_timing(int on);
 int vtkv_attention_kernel_times(float *stream_ms, float *reduce_ms, int capacity);
 
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

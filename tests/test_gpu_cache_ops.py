@@ -206,6 +206,66 @@ def test_paged_scatter_matches_reference_fixture_inputs(dtype):
     assert np.array_equal(back(gk), kc) and np.array_equal(back(gv), vc)
 
 
+@pytest.mark.parametrize("num_heads,head_size,block_size,dtype",
+                         [(8, 64, 8, "bf16"), (8, 80, 16, "f32"), (8, 128, 32, "bf16"), (8, 256, 16, "f16"), (3, 66, 16, "bf16")])
+def test_flash_layout_scatter_like_the_reference_test(num_heads, head_size, block_size, dtype):
+    """tests/kernels/test_cache.py:206-270: 42 tokens of a fused qkv tensor to random slots of K and V caches
+    [num_blocks, block_size, H, D]; the expectation is the reference test's own closed form
+    cache[slot // block_size, slot % block_size] = row, a padded token (slot -1) is skipped, bytes exact.
+    (3 heads of 66 make rows that are no multiple of 16 bytes: the 2-byte path.)"""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    random.seed(0)
+    rng = np.random.default_rng(head_size)
+    num_tokens, num_blocks = 42, 1024
+    slots = random.sample(range(block_size * num_blocks), num_tokens)
+    slots[5] = -1
+    np_t, t_t = {"bf16": (np.uint16, torch.bfloat16), "f16": (np.uint16, torch.float16), "f32": (np.uint32, torch.float32)}[dtype]
+    bits = 8 * np.dtype(np_t).itemsize
+    qkv = rng.integers(0, 1 << bits, (num_tokens, 3, num_heads, head_size), dtype=np.uint64).astype(np_t)
+    kc = rng.integers(0, 1 << bits, (num_blocks, block_size, num_heads, head_size), dtype=np.uint64).astype(np_t)
+    vc = rng.integers(0, 1 << bits, (num_blocks, block_size, num_heads, head_size), dtype=np.uint64).astype(np_t)
+    if dtype == "f32":  # keep the patterns finite floats: NaN payloads need not survive a .cuda()
+        qkv &= np.uint32(0xBF7FFFFF); kc &= np.uint32(0xBF7FFFFF); vc &= np.uint32(0xBF7FFFFF)
+    signed = np.int16 if bits == 16 else np.int32
+    to_t = lambda a: torch.from_numpy(a.view(signed)).cuda().view(t_t)
+    back = lambda t: t.view(torch.int16 if bits == 16 else torch.int32).cpu().numpy().view(np_t)
+    g_qkv, g_k, g_v = to_t(qkv), to_t(kc), to_t(vc)
+    ops.reshape_and_cache_flash(g_qkv[:, 1], g_qkv[:, 2], g_k, g_v, torch.tensor(slots, dtype=torch.int64, device="cuda"),
+                                "auto")
+    torch.cuda.synchronize()
+    for i, s_ in enumerate(slots):
+        if s_ < 0:
+            continue
+        kc[s_ // block_size, s_ % block_size] = qkv[i, 1]
+        vc[s_ // block_size, s_ % block_size] = qkv[i, 2]
+    assert np.array_equal(back(g_k), kc) and np.array_equal(back(g_v), vc)
+    with pytest.raises(Exception):
+        ops.reshape_and_cache_flash(g_qkv[:, 1], g_qkv[:, 2], g_k, g_v, torch.tensor(slots, dtype=torch.int64, device="cuda"),
+                                    "fp8")
+
+
+def test_copy_blocks_takes_more_layers_than_one_launch_holds():
+    """160 layers (two launches of the layer table), small blocks, and the call returns without waiting."""
+    import torch
+
+    from glake_amd import _custom_ops as ops
+
+    rng = np.random.default_rng(8)
+    layers, num_blocks = 160, 12
+    mapping = [(0, 5), (3, 7), (3, 11), (9, 1)]
+    ks = [rng.integers(0, 65536, (num_blocks, 2, 4, 8)).astype(np.uint16) for _ in range(layers)]
+    vs = [rng.integers(0, 65536, (num_blocks, 2, 4, 8)).astype(np.uint16) for _ in range(layers)]
+    gk, gv = [torch_bf16_from_bits(k) for k in ks], [torch_bf16_from_bits(v) for v in vs]
+    ops.copy_blocks(gk, gv, torch.tensor(mapping, dtype=torch.int64, device="cuda"))
+    O.copy_blocks(ks, vs, np.array(mapping))
+    torch.cuda.synchronize()
+    for a, b in zip(gk + gv, ks + vs):
+        assert np.array_equal(bits_from_torch_bf16(a), b)
+
+
 def test_copy_blocks_like_the_reference_test():
     """tests/kernels/test_cache.py:31-102: every source block copied to two destinations, 3 layers."""
     import torch

@@ -30,6 +30,41 @@ def to_model(x32, dtype):
     return b, O.bf16_to_f32(b)
 
 
+def check_partition_buffers(side, out, q32, k32, v32, lens, hq, hkv, d, scale, slopes):
+    """The caller's buffers of paged_attention_v2 (csrc/attention/attention_kernels.cu:451-583): partition j of a
+    sequence is rows [512 j, 512 j + 512).  tmp_out[j] is plain attention over those rows alone (a softmax does not
+    see the constant that ALiBi's `- seq_len + 1` adds inside a partition, so the v1 oracle on a slice of the cache
+    with the slice's own length gives it), max_logits and exp_sums come from a float64 q.K^T with the ALiBi bias of
+    the row's place in the whole sequence (:404-419 qk_max carries it), and merging the buffers by the reference's
+    rule (:515-582) gives `out` again."""
+    import torch
+
+    es, ml, tmp = (t.float().cpu().numpy() for t in side)
+    g, tol = hq // hkv, 2e-3
+    step = 2.0 ** -8 if side[2].dtype == torch.bfloat16 else 2.0 ** -11
+    for i, n in enumerate(lens):
+        np_i = (n + 511) // 512
+        assert np.all(es[i, :, np_i:] == -7.0) and np.all(ml[i, :, np_i:] == -7.0) and np.all(tmp[i, :, np_i:] == -7.0)
+        for j in range(np_i):
+            lo, hi = 512 * j, min(n, 512 * j + 512)
+            sl_k, sl_v = np.ascontiguousarray(k32[i][lo:hi]), np.ascontiguousarray(v32[i][lo:hi])
+            part = O.paged_attention_v1(q32[i:i + 1], O.VTensorCache([sl_k], [sl_v], np.zeros(1, np.int64), hkv, d),
+                                        scale, [hi - lo], slopes)[0]
+            # tmp_out is stored in the model's type: one more rounding
+            assert np.all(np.abs(tmp[i, :, j] - part) <= tol + (tol + step) * np.abs(part))
+            for h in range(hq):
+                s = scale * (sl_k[:, h // g].astype(np.float64) @ q32[i, h].astype(np.float64))
+                if slopes is not None:
+                    s = s + float(slopes[h]) * (np.arange(lo, hi) - n + 1)
+                assert abs(ml[i, h, j] - s.max()) <= 1e-4 + 1e-5 * abs(s.max())
+                sm = np.exp(s - s.max()).sum()
+                assert abs(es[i, h, j] - sm) <= 1e-4 * sm
+        m = ml[i, :, :np_i].max(axis=1, keepdims=True)
+        w = es[i, :, :np_i] * np.exp(ml[i, :, :np_i] - m)
+        merged = (tmp[i, :, :np_i] * w[..., None]).sum(axis=1) / (w.sum(axis=1, keepdims=True) + 1e-6)
+        assert np.all(np.abs(merged - out[i]) <= 4e-3 + 4e-3 * np.abs(out[i]))
+
+
 def run_case(vmm, seed, lens, hq, hkv, d, dtype, fp8=False, alibi=False, version="v1", partition_tokens=0):
     import torch
 
@@ -71,22 +106,26 @@ def run_case(vmm, seed, lens, hq, hkv, d, dtype, fp8=False, alibi=False, version
     al = None if slopes is None else torch.from_numpy(slopes).cuda()
     out32 = torch.empty(b, hq, d, dtype=torch.float32, device="cuda")
     out16 = torch.empty(b, hq, d, dtype=tdt, device="cuda")
+    side = None
     for o in (out32, out16):
         if version == "v1":
             ops.paged_attention_v1(o, q_t, kt, vt, hkv, scale, sl, 1, max(lens), al, "fp8" if fp8 else "auto", k_scale,
                                    slots, v_scale=v_scale, partition_tokens=partition_tokens)
         else:
-            parts = (max(lens) + 511) // 512
-            es = torch.zeros(b, hq, parts, dtype=torch.float32, device="cuda")
-            ml = torch.zeros_like(es)
-            tmp = torch.zeros(b, hq, parts, d, dtype=tdt, device="cuda")
+            parts = (max(lens) + 511) // 512 + 1           # one spare partition column: must stay untouched
+            es = torch.full((b, hq, parts), -7.0, dtype=torch.float32, device="cuda")
+            ml = torch.full((b, hq, parts), -7.0, dtype=torch.float32, device="cuda")
+            tmp = torch.full((b, hq, parts, d), -7.0, dtype=tdt, device="cuda")
             ops.paged_attention_v2(o, es, ml, tmp, q_t, kt, vt, hkv, scale, sl, 1, max(lens), al,
                                    "fp8" if fp8 else "auto", k_scale, slots, v_scale=v_scale)
+            side = (es, ml, tmp)
     torch.cuda.synchronize()
     gpu.close()
     got = out32.cpu().numpy()
     assert np.isfinite(got).all()
     want = O.paged_attention_v1(q32, O.VTensorCache(k32, v32, np.arange(b), hkv, d), scale, lens, slopes)
+    if side is not None:
+        check_partition_buffers(side, got, q32, k32, v32, lens, hq, hkv, d, scale, slopes)
     err = np.abs(got - want)
     ok = bool(np.all(err <= 2e-3 + 2e-3 * np.abs(want)))
     assert ok, f"max err {err.max():.3e} at {np.unravel_index(err.argmax(), err.shape)}"
@@ -119,11 +158,19 @@ def test_forty_heads_without_grouping_and_alibi(gpu_pool, d, dtype):
     run_case(gpu_pool, 200 + d, [33, 700, 1, 2049, 130], 40, 40, d, dtype, alibi=True)
 
 
-@pytest.mark.parametrize("d,dtype,fp8", [(64, "f16", False), (80, "bf16", True), (96, "f16", True), (112, "bf16", False),
-                                         (256, "f16", False)])
-def test_split_k_interface_and_fixed_partitions_on_other_head_sizes(gpu_pool, d, dtype, fp8):
-    run_case(gpu_pool, 300 + d, [513, 2000, 100, 1025], 32, 8, d, dtype, fp8=fp8, version="v2")
-    run_case(gpu_pool, 400 + d, [513, 2000, 100, 1025], 32, 8, d, dtype, fp8=fp8, partition_tokens=256)
+@pytest.mark.parametrize("d,dtype,fp8,alibi,heads", [
+    (64, "f16", False, False, (32, 8)), (64, "bf16", False, True, (32, 8)), (80, "bf16", True, False, (32, 8)),
+    (80, "f16", False, True, (32, 8)), (96, "f16", True, True, (32, 8)), (112, "bf16", False, False, (32, 8)),
+    (112, "f16", True, True, (64, 8)), (128, "f16", False, True, (32, 8)), (128, "bf16", False, True, (32, 8)),
+    (128, "f16", True, False, (32, 8)), (128, "bf16", True, True, (64, 8)), (256, "f16", False, False, (32, 8)),
+    (256, "bf16", True, True, (16, 4)), (128, "bf16", False, True, (40, 2)), (96, "bf16", False, True, (40, 40))])
+def test_split_k_interface_and_fixed_partitions_on_other_head_sizes(gpu_pool, d, dtype, fp8, alibi, heads):
+    """The split-K interface with the caller's buffers over head sizes, fp16, fp8 rows and ALiBi, with head counts that
+    take the variants of several kv heads per segment (32 over 8 at 64 to 112), the padded head sizes and kv heads
+    served in parts (40 over 2): every partition's max, sum and partial result, not only the merged output."""
+    hq, hkv = heads
+    run_case(gpu_pool, 300 + d, [513, 2000, 100, 1025, 1], hq, hkv, d, dtype, fp8=fp8, alibi=alibi, version="v2")
+    run_case(gpu_pool, 400 + d, [513, 2000, 100, 1025], hq, hkv, d, dtype, fp8=fp8, alibi=alibi, partition_tokens=256)
 
 
 def test_long_context_on_a_small_head_and_a_large_one(gpu_pool):

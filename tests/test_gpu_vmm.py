@@ -234,7 +234,8 @@ def test_map_ahead_requests_run_on_the_worker_and_settle(gpu_pool):
     segs[2].eagerExtend(row, 0)
     vmm.wait_map_ahead()
     assert segs[2].actual_size == 6 * CHUNK
-    # a request the pool cannot serve: reported by the next call on that segment, nothing half-mapped
+    # a request the pool cannot serve leaves nothing half-mapped and no error behind; growth that the pool
+    # still cannot serve fails by itself
     hog = vmm.KVcacheSegment(1, (vmm.showFreeBlocks() // 2 + 2) * CHUNK, 0, False)
     hog.expandMultiSegment((vmm.showFreeBlocks() - 2) // 2)      # leaves fewer chunks than segs[4] needs
     segs[4].eagerExtend(row, 0)
@@ -291,8 +292,9 @@ def test_map_ahead_batch_asks_for_what_is_about_to_be_needed(gpu_pool):
 
 def test_failed_map_ahead_does_not_stop_a_preemption(gpu_pool):
     """Pool exhausted, a map-ahead request fails: calls that shrink the segment still do their work (that is how
-    the scheduler gets chunks back), the failure is reported once by the next call that grows it, and a step
-    that fails part of the way leaves every sequence's used size as it was."""
+    the scheduler gets chunks back), the failed request is advisory (a step whose rows fit what is mapped runs,
+    a row that needs the chunk maps it in the calling thread), and a step that fails part of the way because the
+    pool really is empty leaves every sequence's used size as it was."""
     from glake_amd import _C
 
     vmm = gpu_pool
@@ -316,21 +318,63 @@ def test_failed_map_ahead_does_not_stop_a_preemption(gpu_pool):
     assert vmm.showFreeBlocks() >= 2
     segs[0].expandMultiSegment(1)                                # the old failure is forgotten, not reported here
     segs[0].preempt_seq(0)
-    # a growing call reports the stale failure once, although nothing is pending, and rolls the step back
+    # rows that fit what is mapped: the failed requests of segs[1] and segs[2] do not fail the step
     used = [s.used_size for s in segs[1:]]
-    with pytest.raises(_C.VtkvOutOfChunks):
-        vmm.extend_kv_cache_batch(None, None, [1, 2], [row, row], segs[1:], [0, 0], row, True)
-    assert [s.used_size for s in segs[1:]] == used
-    with pytest.raises(_C.VtkvOutOfChunks):                      # segs[2]'s own failure, reported in its turn
-        vmm.extend_kv_cache_batch(None, None, [1, 2], [row, row], segs[1:], [0, 0], row, True)
-    assert [s.used_size for s in segs[1:]] == used
     slot_m = vmm.extend_kv_cache_batch(None, None, [1, 2], [row, row], segs[1:], [0, 0], row, True)
     assert slot_m == used and [s.used_size for s in segs[1:]] == [u + row for u in used]
+    # the next rows cross the chunk boundary.  The pool holds exactly the two chunks of one sequence (K and V):
+    # the first sequence maps them in the calling thread, the second finds the pool empty, and the step is
+    # rolled back as a whole (the first sequence keeps its chunk, not its row)
+    assert 2 <= vmm.showFreeBlocks() < 4
+    used = [s.used_size for s in segs[1:]]
+    with pytest.raises(_C.VtkvOutOfChunks):
+        vmm.extend_kv_cache_batch(None, None, [1, 2], [2 * row, 2 * row], segs[1:], [0, 0], row, True)
+    assert [s.used_size for s in segs[1:]] == used and segs[1].actual_size == 2 * CHUNK
+    # the caller preempts the second sequence and runs the step again with what is left
+    segs[2].preempt_seq(2)
+    slot_m = vmm.extend_kv_cache_batch(None, None, [1], [2 * row], segs[1:2], [0], row, True)
+    assert slot_m == used[:1] and segs[1].used_size == used[0] + 2 * row
     segs[1].release_seq(1)
     hog.destroy()
     for s in segs:
         s.destroy()
     assert vmm.showFreeBlocks() == free0
+
+
+def test_map_ahead_that_loses_the_race_for_the_last_chunks_is_not_an_error(gpu_pool):
+    """A pool with exactly the chunks the step itself needs: requests made ahead of need count what earlier
+    requests in the queue will take, one that comes too late leaves no error, and the rows that need a chunk now
+    get it from the calling thread."""
+    vmm = gpu_pool
+    vmm.trim()
+    row, layers = 2048, 2
+    segs = [vmm.KVcacheSegment(layers, 4 * CHUNK, 0, False) for _ in range(3)]
+    for s in segs:
+        s.expandMultiSegment(1)
+        s.set_used_size(CHUNK - 3 * row)
+    spare = vmm.showFreeBlocks()
+    hog = vmm.KVcacheSegment(1, (spare // 2 + 2) * CHUNK, 0, False)
+    hog.expandMultiSegment((spare - 2 * layers) // 2)             # leaves the chunks of ONE growth step (4 or 5)
+    assert 2 * layers <= vmm.showFreeBlocks() < 4 * layers
+    # an explicit request takes them; the batch call that follows knows and asks for nothing
+    segs[0].eagerExtend(row, 0)
+    assert vmm.map_ahead_batch(segs[1:], 40 * row) == 0
+    vmm.wait_map_ahead()
+    assert segs[0].actual_size == 2 * CHUNK and segs[1].actual_size == CHUNK
+    # a request that cannot be served any more fails in the worker and is forgotten
+    segs[1].eagerExtend(row, 0)
+    vmm.wait_map_ahead()
+    assert segs[1].actual_size == CHUNK
+    for _ in range(3):                                            # rows that still fit: no error
+        vmm.extend_kv_cache_batch(None, None, [1], [row], segs[1:2], [0], row, True)
+    hog.preempt_seq(0)                                            # chunks come back; the row that crosses maps in the caller
+    vmm.extend_kv_cache_batch(None, None, [1], [row], segs[1:2], [0], row, True)
+    assert segs[1].actual_size == 2 * CHUNK and segs[1].used_size == CHUNK + row
+    assert vmm.map_ahead_batch(segs[2:], 40 * row) == 1           # and a later request is made again
+    vmm.wait_map_ahead()
+    assert segs[2].actual_size == 2 * CHUNK
+    for s in segs + [hog]:
+        s.destroy()
 
 
 def test_shared_prefix_maps_whole_chunks_twice_and_copies_the_tail(gpu_pool):

@@ -107,3 +107,67 @@ def test_noalloc_entry_point_refuses_what_its_scratch_cannot_hold(gpu_pool):
     rc = lib.vtkv_decode_attention_noalloc(p(out), p(dummy), p(tab), p(tab), p(tab), p(lens), b, hq, hkv, d, hq * d,
                                            1.0, 1, None, _C.BF16, _C.F32, _C.BF16, 1.0, 1.0, None)
     assert rc == _C.EINVAL and "static scratch" in _C.last_error()
+
+
+@pytest.mark.parametrize("merge", [0, 1])
+def test_noalloc_entry_point_under_graph_capture_and_without_allocations(gpu_pool, merge):
+    """What the entry point is for.  After one call outside capture (the first call on a device looks up the
+    scratch's address and the kernels' occupancy), a call is recorded into a HIP graph and replayed three times
+    with other lengths in the device-side seq_lens, eager calls and synchronisations in between; every replay is
+    compared with the oracle and with the eager call.  Free device memory (hipMemGetInfo) and torch's own
+    allocation counters are the same before and after the eager calls."""
+    import torch
+
+    from glake_amd import _C
+
+    lib = _C.lib()
+    rng = np.random.default_rng(23)
+    hq, hkv, d = 32, 8, 128
+    scale = d ** -0.5
+    cap = [700, 64, 1500, 2100, 33, 900]
+    b = len(cap)
+    gpu = GpuSeqs(gpu_pool, b, hkv, d, 2, max(cap), value_skew=256)
+    ks = [bf16_randn(rng, (n, hkv, d)) for n in cap]
+    vs = [bf16_randn(rng, (n, hkv, d)) for n in cap]
+    for i in range(b):
+        gpu.upload(i, ks[i], vs[i])
+    kt, vt = gpu.table_tensors()
+    q = bf16_randn(rng, (b, hq, d))
+    q_t = torch_bf16_from_bits(q)
+    slot_t = torch.arange(b, dtype=torch.int64, device="cuda")
+    sl_t = torch.tensor(cap, dtype=torch.int32, device="cuda")
+    out_graph = torch.zeros(b, hq, d, dtype=torch.float32, device="cuda")
+    out_eager = torch.zeros_like(out_graph)
+    lens_sets = [cap, [n // 2 + 1 for n in cap], [1, 64, 17, 2100, 33, 5], [n - 1 for n in cap]]
+    staged = [torch.tensor(l, dtype=torch.int32, device="cuda") for l in lens_sets]
+    want = [O.paged_attention_v1(O.bf16_to_f32(q), O.VTensorCache(ks, vs, np.arange(b), hkv, d), scale, l)
+            for l in lens_sets]
+    _C.check(lib.vtkv_set_fused_merge(merge))
+    try:
+        call = lambda out: attend("noalloc", out, q_t, kt, vt, slot_t, sl_t, b, hq, hkv, d, scale, max(cap), _C.BF16,
+                                  1.0, 1.0)
+        call(out_eager)                      # the first call on this device, outside capture
+        torch.cuda.synchronize()
+        free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+        for _ in range(3):
+            call(out_eager)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0, "free device memory changed across noalloc calls"
+        assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            call(out_graph)
+        for i, lens in enumerate(lens_sets):
+            sl_t.copy_(staged[i])
+            out_graph.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = out_graph.cpu().numpy()
+            err = np.abs(got - want[i])
+            assert np.all(err <= 2e-3 + 2e-3 * np.abs(want[i])), f"replay {i}: max err {err.max():.3e}"
+            call(out_eager)                  # eager work between the replays, on the same scratch
+            torch.cuda.synchronize()
+            assert torch.equal(out_graph, out_eager), f"replay {i} differs from the eager call"
+    finally:
+        _C.check(lib.vtkv_set_fused_merge(-1))
+        gpu.close()
