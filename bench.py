@@ -175,6 +175,9 @@ def main() -> int:
                     help="bytes between the base of a V range and its first row (0 = the reference's placement)")
     ap.add_argument("--head-major", default="auto", choices=["auto", "on", "off"],
                     help="tile order of the decode kernel: (kv head, sequence, rows) or (sequence, kv head, rows)")
+    ap.add_argument("--workgroup-trace", action="store_true",
+                    help="with a library built by `python -m glake_amd.build --define VTKV_ATTN_TRACE --out X` "
+                         "(VTKV_LIBRARY_PATH=X): when the workgroups of the decode kernel's last launch ended, by XCD")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", action="store_true",
                     help="with --config c2: leave out the other BASELINE configurations (c3, c4 and the growth-and-swap "
@@ -431,6 +434,28 @@ def decode_run(args, config: str, R: int, with_swap: bool, with_cpu: bool) -> di
 
     final_lens = [s.get_used_slot() // row for s in segs]
 
+    trace = None
+    if args.workgroup_trace:
+        # the tracing build keeps {XCC id, start, span, end, tiles} of every workgroup of the last launch (100 MHz clock)
+        torch.cuda.synchronize()
+        step()
+        torch.cuda.synchronize()
+        buf = (C.c_ulonglong * (1024 * 6))()
+        fn = lib.vtkv_debug_attn_trace
+        fn.argtypes = [C.c_void_p, C.c_int]
+        _C.check(fn(buf, 1024))
+        t = np.array(list(buf), dtype=np.int64).reshape(1024, 6)
+        t = t[t[:, 1] > 0]
+        t0 = t[:, 1].min()
+        end = (t[:, 3] - t0) / 100.0
+        trace = {"workgroups": int(len(t)), "end_us": {"min": round(float(end.min()), 1), "mean": round(float(end.mean()), 1),
+                                                        "p90": round(float(np.percentile(end, 90)), 1),
+                                                        "max": round(float(end.max()), 1)},
+                 "start_spread_us": round(float((t[:, 1].max() - t0) / 100.0), 1),
+                 "end_us_mean_by_xcc": [round(float(end[t[:, 0] == x].mean()), 1) for x in range(8)],
+                 "end_us_by_dispatch_third": [round(float(end[(t[:, 2] % (len(t) // 8)) * 3 // (len(t) // 8) == k].mean()), 1)
+                                              for k in range(3)]}
+
     # ---- swap: 25 % of the sequences out to pinned host memory and back.  Unmapping is lazy, so a
     # sequence swapped back in before its chunks were needed elsewhere finds them still mapped ("warm");
     # the second round trip forces the unmapping in between ("cold": swap-in has to map every chunk).
@@ -480,6 +505,7 @@ def decode_run(args, config: str, R: int, with_swap: bool, with_cpu: bool) -> di
         "ms_per_layer": round(ms_per_step / L, 4),
         "host_issue_ms_per_step": round(host_dt / K * 1e3, 4),
         "swap": swap,
+        "workgroup_trace": trace,
         "roofline": roofline,
         # matrix pipe of the dominant kernel, from the same counter runs as `traffic`: the share of SIMD
         # cycles with an MFMA executing, and the part of it that is real work (G of the 16 head columns)

@@ -67,4 +67,12 @@ def build_library(verbose: bool = False, out_path: str = LIB_PATH, extra_flags=(
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    import argparse
+
+    ap = argparse.ArgumentParser(description="compile libvtkv.so for gfx950")
+    ap.add_argument("--define", action="append", default=[], metavar="NAME[=VALUE]",
+                    help="a tuning build: -DNAME[=VALUE] for every source (e.g. VTKV_ATTN_TRACE: the decode kernel "
+                         "records when each of its workgroups starts and ends, for bench.py --workgroup-trace)")
+    ap.add_argument("--out", default=LIB_PATH, help="where the shared object goes (VTKV_LIBRARY_PATH selects it at run time)")
+    cli = ap.parse_args()
+    print(build_library(verbose=True, out_path=os.path.abspath(cli.out), extra_flags=["-D" + d for d in cli.define]))

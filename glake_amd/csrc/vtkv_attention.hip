@@ -66,6 +66,12 @@ static_assert(VTKV_ATTN_STAGES >= 1 && VTKV_ATTN_STAGES <= 4, "1 to 4 register t
 #include "vtkv_attn_common.h"
 #include "vtkv_fp8.h"
 
+#ifdef VTKV_ATTN_TRACE
+// Tuning builds only: per workgroup of the last launch {XCC id, start, first segment's loads issued, end of the
+// streaming loop, end} on the 100 MHz wall clock.
+__device__ unsigned long long g_attn_trace[4096][6];
+#endif
+
 namespace {
 
 using namespace vtkv_attn;
@@ -82,6 +88,12 @@ constexpr int kStagesFp8 = VTKV_ATTN_FP8_STAGES;  // likewise for the fp8 varian
 #endif
 #ifndef VTKV_ATTN_FP8_WAVES
 #define VTKV_ATTN_FP8_WAVES 3  // waves per SIMD of the fp8 variants
+#endif
+#ifndef VTKV_ATTN_SMALL_WAVES
+#define VTKV_ATTN_SMALL_WAVES 2      // waves per SIMD of the 16-bit variants with head sizes below 128
+#endif
+#ifndef VTKV_ATTN_SMALL_FP8_WAVES
+#define VTKV_ATTN_SMALL_FP8_WAVES 3  // likewise with fp8 rows
 #endif
 constexpr int kStagesBf16 = VTKV_ATTN_STAGES;  // register tiles per wave (prefetch distance kStages-1)
 constexpr int kMaxSeqs = 1024;     // sequences per call (prefix sums of tile counts live in LDS)
@@ -105,6 +117,7 @@ struct AttnParams {
   uint32_t *seg_count;
   int fused_merge;
   int heads_per_seg;  // kv heads that share a segment of the tile order: 1, or 2 for the PAIR variants
+  int reduce_sets;    // workgroups of the merge kernel that share the heads of a (kv head, sequence)
   void *out;           // [B,Hq,D] bf16, or fp32 when out_f32
   int out_f32;
   int64_t q_stride;
@@ -174,13 +187,30 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 //
 // SPLIT: some kv head has more than 16 query heads and is served in parts (see first_head_of); the variants
 // without it index heads as kv head * group and carry none of that arithmetic.
-template <bool ALIBI, bool FP8, bool APPEND, int HPS, int D = 128, bool F16 = false, bool SPLIT = false>
+//
+// GW > 1 (kv heads per wave tile): GW adjacent kv heads whose query heads fit the 16 MFMA columns together are
+// one kv head to everything outside the tile loop (the host hands over num_kv_heads / GW heads of group * GW
+// query heads): column n belongs to sub-head n / (group / GW).  A wave's tile is 16 tokens of all GW sub-heads,
+// GW * D * e contiguous bytes per token, a whole number of 128-byte lines, and it is loaded line by line: one
+// load instruction takes one line of eight tokens, so that every line is asked for once.  A head row of 160,
+// 192 or 224 bytes asked for by itself occupies two or three line requests of the CU's limited number in
+// flight for 1.25 to 1.75 lines of data (head size 80: 0.62 of the peak, what 160 / 256 of the streaming rate
+// gives).  The sub-heads then pass through the wave's K and V tiles one after the other: the lanes that hold
+// pieces of a sub-head store them, all 16 columns get logits against its K rows, and the columns of other
+// sub-heads are given weight zero before P.V, which adds nothing to their accumulators.  Per byte this is the
+// arithmetic of the one-head tiles (whose unused columns compute throw-away values just the same).
+template <bool ALIBI, bool FP8, bool APPEND, int HPS, int D = 128, bool F16 = false, bool SPLIT = false, int GW = 1>
 __global__ void __launch_bounds__(kThreads)
-    __attribute__((amdgpu_waves_per_eu(D > 128 ? 1 : (FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES))))
+    __attribute__((amdgpu_waves_per_eu(D > 128   ? 1
+                                       : GW > 1  ? (FP8 && D <= 64 ? 3 : 2)  // (a tile of several kv heads is held in registers)
+                                       : D < 128 ? (FP8 ? VTKV_ATTN_SMALL_FP8_WAVES : VTKV_ATTN_SMALL_WAVES)
+                                                 : (FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES))))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
   static_assert(D % 16 == 0 && D >= 64 && D <= 256, "head sizes are multiples of 16 from 64 to 256");
   static_assert(!APPEND || D == 128, "the fused append is built for head size 128 only");
   static_assert(!SPLIT || HPS == 1, "a segment of several kv heads is never one of split kv heads");
+  static_assert(GW == 1 || (HPS == 1 && !APPEND && !SPLIT), "sub-heads per wave tile: plain attention, one segment per kv head group");
+  static_assert(GW == 1 || (GW * (FP8 ? D : 2 * D)) % 128 == 0, "the sub-heads of a token must fill whole cache lines");
   constexpr int kHD = FP8 ? (D + 63) / 64 * 64 : (D + 31) / 32 * 32;  // head size as held in LDS and registers
   constexpr int kKSteps = kHD / 32;                                  // MFMA steps of S^T = K.Q^T
   constexpr int kDBlocks = kHD / 16;                                 // 16-row blocks of O^T
@@ -223,6 +253,9 @@ __global__ void __launch_bounds__(kThreads)
     return APPEND ? (len - 1 + kTile - 1) / kTile + 1 : (len + kTile - 1) / kTile;
   };
 
+#ifdef VTKV_ATTN_TRACE
+  const unsigned long long trace_t0 = wall_clock64();
+#endif
   if (threadIdx.x == 0) s_npend = 0;
   // ---- exclusive prefix sums of the per-sequence tile counts (every workgroup computes its own copy)
   {
@@ -318,10 +351,12 @@ __global__ void __launch_bounds__(kThreads)
   constexpr int kKvRowBytes = FP8 ? D : 2 * D;       // bytes of one head row in global memory
   constexpr int kPieces = kKvRowBytes / 16;          // 16-byte pieces of a head row
   constexpr int kTilePieces = kTile * kPieces;       // ... of a 16-row tile, dealt to the lanes in order:
-  constexpr int kLoads = (kTilePieces + 63) / 64;    // load j of lane l takes piece 64 j + l, i.e. row (64 j + l) / kPieces
-  constexpr bool kEvenLoads = kTilePieces % 64 == 0; // every load of every lane carries a piece of the tile
+  // GW > 1: load j takes line j / 2 of tokens 8 (j % 2) .. + 8 of the tile, lane l the piece l % 8 of token l / 8
+  constexpr int kLines = GW * kKvRowBytes / 128;     // (GW > 1) cache lines of a token's sub-heads
+  constexpr int kLoads = GW > 1 ? 2 * kLines : (kTilePieces + 63) / 64;  // GW == 1: load j of lane l takes piece 64 j + l, i.e. row (64 j + l) / kPieces
+  constexpr bool kEvenLoads = GW > 1 || kTilePieces % 64 == 0;  // every load of every lane carries a piece of the tile
   constexpr int kKa = FP8 ? kHD / 64 : kKSteps;      // 16-byte A-operand pieces a lane reads back per K tile
-  const uint32_t row_stride = (uint32_t)(SPLIT ? Hkv / p.kv_split : Hkv) * kKvRowBytes;  // bytes between consecutive tokens
+  const uint32_t row_stride = (uint32_t)(SPLIT ? Hkv / p.kv_split : Hkv) * (kKvRowBytes * GW);  // bytes between consecutive tokens
   char *v_tile = smem + wave * kTileBytes;
   char *k_tile = smem + kWaves * kTileBytes + 1024 + wave * kTileBytes;
   // tile layouts in LDS (see vtkv_attn_common.h for the swizzles), with this head size's row pitch
@@ -330,8 +365,9 @@ __global__ void __launch_bounds__(kThreads)
     return FP8 ? row * kPitch8 + ((piece16 ^ ((row >> 1) & 7)) << 4) : row * kPitch + ((piece16 ^ (row & 15)) << 4);
   };
   // where this lane's j-th load of a tile goes: (row, piece) of the tile, or nothing
-  auto load_row = [&](int j) { return (64 * j + lane) / kPieces; };
-  auto load_piece = [&](int j) { return (64 * j + lane) % kPieces; };
+  auto load_row = [&](int j) { return GW > 1 ? 8 * (j & 1) + (lane >> 3) : (64 * j + lane) / kPieces; };
+  // (GW > 1: the piece's place in the token's region of GW head rows; sub-head and piece inside it follow from it)
+  auto load_piece = [&](int j) { return GW > 1 ? 8 * (j >> 1) + (lane & 7) : (64 * j + lane) % kPieces; };
   auto load_live = [&](int j) { return kEvenLoads || 64 * j + lane < kTilePieces; };
   if constexpr ((FP8 ? kHD / 16 : kHD / 8) != kPieces) {
     // padded head size: the pad pieces of both tiles are cleared once; no load ever writes them
@@ -365,8 +401,8 @@ __global__ void __launch_bounds__(kThreads)
       head0 = kv_real * p.group_real + part * G;
       n_heads = min(G, p.group_real - part * G);
     }
-    gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kv_real * kKvRowBytes;
-    gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kv_real * kKvRowBytes;
+    gptr k_base = (gptr)(uintptr_t)p.k_ptrs[slot] + kv_real * (kKvRowBytes * GW);
+    gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kv_real * (kKvRowBytes * GW);
     gptr nk_base = k_base, nv_base = v_base;
     if (APPEND) {
       nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kv_real * (2 * D);
@@ -389,6 +425,7 @@ __global__ void __launch_bounds__(kThreads)
         qop[ks] = raw;
       }
     }
+    const int my_sub = GW > 1 ? n / (G / GW) : 0;  // sub-head of this lane's column
     float slope_log2 = 0.f;
     if (ALIBI) slope_log2 = (n < n_heads && p.alibi_slopes) ? p.alibi_slopes[head0 + n] * kLog2e : 0.f;
 
@@ -408,7 +445,9 @@ __global__ void __launch_bounds__(kThreads)
     // per-lane byte offsets inside a K or V tile: load j of a lane takes row 4j+g, piece n, i.e. four
     // whole rows per load (fp8 rows are 128 bytes: a load then covers eight rows, lane l takes row
     // 8j + l/8, piece l%8).
-    uint32_t t_off[kLoads], t_off_last[kLoads];
+    // (GW > 1: two offsets, one per half of the tile's tokens; load j adds its line, 128 (j / 2), as a constant)
+    constexpr int kOffs = GW > 1 ? 2 : kLoads;
+    uint32_t t_off[kOffs], t_off_last[kOffs];
     // The new row's tile.  bf16 cache: every row slot holds the one new row, lane (g, n) its piece n.
     // fp8 cache: the new row arrives as bf16 and is quantised in consume(): a lane's two loads fetch the
     // two bf16 pieces that become its 16 codes, pieces 2*(lane%8) and 2*(lane%8)+1 of the 256-byte row.
@@ -416,18 +455,24 @@ __global__ void __launch_bounds__(kThreads)
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) t_off_new[j] = FP8 ? ((lane & 7) * 2 + j) * 16 : n * 16;
 #pragma unroll
-    for (int j = 0; j < kLoads; ++j) {
+    for (int j = 0; j < kOffs; ++j) {
       // (lanes past the end of the tile, where the head size leaves some, fetch its last row's first piece)
       const int row = load_live(j) ? load_row(j) : kTile - 1;
       const int col = load_live(j) ? load_piece(j) * 16 : 0;
       t_off[j] = (uint32_t)row * row_stride + col;
       t_off_last[j] = (uint32_t)min(row, valid_last - 1) * row_stride + col;
     }
+    auto off_of = [&](int j, bool last) {
+      if constexpr (GW > 1) return (last ? t_off_last[j & 1] : t_off[j & 1]) + (uint32_t)(j >> 1) * 128u;
+      else return last ? t_off_last[j] : t_off[j];
+    };
 
     // Loads of the i-th tile of this wave.  Always issued, never predicated, so the wait counters the
     // compiler derives are exact; past the wave's last tile every lane loads the segment's first 16
     // bytes instead (one cache line per load, not consumed).
-    auto load_tile = [&](gptr base, gptr new_base, int i, u32x4 *regs) {
+    // `want(j)` (compile-time after unrolling) picks the loads to issue now: all of them, or with GW > 1 those of
+    // the lines whose last sub-head has just gone to LDS, so that a tile's loads are spread over the previous one
+    auto load_tile = [&](gptr base, gptr new_base, int i, u32x4 *regs, auto want) {
       const bool live = i < my_tiles;
       const int tile = ws + kWph * i;
       const bool last = tile == n_tiles - 1;
@@ -440,13 +485,28 @@ __global__ void __launch_bounds__(kThreads)
       if (APPEND) src = (gptr)((uintptr_t)base + (((uintptr_t)new_base - (uintptr_t)base) & (uintptr_t)(int64_t)(int32_t)mask_new));  // base or new_base
 #pragma unroll
       for (int j = 0; j < kLoads; ++j) {
-        uint32_t off = (last ? t_off_last[j] : t_off[j]) & mask;
-        if (APPEND) off |= t_off_new[j] & mask_new;
-        regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off));
+        if (!want(j)) continue;
+        if constexpr (GW > 1) {
+          // (the line's constant stays outside the mask: past the wave's last tile load j reads line j / 2 of the
+          // segment's first token, which is mapped)
+          const uint32_t off = (last ? t_off_last[j & 1] : t_off[j & 1]) & mask;
+          regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off + (j >> 1) * 128));
+        } else {
+          uint32_t off = off_of(j, last) & mask;
+          if (APPEND) off |= t_off_new[j] & mask_new;
+          // A head row that is no whole number of lines shares its first and last line with its neighbours,
+          // which other waves of the workgroup ask for at about the same time: plain loads find them in L2
+          // (HBM reads of head size 80: 1.27 x the rows with the streaming hint, 1.02 x without).
+          if constexpr (kKvRowBytes % 128 != 0)
+            regs[j] = *(gvec)(src + row0 + off);
+          else
+            regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off));
+        }
       }
     };
-    auto load_k = [&](int i, u32x4 *kr) { load_tile(k_base, nk_base, i, kr); };
-    auto load_v = [&](int i, u32x4 *vr) { load_tile(v_base, nv_base, i, vr); };
+    auto every = [](int) { return true; };
+    auto load_k = [&](int i, u32x4 *kr) { load_tile(k_base, nk_base, i, kr, every); };
+    auto load_v = [&](int i, u32x4 *vr) { load_tile(v_base, nv_base, i, vr, every); };
 
     // one 16-row tile: logits, online softmax update, P.V
     auto consume = [&](int i, u32x4 *kreg, u32x4 *vreg) {
@@ -491,6 +551,20 @@ __global__ void __launch_bounds__(kThreads)
         *(gvec_rw)((uintptr_t)k_base + dst) = kreg[0];
         *(gvec_rw)((uintptr_t)v_base + dst) = vreg[0];
       }
+      // GW > 1: the tile's sub-heads one after the other through the same K and V tiles (once for GW == 1).
+      // Load j of a lane holds a piece of sub-head hh iff its place in the token's region lies in that head's
+      // pieces; which loads can hold any is known at compile time (line j / 2 against the head's byte range).
+#pragma unroll
+      for (int hh = 0; hh < GW; ++hh) {
+      auto sub_live = [&](int j) {
+        if constexpr (GW == 1) return load_live(j);
+        else return load_piece(j) >= hh * kPieces && load_piece(j) < (hh + 1) * kPieces;
+      };
+      auto sub_line = [&](int j) {  // compile-time part of sub_live
+        return GW == 1 || (8 * (j >> 1) < (hh + 1) * kPieces && 8 * (j >> 1) + 8 > hh * kPieces);
+      };
+      auto sub_piece = [&](int j) { return GW == 1 ? load_piece(j) : load_piece(j) - hh * kPieces; };
+      const bool mine = GW == 1 || my_sub == hh;  // this lane's column belongs to the sub-head
       // S^T[row, head] = sum_d K[row, d] q[head, d]
       f32x4 s = {0.f, 0.f, 0.f, 0.f};
       // K tile through LDS: in as loaded, out as A operand (lane (n, g): row n, bytes [16g, +16) of
@@ -498,12 +572,14 @@ __global__ void __launch_bounds__(kThreads)
       u32x4 ka[kKa];
 #pragma unroll
       for (int j = 0; j < kLoads; ++j)
-        if (load_live(j)) *reinterpret_cast<u32x4 *>(k_tile + k_off(load_row(j), load_piece(j))) = kreg[j];
+        if (sub_line(j) && sub_live(j)) *reinterpret_cast<u32x4 *>(k_tile + k_off(load_row(j), sub_piece(j))) = kreg[j];
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 #pragma unroll
       for (int c = 0; c < kKa; ++c) ka[c] = *reinterpret_cast<const u32x4 *>(k_tile + k_off(n, 4 * c + g));
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      if (kStages == 1) load_k(i + 1, kreg);  // the K registers are free again: refill them
+      // the K registers are free again: refill them (GW > 1: those of the lines that end in this sub-head)
+      auto done_with = [&](int j) { return GW == 1 || min(GW - 1, (8 * (j >> 1) + 7) / kPieces) == hh; };
+      if (kStages == 1) load_tile(k_base, nk_base, i + 1, kreg, done_with);
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
         const u32x4 kop =
@@ -515,17 +591,17 @@ __global__ void __launch_bounds__(kThreads)
       if constexpr (FP8) {
 #pragma unroll
         for (int j = 0; j < kLoads; ++j) {
-          if (!load_live(j)) continue;
-          const int row = load_row(j), piece = 2 * load_piece(j);
+          if (!sub_line(j) || !sub_live(j)) continue;
+          const int row = load_row(j), piece = 2 * sub_piece(j);
           *reinterpret_cast<u32x4 *>(v_tile + v_off(row, piece)) = fp8x8_widen<F16>(vreg[j][0], vreg[j][1]);
           *reinterpret_cast<u32x4 *>(v_tile + v_off(row, piece + 1)) = fp8x8_widen<F16>(vreg[j][2], vreg[j][3]);
         }
       } else {
 #pragma unroll
         for (int j = 0; j < kLoads; ++j)
-          if (load_live(j)) *reinterpret_cast<u32x4 *>(v_tile + v_off(load_row(j), load_piece(j))) = vreg[j];
+          if (sub_line(j) && sub_live(j)) *reinterpret_cast<u32x4 *>(v_tile + v_off(load_row(j), sub_piece(j))) = vreg[j];
       }
-      if (kStages == 1) load_v(i + 1, vreg);  // likewise the V registers once they are in LDS
+      if (kStages == 1) load_tile(v_base, nv_base, i + 1, vreg, done_with);  // likewise the V registers once they are in LDS
 
       // logits in log2 units; lane owns rows t0 + 4*g + r of head n
       float x[4];
@@ -540,12 +616,18 @@ __global__ void __launch_bounds__(kThreads)
           if (4 * g + r >= valid) x[r] = -INFINITY;
       }
       const float tmax = max_over_row_groups(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])));
-      const float m_new = fmaxf(m_run, tmax);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
+      // (a column of another sub-head: maximum and accumulators stay as they are, its weights are zero; the selects
+      // also discard whatever the arithmetic makes of a maximum that is still -inf)
+      const float m_new = mine ? fmaxf(m_run, tmax) : m_run;
+      const float alpha_raw = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first tile (m_run = -inf)
+      const float alpha = mine ? alpha_raw : 1.f;
       m_run = m_new;
       float pr[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+      for (int r = 0; r < 4; ++r) {
+        const float e = __builtin_amdgcn_exp2f(x[r] - m_new);
+        pr[r] = mine ? e : 0.f;
+      }
       l_run = l_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
@@ -598,6 +680,7 @@ __global__ void __launch_bounds__(kThreads)
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }  // sub-heads
     };
 
     // A ring of kStages register tiles per wave: while one tile is consumed the loads of the wave's next
@@ -769,6 +852,17 @@ __global__ void __launch_bounds__(kThreads)
     }
   }
 
+#ifdef VTKV_ATTN_TRACE
+  if (threadIdx.x == 0 && blockIdx.x < 4096) {
+    unsigned xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    g_attn_trace[blockIdx.x][0] = xcc & 0xf;
+    g_attn_trace[blockIdx.x][1] = trace_t0;
+    g_attn_trace[blockIdx.x][2] = (unsigned long long)wg;
+    g_attn_trace[blockIdx.x][3] = wall_clock64();
+    g_attn_trace[blockIdx.x][4] = (unsigned long long)(g_end - wg * span);
+  }
+#endif
   // ---- arrivals and merges of the shared segments (the rule of decode_attn_reduce_kernel below).
   // Pieces come from other CUs and other L2s: they were written with device-coherent stores, every wave
   // waits until its stores have completed before the arrivals are counted, and the pieces are read with
@@ -863,7 +957,9 @@ template <int GROUPS, int HSETS, int HD = 128, bool SPLIT = false>
 __global__ void __launch_bounds__(HD * GROUPS * HSETS) decode_attn_reduce_kernel(AttnParams p) {
   static_assert(GROUPS == 1 || HSETS == 1, "head sets only without piece groups");
   constexpr int kD = HD;  // (shadows the library-wide 128 inside this kernel)
-  const int kvh = blockIdx.x, b = blockIdx.y, d = threadIdx.x % kD;
+  // (groups above 8: the heads of a kv head are dealt to p.reduce_sets workgroups, four heads at a time in turn)
+  const int sets = p.reduce_sets, kvh = blockIdx.x / sets, bset = blockIdx.x % sets;
+  const int b = blockIdx.y, d = threadIdx.x % kD;
   const int grp = GROUPS > 1 ? threadIdx.x / kD : 0, hset = HSETS > 1 ? threadIdx.x / kD : 0;
   __shared__ float sm_red[GROUPS > 1 ? 3 * GROUPS * 4 * kD : 1];
   const int G = p.group, Hkv = p.num_kv_heads;
@@ -880,7 +976,8 @@ __global__ void __launch_bounds__(HD * GROUPS * HSETS) decode_attn_reduce_kernel
     w1 = w0 + (nt + span - 1) / span - 1;
   }
   const int64_t seg = p.head_major ? ((int64_t)(kvh / hps) * p.num_seqs + b) * hps + kvh % hps : (int64_t)b * Hkv + kvh;
-  for (int h0 = 4 * hset; h0 < G; h0 += 4 * HSETS) {
+  bool first_pass = true;
+  for (int h0 = 4 * (hset + HSETS * bset); h0 < G; h0 += 4 * HSETS * sets) {
     float m[4], wsum[4], o[4];
 #pragma unroll
     for (int hh = 0; hh < 4; ++hh) m[hh] = -INFINITY, wsum[hh] = 0.f, o[hh] = 0.f;
@@ -915,7 +1012,8 @@ __global__ void __launch_bounds__(HD * GROUPS * HSETS) decode_attn_reduce_kernel
       }
     }
     if constexpr (GROUPS > 1) {
-      if (h0 > 0) __syncthreads();  // the previous heads' values have been read
+      if (!first_pass) __syncthreads();  // the previous heads' values have been read
+      first_pass = false;
 #pragma unroll
       for (int hh = 0; hh < 4; ++hh) {
         float *at = sm_red + ((grp * 4 + hh) * kD + d) * 3;
@@ -1011,10 +1109,11 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16 + 24 + 2 + 18 + 28;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
+constexpr int kVariants = 16 + 24 + 2 + 18 + 28 + 6;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
                                                   // others, the fused append for fp16 at head size 128 (fp16 rows,
                                                   // fp8 rows), 18 that stream several kv heads per segment at other
-                                                  // shapes, 28 for kv heads of more than 16 query heads (SPLIT)
+                                                  // shapes, 28 for kv heads of more than 16 query heads (SPLIT), 6
+                                                  // whose wave tiles hold several kv heads (GW)
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
 int head_size_index(int head_size) {
@@ -1118,7 +1217,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   // what the kernels see; kv_heads_real is what the rows in memory hold.
   const int kv_heads_real = num_kv_heads, group_real = num_heads / num_kv_heads;
   const int kv_split = vtkv_kv_split(group_real);
-  const int group = (group_real + kv_split - 1) / kv_split;
+  int group = (group_real + kv_split - 1) / kv_split;
   num_kv_heads = kv_heads_real * kv_split;
   VTKV_REQUIRE(num_kv_heads <= kMaxKvHeads, "%d kv heads (as %d of at most 16 query heads each) exceed %d", kv_heads_real,
                num_kv_heads, kMaxKvHeads);
@@ -1171,6 +1270,23 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
       variant = head_size == 128 ? 58 + (append ? 1 : 0) : 42 + d_index * 4 + (f16 ? 2 : 0) + (fp8 ? 1 : 0);
     }
   }
+  // Several kv heads per wave tile (GW, see the kernel) for 16-bit rows of head sizes 64 (2 kv heads: 256 bytes per
+  // token), 80 (4: 640 bytes) and 96 (2: 384 bytes), where the heads that make whole lines have room in the 16
+  // columns together.  To everything below, the GW heads are one kv head of group * GW query heads.  64 sequences
+  // of 512..4096 rows, 8 kv heads of 4 query heads, stream kernel, share of the HBM peak, against one wave per head
+  // with plain loads: 80: 0.675 against 0.62, 96: 0.766 against 0.67, 64: 0.73 either way.  Measured and left out:
+  // 112 with 4 heads per tile (28 registers of 16 bytes to hold a tile: spills, 0.57 against 0.66), fp8 rows of 64
+  // and 96 with 4 (0.48 and 0.49 against 0.56 and 0.61).
+  if (!tuned && !fp8 && kv_split == 1 && !append && d_index < 3) {
+    static const int kGw16[3] = {2, 4, 2};
+    const int gw = kGw16[d_index];
+    if (num_kv_heads % gw == 0 && group * gw <= 16) {
+      seg_heads = 1;
+      variant = 88 + d_index * 2 + (f16 ? 1 : 0);
+      num_kv_heads /= gw;
+      group *= gw;
+    }
+  }
   // kv heads of more than 16 query heads: one variant per (head size, type, cache type), the fused append at 128
   if (kv_split > 1)
     variant = append ? 84 + (f16 ? 2 : 0) + (fp8 ? 1 : 0) : 60 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
@@ -1196,6 +1312,10 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
       VTKV_SPLIT(64, false), VTKV_SPLIT(80, false), VTKV_SPLIT(96, false), VTKV_SPLIT(112, false), VTKV_SPLIT(128, false),
       VTKV_SPLIT(256, false), VTKV_SPLIT(128, true),
 #undef VTKV_SPLIT
+#define VTKV_GW(DD, F8, W)                                                                                     \
+  decode_attn_stream_kernel<true, F8, false, 1, DD, false, false, W>, decode_attn_stream_kernel<true, F8, false, 1, DD, true, false, W>
+      VTKV_GW(64, false, 2), VTKV_GW(80, false, 4), VTKV_GW(96, false, 2),
+#undef VTKV_GW
   };
 #undef VTKV_ROW
 #undef VTKV_SIZE
@@ -1262,6 +1382,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   const bool hm_auto = knob_hm != 0 && hm_fits;  // the head-major order is open to this call
   p.fused_merge = !v2 && (knob_merge == 1 || (knob_merge < 0 && (hm_auto ? segs >= 2 * grid : 2 * segs >= 5 * grid)));
   p.heads_per_seg = seg_heads;
+  p.reduce_sets = 1;
   p.cum_tiles = (int32_t *)((char *)workspace + count_bytes);
   p.part_out = (float *)((char *)workspace + count_bytes + cum_bytes);
   p.part_max = p.part_out + n_stat * hd;
@@ -1330,7 +1451,10 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   }
   if (!p.fused_merge) {
     // segments of at least four pieces on average: four sets of threads share a segment's pieces
-    const dim3 rgrid(num_kv_heads, num_seqs);
+    // (several workgroups per (kv head, sequence) where its heads would take more than one pass: four heads per pass
+    // when the pieces of a segment are shared out over four sets of threads, else eight)
+    p.reduce_sets = 4 * segs <= grid ? (group + 3) / 4 : (group + 7) / 8;
+    const dim3 rgrid(num_kv_heads * p.reduce_sets, num_seqs);
 #define VTKV_REDUCE_LAUNCH_(G, S, HD, SP)                                                                     \
   do {                                                                                                        \
     if (timed)                                                                                                \
@@ -1494,6 +1618,13 @@ int vtkv_decode_append_attention(void *out, const void *q, const void *key, cons
                         v_scale, workspace, workspace_bytes, partition_tokens, stream, key, value, key_stride,
                         value_stride);
 }
+
+#ifdef VTKV_ATTN_TRACE
+__attribute__((visibility("default"))) int vtkv_debug_attn_trace(unsigned long long *out, int n) {
+  VTKV_HIP(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_attn_trace), (size_t)n * 6 * sizeof(unsigned long long)));
+  return VTKV_OK;
+}
+#endif
 
 int vtkv_set_head_major(int on) {
   g_head_major.store(on < 0 ? -1 : (on != 0), std::memory_order_relaxed);
