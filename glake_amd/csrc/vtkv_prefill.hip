@@ -178,12 +178,18 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   const int wave_first_limit = u_pos0 + tok_lo + 1;
 
   f32x4 acc[kNB][kDB];
-  float m_run[kNB], l_run[kNB];
+  // The normaliser of a column is one more row of its output: P^T times a column of ones, accumulated by the matrix
+  // pipe like the others (every lane of the column ends up with the whole sum in each of its four slots), instead
+  // of a chain of vector additions per stage.  m_off: what the exponent's fused multiply-add subtracts, kept with
+  // the reference point it follows.
+  f32x4 acc_l[kNB];
+  float m_run[kNB], m_off[kNB];
   auto reset = [&]() {
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
       m_run[nb] = -INFINITY;
-      l_run[nb] = 0.f;
+      m_off[nb] = 0.f;
+      acc_l[nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < kDB; ++i) acc[nb][i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
@@ -349,27 +355,30 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
             for (int r = 0; r < 4; ++r)
               if (t0 + 16 * t + 4 * g + r >= limit[nb]) x[4 * t + r] = -INFINITY;
         }
-        const float tmax = wave_max_over_row_groups(fmax2(fmax3(x[0], x[1], x[2]), fmax3(fmax3(x[3], x[4], x[5]), x[6], x[7])));
-        const bool grow = tmax > m_run[nb] + lazy;
-        if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // rare: some column of the block moves its reference point
+        // the lane's own maximum; the maximum of the column (its four row groups) is only needed when some lane
+        // sees a value above the reference point's margin, which is exactly when the column's maximum is above it
+        const float lmax = fmax2(fmax3(x[0], x[1], x[2]), fmax3(fmax3(x[3], x[4], x[5]), x[6], x[7]));
+        if (__builtin_amdgcn_ballot_w64(lmax > m_run[nb] + lazy) != 0) {  // rare: some column moves its reference point
+          const float tmax = wave_max_over_row_groups(lmax);
+          const bool grow = tmax > m_run[nb] + lazy;
           const float m_new = grow ? tmax : m_run[nb];
           // (a column that has seen only masked rows keeps -inf and rescales its zeros by 1)
           const float alpha = grow ? __builtin_amdgcn_exp2f(ALIBI ? m_run[nb] - m_new : (m_run[nb] - m_new) * sl) : 1.f;
           m_run[nb] = m_new;
-          l_run[nb] *= alpha;
+          // (a column can have everything so far masked; the reference point 0 keeps exp2(-inf - ref) = 0)
+          const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+          m_off[nb] = ALIBI ? -m_ref : -m_ref * sl;
+          acc_l[nb] *= alpha;
 #pragma unroll
           for (int d = 0; d < kDB; ++d) acc[nb][d] *= alpha;
         }
-        // (a column can have everything so far masked; the reference point 0 keeps exp2(-inf - ref) = 0)
-        const float m_ref = m_run[nb] == -INFINITY ? 0.f : m_run[nb];
         float pr[8];
         if (ALIBI) {
 #pragma unroll
-          for (int r = 0; r < 8; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_ref);
+          for (int r = 0; r < 8; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] + m_off[nb]);
         } else {
-          const float mr = -m_ref * sl;
 #pragma unroll
-          for (int r = 0; r < 8; ++r) pr[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], sl, mr));
+          for (int r = 0; r < 8; ++r) pr[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], sl, m_off[nb]));
         }
         // P^T as fp16 (11 significant bits: the rounding stays below 2^-12 relative, which a bf16 P would
         // miss by a factor 16); the normaliser sums the same rounded weights
@@ -381,10 +390,11 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
             pt[r] = pack_bf16x2(pr[2 * r] - __builtin_bit_cast(float, ph[r] << 16),
                                 pr[2 * r + 1] - __builtin_bit_cast(float, ph[r] & 0xffff0000u));
           }
-          float l = l_run[nb];
-#pragma unroll
-          for (int r = 0; r < 8; ++r) l += pr[r];
-          l_run[nb] = l;
+          {  // the normaliser: head and tail of the weights against ones (1.0 in bf16)
+            const bf16x8 ones = __builtin_bit_cast(bf16x8, (u32x4){0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
+            acc_l[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(bf16x8, ph), acc_l[nb], 0, 0, 0);
+            acc_l[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(bf16x8, pt), acc_l[nb], 0, 0, 0);
+          }
 #pragma unroll
           for (int db = 0; db < kDB; ++db) {
             acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vop[db]),
@@ -396,11 +406,11 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
           u32x4 pb;
 #pragma unroll
           for (int r = 0; r < 4; ++r) pb[r] = pack_f16x2(pr[2 * r], pr[2 * r + 1]);
-          float l = l_run[nb];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) l = add_f16x2(pb[r], l);
-          l_run[nb] = l;
           const f16x8 pop = __builtin_bit_cast(f16x8, pb);
+          {  // the normaliser sums the same rounded weights (1.0 in fp16)
+            const f16x8 ones = __builtin_bit_cast(f16x8, (u32x4){0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u});
+            acc_l[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pop, acc_l[nb], 0, 0, 0);
+          }
 #pragma unroll
           for (int db = 0; db < kDB; ++db)
             acc[nb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, vop[db]), pop, acc[nb][db], 0,
@@ -454,7 +464,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   // ---- normalise and store: lane (n, g) holds O[column n][d = 16*db + 4g + i]
 #pragma unroll
   for (int nb = 0; nb < kNB; ++nb) {
-    const float l = sum_over_row_groups(l_run[nb]);
+    const float l = acc_l[nb][0];  // (already the sum over all rows: see acc_l)
     if (col_tok[nb] < 0) continue;
     const float inv = p.v_scale / l;
     const int64_t o0 = ((int64_t)(u_row0 + col_tok[nb]) * p.num_heads + head0 + col_head[nb]) * kD + 4 * g;
