@@ -73,11 +73,6 @@ __device__ __forceinline__ unsigned pack_f16x2(float a, float b) {
   f16x2 v = {(_Float16)a, (_Float16)b};
   return __builtin_bit_cast(unsigned, v);
 }
-// l + the two fp16 halves of w, in fp32.
-__device__ __forceinline__ float add_f16x2(unsigned w, float l) {
-  const f16x2 ones = {(_Float16)1.f, (_Float16)1.f};
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), ones, l, false);
-}
 // Maxima as single instructions.  fmaxf() first quiets its operands (one more instruction each) wherever the
 // compiler cannot prove them canonical, which it cannot after selects and lane swaps.
 __device__ __forceinline__ float fmax2(float a, float b) {
@@ -311,6 +306,10 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
       // all S MFMAs first, then per column block its softmax followed by its P.V MFMAs, so that the matrix
       // pipe works on one block's P.V while the vector unit does the next block's softmax
       f32x4 sacc[kNB][2];
+      // The S MFMAs of a stage head a chain everything else of the stage hangs on: they are issued at raised
+      // priority, ahead of the other wave of the SIMD, which is mostly in its softmax (2 to 3 % per launch; the
+      // other way round, softmax and P.V raised, changes nothing).
+      __builtin_amdgcn_s_setprio(3);
 #pragma unroll
       for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
@@ -323,6 +322,7 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
       // reduction slot (g, j) of the K=32 P.V MFMA stands for row 4g+j of the first tile (j < 4) and row
       // 4g+j-4 of the second (j >= 4), so a lane's A operand is its transposed quad of the first tile
       // followed by that of the second; read once for both column blocks
+      __builtin_amdgcn_s_setprio(0);
       u32x4 vop[kDB];
 #pragma unroll
       for (int db = 0; db < kDB; ++db) {
