@@ -639,15 +639,25 @@ def growth_and_swap_protocol(args) -> dict:
     blocks, events = [], []
     bit_exact, checked = True, 0
     step_bytes = step_time = 0.0
+    debug_timing = os.environ.get("VTKV_BENCH_BLOCK_KERNEL_TIMES") == "1"   # (events on every launch: slows the steps)
+    kernel_us = []
     for blk in range(steps // every):
         torch.cuda.synchronize()
+        if debug_timing:
+            _C.check(_C.lib().vtkv_set_kernel_timing(1))
         t0 = time.perf_counter()
         nbytes = 0
         for _ in range(every):
             plan.run(q, new_k, new_v, out)
             nbytes += int(plan.seq_lens.sum()) * 2 * row + 2 * B * Hq * D * 2 + B * 2 * row * 2
+        host_dt = time.perf_counter() - t0
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        if debug_timing:
+            _C.check(_C.lib().vtkv_set_kernel_timing(0))
+            ts, tr = (C.c_float * every)(), (C.c_float * every)()
+            _C.check(_C.lib().vtkv_attention_kernel_times(ts, tr, every))
+            kernel_us.append([round(x * 1e3, 1) for x in ts] + [round(host_dt * 1e6 / every, 1)])
         blocks.append(round(nbytes / dt / 1e9, 1))
         step_bytes += nbytes
         step_time += dt
@@ -694,6 +704,7 @@ def growth_and_swap_protocol(args) -> dict:
         "swap_out_gbps": med([e["out_gbps"] for e in events]), "swap_in_gbps": med([e["in_gbps"] for e in events]),
         "bit_exact": bool(bit_exact and appended_exact), "swapped_bytes_checked": int(checked),
         "appended_rows_checked": B * steps * 2,
+        **({"kernel_us_by_block_and_host_us_per_step": kernel_us} if debug_timing else {}),
     }
 
 def cpu_model() -> str:
