@@ -180,6 +180,8 @@ def main() -> int:
                          "256): the step then is reshape_and_cache + attention as two launches (the fused append is "
                          "built for 128)")
     ap.add_argument("--heads", default="", metavar="HQ,HKV", help="likewise with other head counts")
+    ap.add_argument("--chunk-mib", type=int, default=2,
+                    help="size of a physical chunk (the reference's granularity is 2 MiB; vtkv_pool_set_chunk_bytes)")
     ap.add_argument("--workgroup-trace", action="store_true",
                     help="with a library built by `python -m glake_amd.build --define VTKV_ATTN_TRACE --out X` "
                          "(VTKV_LIBRARY_PATH=X): when the workgroups of the decode kernel's last launch ended, by XCD")
@@ -202,6 +204,10 @@ def main() -> int:
         return prompt_run(args, cfg)
     from glake_amd import _C
 
+    if args.chunk_mib != 2:
+        from glake_amd import vmm_allocator as vmm
+
+        vmm.set_chunk_bytes(args.chunk_mib << 20)
     _C.check(_C.lib().vtkv_set_fused_merge({"auto": -1, "fused": 1, "separate": 0}[args.merge]))
     _C.check(_C.lib().vtkv_set_head_major({"auto": -1, "on": 1, "off": 0}[args.head_major]))
     R = args.repeats if args.repeats > 0 else (21 if args.steps <= 50 else 3)
@@ -252,7 +258,8 @@ def decode_run(args, config: str, R: int, with_swap: bool, with_cpu: bool) -> di
     kv_dtype = "fp8" if fp8 else "auto"
     row = Hkv * D * eb
     max_tokens = max(ctx0) + total_steps + 1
-    chunks_per_range = (max_tokens * row + args.value_skew + (2 << 20) - 1) // (2 << 20)
+    chunk = vmm.chunkBytes()
+    chunks_per_range = (max_tokens * row + args.value_skew + chunk - 1) // chunk
     ensure_pool(2 * L * B * chunks_per_range + 16)
     engine = CacheEngine(num_layers=L, num_kv_heads=Hkv, head_size=D, dtype=torch.uint8 if fp8 else torch.bfloat16,
                          max_num_seqs=B, max_num_batched_tokens=max_tokens,
@@ -348,7 +355,7 @@ def decode_run(args, config: str, R: int, with_swap: bool, with_cpu: bool) -> di
     mgr = ChunkSpaceManager(B, 2 * B * chunks_per_range + 16, watermark=0.0)
     claims = []
     for b in range(B):
-        c = SequenceChunks(row, value_skew=args.value_skew)
+        c = SequenceChunks(row, chunk_bytes=chunk, value_skew=args.value_skew)
         c.append_tokens(ctx0[b])
         assert mgr.allocate(c)
         claims.append(c)
@@ -504,7 +511,7 @@ def decode_run(args, config: str, R: int, with_swap: bool, with_cpu: bool) -> di
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 (fp8-e4m3 KV)" if fp8 else "bf16", "data": "synthetic",
-        "config": {"workload": cfg["name"], "layers": L, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
+        "config": {"workload": cfg["name"], "layers": L, "new_tokens_per_step": B, "kv_chunk": f"{chunk >> 20}MiB VMM",
                    "mean_ctx": round(float(np.mean(final_lens)), 1), "host_path": args.host_path,
                    "fused_append": (bool(plan.fused) and step is step_plan) or (backend_path and not args.unfused),
                    "value_skew_bytes": engine.value_skew},
