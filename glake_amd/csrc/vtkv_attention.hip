@@ -207,9 +207,9 @@ __global__ void __launch_bounds__(kThreads)
                                                  : (FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES))))
     decode_attn_stream_kernel(AttnParams p, InlineLens il) {
   static_assert(D % 16 == 0 && D >= 64 && D <= 256, "head sizes are multiples of 16 from 64 to 256");
-  static_assert(!APPEND || D == 128, "the fused append is built for head size 128 only");
+  static_assert(!APPEND || D == 128 || !FP8, "the fused append quantises new rows for head size 128 only");
   static_assert(!SPLIT || HPS == 1, "a segment of several kv heads is never one of split kv heads");
-  static_assert(GW == 1 || (HPS == 1 && !APPEND && !SPLIT), "sub-heads per wave tile: plain attention, one segment per kv head group");
+  static_assert(GW == 1 || (HPS == 1 && !SPLIT), "sub-heads per wave tile: one segment per kv head group");
   static_assert(GW == 1 || (GW * (FP8 ? D : 2 * D)) % 128 == 0, "the sub-heads of a token must fill whole cache lines");
   constexpr int kHD = FP8 ? (D + 63) / 64 * 64 : (D + 31) / 32 * 32;  // head size as held in LDS and registers
   constexpr int kKSteps = kHD / 32;                                  // MFMA steps of S^T = K.Q^T
@@ -405,8 +405,8 @@ __global__ void __launch_bounds__(kThreads)
     gptr v_base = (gptr)(uintptr_t)p.v_ptrs[slot] + kv_real * (kKvRowBytes * GW);
     gptr nk_base = k_base, nv_base = v_base;
     if (APPEND) {
-      nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kv_real * (2 * D);
-      nv_base = (gptr)(uintptr_t)p.new_v + (int64_t)b * p.new_v_stride + kv_real * (2 * D);
+      nk_base = (gptr)(uintptr_t)p.new_k + (int64_t)b * p.new_k_stride + kv_real * (2 * D * GW);
+      nv_base = (gptr)(uintptr_t)p.new_v + (int64_t)b * p.new_v_stride + kv_real * (2 * D * GW);
     }
 
     // B operand of S^T = K.Q^T: for MFMA step ks lane (n, g) holds the eight q[head n][d] whose K
@@ -448,12 +448,14 @@ __global__ void __launch_bounds__(kThreads)
     // (GW > 1: two offsets, one per half of the tile's tokens; load j adds its line, 128 (j / 2), as a constant)
     constexpr int kOffs = GW > 1 ? 2 : kLoads;
     uint32_t t_off[kOffs], t_off_last[kOffs];
-    // The new row's tile.  bf16 cache: every row slot holds the one new row, lane (g, n) its piece n.
+    // The new row's tile.  16-bit cache: every row slot holds the one new row, a lane's load j the piece it
+    // takes of any row (GW > 1: piece lane % 8 of line j / 2, the line added as a constant like above).
     // fp8 cache: the new row arrives as bf16 and is quantised in consume(): a lane's two loads fetch the
     // two bf16 pieces that become its 16 codes, pieces 2*(lane%8) and 2*(lane%8)+1 of the 256-byte row.
     uint32_t t_off_new[kLoads];
 #pragma unroll
-    for (int j = 0; j < kLoads; ++j) t_off_new[j] = FP8 ? ((lane & 7) * 2 + j) * 16 : n * 16;
+    for (int j = 0; j < kLoads; ++j)
+      t_off_new[j] = FP8 ? ((lane & 7) * 2 + j) * 16 : GW > 1 ? (lane & 7) * 16 : load_live(j) ? load_piece(j) * 16 : 0;
 #pragma unroll
     for (int j = 0; j < kOffs; ++j) {
       // (lanes past the end of the tile, where the head size leaves some, fetch its last row's first piece)
@@ -489,7 +491,8 @@ __global__ void __launch_bounds__(kThreads)
         if constexpr (GW > 1) {
           // (the line's constant stays outside the mask: past the wave's last tile load j reads line j / 2 of the
           // segment's first token, which is mapped)
-          const uint32_t off = (last ? t_off_last[j & 1] : t_off[j & 1]) & mask;
+          uint32_t off = (last ? t_off_last[j & 1] : t_off[j & 1]) & mask;
+          if (APPEND) off |= t_off_new[j] & mask_new;
           regs[j] = __builtin_nontemporal_load((gvec)(src + row0 + off + (j >> 1) * 128));
         } else {
           uint32_t off = off_of(j, last) & mask;
@@ -544,12 +547,23 @@ __global__ void __launch_bounds__(kThreads)
             *(gvec_rw)((uintptr_t)v_base + dst) = vreg[0];
           }
         }
-      } else if (APPEND && is_new && g == 0) {
-        // lanes 0..15 hold the sixteen 16-byte pieces of the new K and V rows: append them to the cache
+      } else if (APPEND && is_new) {
+        // the lanes that hold row 0 of the tile hold the 16-byte pieces of the new K and V rows: append them to
+        // the cache (one head row: lanes 0 .. kPieces - 1 of load 0; GW > 1: lanes 0..7 of each line's first load)
         typedef __attribute__((address_space(1))) u32x4 *gvec_rw;
-        const int64_t dst = (int64_t)(seq_len - 1) * row_stride + n * 16;
-        *(gvec_rw)((uintptr_t)k_base + dst) = kreg[0];
-        *(gvec_rw)((uintptr_t)v_base + dst) = vreg[0];
+        const int64_t dst = (int64_t)(seq_len - 1) * row_stride + lane * 16;
+        if constexpr (GW > 1) {
+          if (lane < 8) {
+#pragma unroll
+            for (int line = 0; line < kLines; ++line) {
+              *(gvec_rw)((uintptr_t)k_base + dst + line * 128) = kreg[2 * line];
+              *(gvec_rw)((uintptr_t)v_base + dst + line * 128) = vreg[2 * line];
+            }
+          }
+        } else if (lane < kPieces) {
+          *(gvec_rw)((uintptr_t)k_base + dst) = kreg[0];
+          *(gvec_rw)((uintptr_t)v_base + dst) = vreg[0];
+        }
       }
       // GW > 1: the tile's sub-heads one after the other through the same K and V tiles (once for GW == 1).
       // Load j of a lane holds a piece of sub-head hh iff its place in the token's region lies in that head's
@@ -1109,11 +1123,12 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16 + 24 + 2 + 18 + 28 + 6;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
-                                                  // others, the fused append for fp16 at head size 128 (fp16 rows,
-                                                  // fp8 rows), 18 that stream several kv heads per segment at other
-                                                  // shapes, 28 for kv heads of more than 16 query heads (SPLIT), 6
-                                                  // whose wave tiles hold several kv heads (GW)
+constexpr int kVariants = 16 + 24 + 2 + 18 + 28 + 6 + 18;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
+                                                       // others, the fused append for fp16 at head size 128 (fp16 rows,
+                                                       // fp8 rows), 18 that stream several kv heads per segment at other
+                                                       // shapes, 28 for kv heads of more than 16 query heads (SPLIT), 6
+                                                       // whose wave tiles hold several kv heads (GW), 18 with the fused
+                                                       // append for 16-bit rows of the other head sizes
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
 int head_size_index(int head_size) {
@@ -1231,7 +1246,8 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
                "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
   if (append) {
     VTKV_REQUIRE(new_value != nullptr, "null argument");
-    VTKV_REQUIRE(head_size == 128, "the fused append needs head size 128");
+    VTKV_REQUIRE(head_size == 128 || (kv_dtype == q_dtype && kv_split == 1),
+                 "the fused append at head sizes other than 128 needs 16-bit rows and at most 16 query heads per kv head");
     const int64_t row = (int64_t)kv_heads_real * head_size;
     VTKV_REQUIRE(key_stride >= row && value_stride >= row && key_stride % 8 == 0 && value_stride % 8 == 0 &&
                      (uintptr_t)new_key % 16 == 0 && (uintptr_t)new_value % 16 == 0,
@@ -1257,6 +1273,8 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   int variant = tuned    ? (fp8 ? 8 : 0) + (pair ? 4 : 0) + (append ? 2 : 0) + (alibi ? 1 : 0)
                 : append ? 40 + (fp8 ? 1 : 0)
                          : 16 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
+  const bool append_other = append && head_size != 128;  // (16-bit rows: checked above)
+  if (append_other) variant = 94 + (d_index < 4 ? d_index : 4) * 2 + (f16 ? 1 : 0);
   if (!tuned) {
     // A head row that is no whole number of 128-byte lines (160, 192, 224 bytes; 64 to 112 bytes of fp8 codes)
     // drags its neighbours' bytes along with every fetch, and a lone line streams slower than a pair (see the
@@ -1265,9 +1283,11 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
     // HBM peak with one head per segment: head size 80 0.51, 96 0.60, 112 0.53, 64 0.72; fp8 rows 0.29 to 0.40.
     static const int kHeads16[6] = {2, 4, 2, 4, 1, 1}, kHeads8[6] = {4, 4, 4, 4, 2, 1};
     const int want = fp8 ? kHeads8[d_index] : kHeads16[d_index];
-    if (want > 1 && kv_split == 1 && num_kv_heads % want == 0 && group * want <= 16) {
+    if (want > 1 && kv_split == 1 && num_kv_heads % want == 0 && group * want <= 16 && (!append_other || d_index == 3)) {
       seg_heads = want;
-      variant = head_size == 128 ? 58 + (append ? 1 : 0) : 42 + d_index * 4 + (f16 ? 2 : 0) + (fp8 ? 1 : 0);
+      variant = head_size == 128 ? 58 + (append ? 1 : 0)
+                : append_other   ? 110 + (f16 ? 1 : 0)
+                                 : 42 + d_index * 4 + (f16 ? 2 : 0) + (fp8 ? 1 : 0);
     }
   }
   // Several kv heads per wave tile (GW, see the kernel) for 16-bit rows of head sizes 64 (2 kv heads: 256 bytes per
@@ -1277,12 +1297,12 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   // with plain loads: 80: 0.675 against 0.62, 96: 0.766 against 0.67, 64: 0.73 either way.  Measured and left out:
   // 112 with 4 heads per tile (28 registers of 16 bytes to hold a tile: spills, 0.57 against 0.66), fp8 rows of 64
   // and 96 with 4 (0.48 and 0.49 against 0.56 and 0.61).
-  if (!tuned && !fp8 && kv_split == 1 && !append && d_index < 3) {
+  if (!tuned && !fp8 && kv_split == 1 && d_index < 3) {
     static const int kGw16[3] = {2, 4, 2};
     const int gw = kGw16[d_index];
     if (num_kv_heads % gw == 0 && group * gw <= 16) {
       seg_heads = 1;
-      variant = 88 + d_index * 2 + (f16 ? 1 : 0);
+      variant = (append ? 104 : 88) + d_index * 2 + (f16 ? 1 : 0);
       num_kv_heads /= gw;
       group *= gw;
     }
@@ -1316,6 +1336,11 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   decode_attn_stream_kernel<true, F8, false, 1, DD, false, false, W>, decode_attn_stream_kernel<true, F8, false, 1, DD, true, false, W>
       VTKV_GW(64, false, 2), VTKV_GW(80, false, 4), VTKV_GW(96, false, 2),
 #undef VTKV_GW
+#define VTKV_APPEND16(DD, H, W)                                                                                 \
+  decode_attn_stream_kernel<true, false, true, H, DD, false, false, W>, decode_attn_stream_kernel<true, false, true, H, DD, true, false, W>
+      VTKV_APPEND16(64, 1, 1), VTKV_APPEND16(80, 1, 1), VTKV_APPEND16(96, 1, 1), VTKV_APPEND16(112, 1, 1), VTKV_APPEND16(256, 1, 1),
+      VTKV_APPEND16(64, 1, 2), VTKV_APPEND16(80, 1, 4), VTKV_APPEND16(96, 1, 2), VTKV_APPEND16(112, 4, 1),
+#undef VTKV_APPEND16
   };
 #undef VTKV_ROW
 #undef VTKV_SIZE

@@ -174,7 +174,10 @@ class DecodeStepPlan:
         self._ws = torch.zeros(max(int(need), 1 << 20), dtype=torch.uint8, device=self.device)
         self._ws_p, self._ws_n = C.c_void_p(self._ws.data_ptr()), self._ws.numel()
         self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
-        self.fused = (bool(fused) and self.head_size == 128 and self._kv_dt in (self._src_dt, _C.FP8_E4M3))
+        # one launch per step: any cache type at head size 128; 16-bit caches at the other head sizes when a kv head
+        # has at most 16 query heads
+        self.fused = bool(fused) and (self.head_size == 128 or (
+            self._kv_dt == self._src_dt and self.num_heads // self.num_kv_heads <= 16))
         self._inline = self.fused and n <= 512
         self._host_lens_p = [C.c_void_p(self._stage[i].data_ptr() + 8 * n) for i in range(ring)]
 

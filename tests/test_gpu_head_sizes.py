@@ -243,51 +243,47 @@ def run_prompt_case(vmm, seed, query_lens, seq_lens, hq, hkv, d, dtype, fp8=Fals
     assert torch.equal(out16.cpu(), torch.from_numpy(got).to(tdt))
 
 
-@pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("lens_from", ["host", "device"])
-def test_fused_append_for_fp16_models(gpu_pool, fp8, lens_from):
-    """vtkv_decode_append_attention with fp16 queries and new rows (head size 128): the new row lands in the cache
-    as reshape_and_cache stores it (the fp16 bits, or the e4m3fn codes of value / scale), attention over all
-    rows against the oracle; lengths around tile and chunk boundaries, ALiBi, lengths from either side."""
+def run_append_case(vmm, seed, lens, hq, hkv, d, dtype, fp8=False, lens_from="host", alibi=True, partition_tokens=0):
+    """vtkv_decode_append_attention: `lens` count the new token.  The new row must land in the cache as
+    reshape_and_cache stores it (the 16-bit pattern, or the e4m3fn codes of value / scale) with nothing before it
+    disturbed, and attention over all rows must agree with the oracle."""
     import torch
 
     from glake_amd import _custom_ops as ops
 
-    rng = np.random.default_rng(90 + fp8)
-    hq, hkv, d = 32, 8, 128
+    rng = np.random.default_rng(seed)
     eb = 1 if fp8 else 2
     row = hkv * d * eb
-    per = (2 << 20) // row
-    lens = [1, 2, 16, 17, 18, 33, 257, per - 1, per, per + 1, 2500]      # they count the new token
     b = len(lens)
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
     k_scale, v_scale = (0.021, 0.033) if fp8 else (1.0, 1.0)
 
     def stored(x32, sc):  # (bits in the cache, the values they stand for)
         if fp8:
             codes = O.fp8_encode(x32, sc)
             return codes, O.fp8_decode(codes, sc)
-        return to_model(x32, "f16")
+        return to_model(x32, dtype)
 
-    gpu = GpuSeqs(gpu_pool, b, hkv, d, eb, max(lens) + 1, value_skew=256)
+    gpu = GpuSeqs(vmm, b, hkv, d, eb, max(lens) + 1, value_skew=256)
     k_bits, v_bits, k32, v32 = [], [], [], []
     for i, t in enumerate(lens):
         kb, kf = stored(rng.standard_normal((t - 1, hkv, d)).astype(np.float32), k_scale)
         vb, vf = stored(rng.standard_normal((t - 1, hkv, d)).astype(np.float32), v_scale)
         gpu.upload(i, kb, vb)
         k_bits.append(kb), v_bits.append(vb), k32.append(kf), v32.append(vf)
-    used = gpu_pool.extend_kv_cache_batch(None, None, list(range(b)), [row] * b, gpu.segs, [0] * b, row, True)
+    used = vmm.extend_kv_cache_batch(None, None, list(range(b)), [row] * b, gpu.segs, [0] * b, row, True)
     assert used == [(t - 1) * row for t in lens]
-    q16, q32 = to_model(rng.standard_normal((b, hq, d)).astype(np.float32), "f16")
-    nk16, nk32 = to_model(rng.standard_normal((b, hkv, d)).astype(np.float32), "f16")
-    nv16, nv32 = to_model(rng.standard_normal((b, hkv, d)).astype(np.float32), "f16")
-    slopes = (rng.standard_normal(hq) * 0.1).astype(np.float32)
+    q16, q32 = to_model(rng.standard_normal((b, hq, d)).astype(np.float32), dtype)
+    nk16, nk32 = to_model(rng.standard_normal((b, hkv, d)).astype(np.float32), dtype)
+    nv16, nv32 = to_model(rng.standard_normal((b, hkv, d)).astype(np.float32), dtype)
+    slopes = (rng.standard_normal(hq) * 0.1).astype(np.float32) if alibi else None
     kt, vt = gpu.table_tensors()
-    dev = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.float16).cuda()
+    dev = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(tdt).cuda()
     out = torch.empty(b, hq, d, dtype=torch.float32, device="cuda")
     lens_arg = list(lens) if lens_from == "host" else torch.tensor(lens, dtype=torch.int32, device="cuda")
     ops.decode_append_attention(out, dev(q16), dev(nk16).view(b, hkv * d), dev(nv16).view(b, hkv * d), kt, vt, hkv,
-                                d ** -0.5, lens_arg, max(lens), torch.from_numpy(slopes).cuda(),
-                                torch.arange(b, dtype=torch.int64, device="cuda"),
+                                d ** -0.5, lens_arg, max(lens), None if slopes is None else torch.from_numpy(slopes).cuda(),
+                                torch.arange(b, dtype=torch.int64, device="cuda"), partition_tokens=partition_tokens,
                                 kv_cache_dtype="fp8" if fp8 else "auto", kv_scale=k_scale, v_scale=v_scale)
     torch.cuda.synchronize()
     # the appended rows, bit for bit, and nothing before them disturbed
@@ -303,6 +299,45 @@ def test_fused_append_for_fp16_models(gpu_pool, fp8, lens_from):
     want = O.paged_attention_v1(q32, O.VTensorCache(k32, v32, np.arange(b), hkv, d), d ** -0.5, lens, slopes)
     err = np.abs(out.cpu().numpy() - want)
     assert bool(np.all(err <= 2e-3 + 2e-3 * np.abs(want))), f"max err {err.max():.3e}"
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("lens_from", ["host", "device"])
+def test_fused_append_for_fp16_models(gpu_pool, fp8, lens_from):
+    """fp16 queries and new rows at head size 128, 16-bit and fp8 caches; lengths around tile and chunk boundaries,
+    ALiBi, lengths from either side."""
+    per = (2 << 20) // (8 * 128 * (1 if fp8 else 2))
+    lens = [1, 2, 16, 17, 18, 33, 257, per - 1, per, per + 1, 2500]      # they count the new token
+    run_append_case(gpu_pool, 90 + fp8, lens, 32, 8, 128, "f16", fp8=fp8, lens_from=lens_from)
+
+
+@pytest.mark.parametrize("heads", [(32, 8), (40, 40), (15, 5), (64, 8)])
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("d", [64, 80, 96, 112, 256])
+def test_fused_append_on_other_head_sizes(gpu_pool, d, dtype, heads):
+    """The one-launch decode step for 16-bit caches of every other head size.  The head counts take each way the
+    rows are streamed: several kv heads per wave tile (64, 80, 96 with 32 over 8 and 40 over 40; 64 and 96 with 64
+    over 8), four kv heads per segment (112 with 32 over 8 and 40 over 40), one kv head per segment (256; 5 kv heads;
+    80 and 112 with 64 over 8)."""
+    hq, hkv = heads
+    per = (2 << 20) // (hkv * d * 2)
+    lens = [1, 2, 16, 17, 18, 33, 257, per, per + 1, 2 * per + 1, 1500]
+    run_append_case(gpu_pool, 500 + d, lens, hq, hkv, d, dtype, lens_from="host", alibi=(hkv != 5))
+    run_append_case(gpu_pool, 600 + d, [700, 65, 1, 1500, 2049, 17], hq, hkv, d, dtype, lens_from="device",
+                    alibi=False, partition_tokens=256)
+
+
+def test_fused_append_on_other_head_sizes_long_sequences(gpu_pool):
+    # sequences spread over many workgroups: the new row's tile is then a segment of its own for some
+    run_append_case(gpu_pool, 71, [30000, 1, 2, 5000], 32, 8, 80, "bf16", lens_from="device")
+    run_append_case(gpu_pool, 72, [30000, 3, 4097], 32, 8, 112, "f16", lens_from="host")
+    run_append_case(gpu_pool, 73, [20000, 1, 4097], 16, 4, 256, "bf16", lens_from="device")
+    run_append_case(gpu_pool, 74, [30000, 1, 2, 5000], 16, 8, 64, "f16", lens_from="host")
+
+
+def test_fused_append_refuses_fp8_rows_of_other_head_sizes(gpu_pool):
+    with pytest.raises(Exception, match="16-bit rows"):
+        run_append_case(gpu_pool, 75, [5, 40], 32, 8, 64, "bf16", fp8=True)
 
 
 def test_workspace_is_sized_for_the_padded_head_size(gpu_pool):
