@@ -147,6 +147,31 @@ def prompt_run(args, cfg) -> int:
                      "kernel": "prefill_attn_kernel", "avg_call_ms": round(attn_ms, 4),
                      "algorithmic_flops_per_call": flops},
     }
+    if args.workgroup_trace:
+        # the tracing build keeps {XCC id, start, first stage in LDS, end of the stages, end, stages} of every workgroup
+        # of the last launch (100 MHz clock)
+        from glake_amd import _C
+        fn = _C.lib().vtkv_debug_prefill_trace
+        fn.argtypes = [C.c_void_p, C.c_int]
+        per_unit = max(1, 128 // (Hq // Hkv))
+        n_wg = min(4096, sum((n + per_unit - 1) // per_unit for n in lens) * Hkv)
+        buf = (C.c_ulonglong * (4096 * 6))()
+        _C.check(fn(buf, 4096))
+        t = np.array(list(buf), dtype=np.int64).reshape(4096, 6)[:n_wg]
+        t0 = t[:, 1].min()
+        us = lambda a: (a - t0) / 100.0
+        life = (t[:, 4] - t[:, 1]) / 100.0
+        pro, loop, epi = (t[:, 2] - t[:, 1]) / 100.0, (t[:, 3] - t[:, 2]) / 100.0, (t[:, 4] - t[:, 3]) / 100.0
+        span = float(us(t[:, 4]).max())
+        q = lambda a: [round(float(np.percentile(a, x)), 2) for x in (10, 50, 90)]
+        result["workgroup_trace"] = {
+            "workgroups": int(n_wg), "kernel_span_us": round(span, 1),
+            "prologue_us_p10_p50_p90": q(pro), "epilogue_us_p10_p50_p90": q(epi),
+            "stage_ns_p10_p50_p90": q(loop * 1e3 / np.maximum(t[:, 5], 1)),
+            "sum_of_lifetimes_over_span_times_512": round(float(life.sum() / (span * 512)), 3),
+            "share_of_lifetime_in_prologue_and_epilogue": round(float((pro.sum() + epi.sum()) / life.sum()), 3),
+            "last_start_us": round(float(us(t[:, 1]).max()), 1),
+            "end_us_mean_by_xcc": [round(float(us(t[:, 4])[t[:, 0] == x].max()), 1) for x in range(8)]}
     print(json.dumps(result))
     engine.close()
     return 0

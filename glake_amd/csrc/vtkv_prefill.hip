@@ -34,6 +34,12 @@
 
 #include <type_traits>
 
+#ifdef VTKV_PREFILL_TRACE
+// Tuning builds only: per workgroup of the last launch {XCC id, start, first stage in LDS, end of the stages, end,
+// stages} on the 100 MHz wall clock.
+__device__ unsigned long long g_prefill_trace[4096][6];
+#endif
+
 namespace {
 
 using namespace vtkv_attn;
@@ -120,6 +126,10 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
   auto k_lds_offset = [](int row, int piece16) { return row * kRowBytes + ((piece16 ^ (row & 15)) << 4); };
   auto v_lds_offset = [](int row, int piece16) { return row * kRowBytes + ((piece16 ^ ((row & 7) << 1)) << 4); };
   __shared__ __attribute__((aligned(16))) char smem[2 * kStageBytes];
+#ifdef VTKV_PREFILL_TRACE
+  const unsigned long long trace_t0 = wall_clock64();
+  unsigned long long trace_t1 = 0;
+#endif
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int g = lane >> 4, n = lane & 15;
@@ -427,12 +437,18 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
     gload();
     lstore(std::integral_constant<int, 0>{}, widec);
     __syncthreads();
+#ifdef VTKV_PREFILL_TRACE
+    trace_t1 = wall_clock64();
+#endif
     for (int kb = 0; kb < nblocks; kb += 2) {
       stage(std::integral_constant<int, 0>{}, widec, kb);
       if (kb + 1 < nblocks) stage(std::integral_constant<int, 1>{}, widec, kb + 1);
     }
   };
   run(std::false_type{});
+#ifdef VTKV_PREFILL_TRACE
+  const unsigned long long trace_t2 = wall_clock64();
+#endif
   if constexpr (!FP8 && !F16) {
     // A V value beyond the fp16 range went into LDS as infinity and has made some accumulator of the workgroup
     // infinite or NaN (a weight of exactly zero gives NaN).  Then the whole unit is computed again with V in
@@ -479,6 +495,18 @@ __global__ void __launch_bounds__(kThreads) prefill_attn_kernel(PrefillParams p)
       }
     }
   }
+#ifdef VTKV_PREFILL_TRACE
+  if (threadIdx.x == 0 && blockIdx.x < 4096) {
+    unsigned xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    g_prefill_trace[blockIdx.x][0] = xcc & 0xf;
+    g_prefill_trace[blockIdx.x][1] = trace_t0;
+    g_prefill_trace[blockIdx.x][2] = trace_t1;
+    g_prefill_trace[blockIdx.x][3] = trace_t2;
+    g_prefill_trace[blockIdx.x][4] = wall_clock64();
+    g_prefill_trace[blockIdx.x][5] = (unsigned long long)nblocks;
+  }
+#endif
 }
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
@@ -578,5 +606,12 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
   VTKV_HIP(hipGetLastError());
   return VTKV_OK;
 }
+
+#ifdef VTKV_PREFILL_TRACE
+__attribute__((visibility("default"))) int vtkv_debug_prefill_trace(unsigned long long *out, int n) {
+  VTKV_HIP(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_prefill_trace), (size_t)n * 6 * sizeof(unsigned long long)));
+  return VTKV_OK;
+}
+#endif
 
 }  // extern "C"
