@@ -99,7 +99,8 @@ def test_random_sweep_fp8_decode(gpu_pool, seed):
 def test_random_sweep_over_head_sizes_and_types(gpu_pool, seed):
     """The same sweep over the other head sizes (64, 80, 96, 112, 256, and 128 in fp16), fp16 and bf16, plain and
     fp8 caches, the plain entry point with stream-K or fixed partitions and the split-K interface; for half of
-    the cases also a batch of prompts (some behind cached rows) through the prompt kernel of that shape."""
+    the cases also the fused append on the same shape (where it exists) and a batch of prompts (some behind cached
+    rows) through the prompt kernel of that shape."""
     sweep_head_sizes(gpu_pool, seed, HEADS, 40, always_f16_at_128=True)
 
 
@@ -119,6 +120,7 @@ def sweep_head_sizes(gpu_pool, seed, heads, cases, always_f16_at_128):
 
     lib = _C.lib()
     rng = np.random.default_rng(seed)
+    rng_append = np.random.default_rng(seed + 1)  # (its own stream: the cases above it stay what they were)
     try:
         for case in range(cases):
             hq, hkv = heads[rng.integers(len(heads))]
@@ -142,6 +144,13 @@ def sweep_head_sizes(gpu_pool, seed, heads, cases, always_f16_at_128):
             print(f"case {case}: seed {sub} heads {hq}/{hkv} d {d} {dtype} fp8 {fp8} lens {lens} {version} partition {pt} "
                   f"alibi {alibi} merge {merge}", flush=True)
             H.run_case(gpu_pool, sub, lens, hq, hkv, d, dtype, fp8=fp8, alibi=alibi, version=version, partition_tokens=pt)
+            # the one-launch decode step on the same shape, where it exists: any cache at head size 128, 16-bit caches
+            # of kv heads with at most 16 query heads elsewhere
+            if (d == 128 or (not fp8 and hq // hkv <= 16)) and rng_append.integers(2) == 0:
+                src = "host" if rng_append.integers(2) else "device"
+                print(f"append case {case}: lengths from the {src}", flush=True)
+                H.run_append_case(gpu_pool, sub, lens, hq, hkv, d, dtype, fp8=fp8, lens_from=src, alibi=alibi,
+                                  partition_tokens=pt)
             if rng.integers(2) == 0:
                 seq = [int(x) for x in rng.integers(1, 700, int(rng.integers(1, 6)))]
                 ql = [int(rng.integers(1, s + 1)) if rng.integers(2) else s for s in seq]
