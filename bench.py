@@ -66,6 +66,12 @@ CONFIGS = {
     # outside BASELINE.json: very many short sequences (every workgroup meets many segment starts and ends)
     "t1k": dict(name="many-short-bf16 B=1024 Hq=32 Hkv=8 D=128 ctx~U[64,512]", batch=1024, hq=32, hkv=8, d=128, lo=64,
                 hi=512, seed=1007, kv="bf16"),
+    # BASELINE.json configs[0] (the reference's CPU-runnable case) on the GPU, and configs[1]'s batch in float32:
+    # float32 queries over float32 rows through the float32 kernels
+    "c1": dict(name="fp32 B=8 Hq=32 Hkv=8 D=128 ctx~U[128,1024]", batch=8, hq=32, hkv=8, d=128, lo=128, hi=1024,
+               seed=1000, kv="f32", f32=True),
+    "c2f32": dict(name="llama3-8b-decode-fp32 B=64 Hq=32 Hkv=8 D=128 ctx~U[512,4096]", batch=64, hq=32, hkv=8, d=128,
+                  lo=512, hi=4096, seed=1001, kv="f32", f32=True),
     # outside BASELINE.json: a prompt run (cache write + causal attention over the ranges), 8 prompts of 2048
     "p2k": dict(name="llama3-8b-prompt-run-bf16 B=8 Hq=32 Hkv=8 D=128 prompt=2048", batch=8, hq=32, hkv=8, d=128,
                 lo=2048, hi=2048, seed=1006, kv="bf16", prefill=True),
@@ -177,6 +183,95 @@ def prompt_run(args, cfg) -> int:
     return 0
 
 
+def f32_run(args, cfg) -> int:
+    """A float32 model: one step = reshape_and_cache of one new float32 row per sequence + decode attention over
+    float32 rows (two launches, three where partitions are merged), through DecodeStepPlan.  Reported like the 16-bit
+    workloads: algorithmic bytes (rows + q + out, 4 bytes per element) per second of whole steps, and for the
+    attention call alone by HIP events on the stream it runs on."""
+    import torch
+
+    from glake_amd import _custom_ops as ops, vmm_allocator as vmm
+    from glake_amd.worker.cache_engine import CacheEngine
+    from glake_amd.worker.step import DecodeStepPlan
+
+    B, Hq, Hkv, D = cfg["batch"], cfg["hq"], cfg["hkv"], cfg["d"]
+    K, W = args.steps, args.warmup
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda", 0)
+    ctx0 = torch.randint(cfg["lo"], cfg["hi"] + 1, (B,), generator=torch.Generator().manual_seed(cfg["seed"])).tolist()
+    row = Hkv * D * 4
+    total_steps = 2 * (W + K) + 4
+    chunk = vmm.chunkBytes()
+    chunks_per_range = ((max(ctx0) + total_steps + 1) * row + args.value_skew + chunk - 1) // chunk
+    vmm.init_physical_handle(2 * B * chunks_per_range + 16, 0)
+    engine = CacheEngine(num_layers=1, num_kv_heads=Hkv, head_size=D, dtype=torch.float32, max_num_seqs=B,
+                         max_num_batched_tokens=max(ctx0) + total_steps + 1, swap_space_bytes=0,
+                         value_skew=args.value_skew)
+    segs = engine.vmm_kvcache_segment
+    ggen = torch.Generator(device=dev).manual_seed(cfg["seed"])
+    for b in range(B):
+        nbytes = ctx0[b] * row
+        segs[b].ensure_mapped(nbytes)
+        for base in (segs[b].getKeyDevicePtr(0), segs[b].getValueDevicePtr(0)):
+            t = torch.randn(ctx0[b], Hkv, D, generator=ggen, device=dev, dtype=torch.float32)
+            ops.swap_ranges([t.data_ptr()], [base], [nbytes], "d2d")
+            torch.cuda.synchronize()
+        segs[b].set_used_size(nbytes)
+    q = torch.randn(B, Hq, D, generator=ggen, device=dev, dtype=torch.float32)
+    new_k = torch.randn(B, Hkv * D, generator=ggen, device=dev, dtype=torch.float32)
+    new_v = torch.randn(B, Hkv * D, generator=ggen, device=dev, dtype=torch.float32)
+    out = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
+    plan = DecodeStepPlan(segs, list(range(B)), engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hq, Hkv, D, D ** -0.5,
+                          model_dtype=torch.float32, device=dev)
+    torch.cuda.set_stream(torch.cuda.Stream(device=dev))
+    step_bytes = lambda lens: sum(lens) * 2 * row + 2 * B * Hq * D * 4
+    lens = list(ctx0)
+    for _ in range(W):
+        plan.run(q, new_k, new_v, out)
+        lens = [n + 1 for n in lens]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    moved = 0
+    for _ in range(K):
+        plan.run(q, new_k, new_v, out)
+        lens = [n + 1 for n in lens]
+        moved += step_bytes(lens)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    # the attention call alone (the lengths stay what they are), with HIP events on its stream
+    lens_t = torch.tensor(lens, dtype=torch.int32, device=dev)
+    slot_t = torch.arange(B, dtype=torch.int64, device=dev)
+    attend = lambda: ops.paged_attention_v1(out, q, engine.k_cache_ptr[0], engine.v_cache_ptr[0], Hkv, D ** -0.5, lens_t, 1,
+                                            max(lens), None, "auto", 1.0, slot_t)
+    for _ in range(W):
+        attend()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev[0].record()
+    for _ in range(K):
+        attend()
+    ev[1].record()
+    torch.cuda.synchronize()
+    attn_ms = ev[0].elapsed_time(ev[1]) / K
+    achieved = step_bytes(lens) / (attn_ms * 1e-3) / 1e9
+    value = moved / dt / 1e9
+    result = {
+        "metric": "decode-attn HBM GB/s (% peak) + tokens/s, float32 model", "value": round(value, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(dt / K * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": cfg["name"], "layers": 1, "new_tokens_per_step": B, "kv_chunk": "2MiB VMM",
+                   "mean_ctx": round(sum(ctx0) / B, 1)},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2), "tokens_per_s": round(B * K / dt, 1),
+        "algorithmic_bytes_per_step": step_bytes(lens),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "decode_attn_f32_kernel (+ merge_attn_f32_kernel)", "avg_call_us": round(attn_ms * 1e3, 2),
+                     "algorithmic_bytes_per_launch": step_bytes(lens)},
+    }
+    print(json.dumps(result))
+    engine.close()
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -227,6 +322,10 @@ def main() -> int:
         if args.steps == 200 and args.warmup == 20:
             args.steps, args.warmup = 20, 3
         return prompt_run(args, cfg)
+    if cfg.get("f32"):
+        if args.steps == 200 and args.warmup == 20:
+            args.steps, args.warmup = 50, 5
+        return f32_run(args, cfg)
     from glake_amd import _C
 
     if args.chunk_mib != 2:

@@ -160,10 +160,10 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
         ``slot_m``, ``seq_lens_tensor``) is ordered the same way."""
         from ... import _custom_ops as ops
 
-        if query.dtype not in (torch.bfloat16, torch.float16):
-            # the attention kernels take 16-bit queries; on the reference's vTensor path both decode branches run
-            # an external kernel that exists for fp16 and bf16 only (xformers.py:362-385,407-430)
-            raise ValueError(f"the vtensor backend runs bfloat16 and float16 models, not {query.dtype}")
+        if query.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise ValueError(f"the vtensor backend runs bfloat16, float16 and float32 models, not {query.dtype}")
+        # (float32 models run the separate calls over a float32 cache: the one-launch step is built for 16-bit models)
+        fuse = self.fuse_decode_append and query.dtype != torch.float32
         query = query.view(-1, self.num_heads, self.head_size)
         key = key.view(-1, self.num_kv_heads, self.head_size)
         value = value.view(-1, self.num_kv_heads, self.head_size)
@@ -219,7 +219,7 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
                 d_lens = meta.seq_lens_tensor[n_pre:]
                 d_out = output[num_prefill_tokens:]
             max_len = meta.max_decode_seq_len if n_pre > 0 and meta.max_decode_seq_len else meta.max_seq_len
-            if self.fuse_decode_append and (self.head_size == 128 or (
+            if fuse and (self.head_size == 128 or (
                     self.kv_cache_dtype == "auto" and self.num_queries_per_kv <= 16)):
                 # the cache write (xformers.py:310-312) and the decode attention (:357-371) in one launch.
                 # The row goes to position seq_len - 1 of each range, which is where slot_m points in the

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libvtkv.so")
-SOURCES = ["vtkv_vmm.cpp", "vtkv_cache.hip", "vtkv_attention.hip", "vtkv_prefill.hip"]
+SOURCES = ["vtkv_vmm.cpp", "vtkv_cache.hip", "vtkv_attention.hip", "vtkv_attention_f32.hip", "vtkv_prefill.hip"]
 
 # Packed-FP32 instruction selection is switched off for all device code of this library.
 HIP_FLAGS = [

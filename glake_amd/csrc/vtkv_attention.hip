@@ -1533,6 +1533,22 @@ int attention_impl(void *out, const void *q, const int64_t *k_ptrs, const int64_
                    void *workspace, int64_t workspace_bytes, int partition_tokens, void *stream, const void *new_key,
                    const void *new_value, int64_t key_stride, int64_t value_stride, const V2Side *v2 = nullptr,
                    bool static_scratch = false) {
+  if (q_dtype == VTKV_F32) {
+    // float32 models: a kernel of their own over float32 rows (csrc/vtkv_attention_f32.hip)
+    VTKV_REQUIRE(kv_dtype == VTKV_F32 && out_dtype == VTKV_F32, "float32 queries take a float32 cache and a float32 result");
+    VTKV_REQUIRE(!new_key && !host_seq_lens, "the fused append is built for 16-bit models");
+    VTKV_REQUIRE(seq_lens, "null argument");
+    if (v2) VTKV_REQUIRE(v2->exp_sums && v2->max_logits && v2->tmp_out, "null argument");
+    // (the start of a workspace holds the arrival counters of the 16-bit kernels, which they expect to find at
+    // zero: the partial results of this path go behind them)
+    const int64_t skip = counter_bytes(0, 0);
+    const bool usable = workspace && workspace_bytes > skip;
+    return vtkv::attention_f32((float *)out, (const float *)q, k_ptrs, v_ptrs, slot_ids, seq_lens, nullptr, 0, num_seqs,
+                               num_heads, num_kv_heads, head_size, q_stride, scale, max_seq_len, alibi_slopes,
+                               v2 ? v2->exp_sums : nullptr, v2 ? v2->max_logits : nullptr,
+                               v2 ? (float *)v2->tmp_out : nullptr, v2 ? v2->max_parts : 0,
+                               usable ? (char *)workspace + skip : nullptr, usable ? workspace_bytes - skip : 0, stream);
+  }
   const int per_call = host_seq_lens ? kInlineLens : kMaxSeqs;
   if (num_seqs <= per_call || !out || !q || !slot_ids || num_heads <= 0 || head_size <= 0)
     return attention_batch(out, q, k_ptrs, v_ptrs, slot_ids, seq_lens, host_seq_lens, num_seqs, num_heads, num_kv_heads,

@@ -23,6 +23,14 @@ inline int elem_bytes(int dtype) {
   }
 }
 
+// Float32 attention (csrc/vtkv_attention_f32.hip): decode rows (seq_lens) or prompt tokens (units of up to
+// unit_tokens tokens); the split-K interface's buffers, a workspace for partial results, or neither.
+int attention_f32(float *out, const float *q, const int64_t *k_ptrs, const int64_t *v_ptrs, const int64_t *slot_ids,
+                  const int32_t *seq_lens, const int32_t *units, int unit_tokens, int num_rows, int num_heads,
+                  int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
+                  const float *alibi_slopes, float *exp_sums, float *max_logits, float *tmp_out, int max_parts,
+                  void *workspace, int64_t workspace_bytes, void *stream);
+
 }  // namespace vtkv
 
 #define VTKV_HIP(call)                                                                              \

@@ -548,7 +548,17 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
                "num_heads %d must be a positive multiple of num_kv_heads %d", num_heads, num_kv_heads);
   const int d_index = size_index(head_size);
   VTKV_REQUIRE(d_index >= 0, "head_size %d is not supported (64, 80, 96, 112, 128, 256)", head_size);
-  VTKV_REQUIRE(q_dtype == VTKV_BF16 || q_dtype == VTKV_F16, "q_dtype must be BF16 or F16");
+  if (q_dtype == VTKV_F32) {
+    // float32 models: every prompt token streams its own rows through the float32 decode kernel
+    VTKV_REQUIRE(kv_dtype == VTKV_F32 && out_dtype == VTKV_F32, "float32 queries take a float32 cache and a float32 result");
+    VTKV_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
+    const int per_unit = vtkv_prefill_unit_tokens_for(num_heads, num_kv_heads, head_size, kv_dtype);
+    VTKV_REQUIRE(per_unit > 0, "unsupported head counts");
+    return vtkv::attention_f32((float *)out, (const float *)q, k_ptrs, v_ptrs, slot_ids, nullptr, units, per_unit,
+                               num_units * per_unit, num_heads, num_kv_heads, head_size, q_stride, scale, max_seq_len,
+                               alibi_slopes, nullptr, nullptr, nullptr, 0, nullptr, 0, stream);
+  }
+  VTKV_REQUIRE(q_dtype == VTKV_BF16 || q_dtype == VTKV_F16, "q_dtype must be BF16, F16 or F32");
   VTKV_REQUIRE(out_dtype == q_dtype || out_dtype == VTKV_F32, "out_dtype must be q_dtype or F32");
   VTKV_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
   VTKV_REQUIRE(kv_dtype == q_dtype || kv_dtype == VTKV_FP8_E4M3, "kv_dtype must be q_dtype or FP8_E4M3");

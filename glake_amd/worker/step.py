@@ -129,9 +129,9 @@ class DecodeStepPlan:
             raise _C.VtkvError(_C.EINVAL, "DecodeStepPlan: one slot id per segment, at least one sequence")
         if ring < 2 or ring % 2:
             raise _C.VtkvError(_C.EINVAL, "DecodeStepPlan: ring must be even and at least 2")
-        if model_dtype not in (torch.bfloat16, torch.float16):
-            raise _C.VtkvError(_C.EINVAL, f"DecodeStepPlan: the attention kernels take bfloat16 and float16 queries, "
-                                          f"not {model_dtype}")
+        if model_dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise _C.VtkvError(_C.EINVAL, f"DecodeStepPlan: the attention kernels take bfloat16, float16 and float32 "
+                                          f"queries, not {model_dtype}")
         self._C, self._lib, self._np = _C, _C.lib(), np
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         n = self.n = len(segments)
@@ -140,7 +140,7 @@ class DecodeStepPlan:
         self._src_dt = ops._DTYPES[model_dtype]
         self._kv_dt = ops._kv_dtype(kv_cache_dtype, self._src_dt)
         self.k_scale, self.v_scale = float(k_scale), float(v_scale)
-        self.kv_size = self.num_kv_heads * self.head_size * (1 if self._kv_dt == _C.FP8_E4M3 else 2)  # bytes per row
+        self.kv_size = self.num_kv_heads * self.head_size * {_C.FP8_E4M3: 1, _C.F32: 4}.get(self._kv_dt, 2)  # bytes per row
         self._segments = list(segments)  # keeps the handles alive
         self._segs = (C.c_void_p * n)(*[s._h for s in segments])
         self._tok = (C.c_int64 * n)(*([self.kv_size] * n))
@@ -176,7 +176,7 @@ class DecodeStepPlan:
         self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
         # one launch per step: any cache type at head size 128; 16-bit caches at the other head sizes when a kv head
         # has at most 16 query heads
-        self.fused = bool(fused) and (self.head_size == 128 or (
+        self.fused = bool(fused) and self._src_dt != _C.F32 and (self.head_size == 128 or (
             self._kv_dt == self._src_dt and self.num_heads // self.num_kv_heads <= 16))
         self._inline = self.fused and n <= 512
         self._host_lens_p = [C.c_void_p(self._stage[i].data_ptr() + 8 * n) for i in range(ring)]

@@ -300,13 +300,17 @@ int64_t vtkv_decode_attention_workspace_bytes(int num_seqs, int num_heads, int h
  *                The result does not depend on the choice beyond fp32 summation order.
  * A launch takes up to 1024 sequences; a larger batch runs as consecutive launches of 1024 on `stream` within
  * the one call.
- * Supported: q_dtype VTKV_BF16 or VTKV_F16 (VTKV_F32 queries are refused with VTKV_EINVAL: the reference's kernel
- * tests also run float, tests/kernels/test_attention.py:23, but its vTensor path serves 16-bit models only, see
- * xformers.py:362-385), kv_dtype = q_dtype or VTKV_FP8_E4M3, head_size 64, 80, 96, 112, 128 or
- * 256 (the reference's list, vllm/attention/ops/paged_attn.py:33-34), any whole num_heads/num_kv_heads.  The kernel
+ * Supported: q_dtype VTKV_BF16 or VTKV_F16 with kv_dtype = q_dtype or VTKV_FP8_E4M3, head_size 64, 80, 96, 112, 128
+ * or 256 (the reference's list, vllm/attention/ops/paged_attn.py:33-34), any whole num_heads/num_kv_heads.  The kernel
  * is tuned for bf16 and head size 128; the other shapes run the same code with their own tile constants.  A kv head
  * with more than 16 query heads (multi-query models) is served in ceil(n/16) parts of equal size (the last may be
- * smaller) that each read the kv head's rows: the parts count as kv heads towards the limit of 64 per call. */
+ * smaller) that each read the kv head's rows: the parts count as kv heads towards the limit of 64 per call.
+ * q_dtype VTKV_F32 (the reference's kernel tests also run float, tests/kernels/test_attention.py:23): float32 rows
+ * and a float32 result (kv_dtype = out_dtype = VTKV_F32), every head size and head count, through a simpler kernel
+ * of its own that computes in fp32 on the vector unit; partition_tokens is ignored (partitions of 512 rows, fewer
+ * rows for small batches, more where the workspace does not hold the partial results); also through
+ * vtkv_decode_attention_v2, vtkv_decode_attention_noalloc and vtkv_prefill_attention (where every prompt token
+ * streams its own rows: right, and quadratic in HBM traffic), not through vtkv_decode_append_attention. */
 int vtkv_decode_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                           const int64_t *slot_ids, const int32_t *seq_lens, int num_seqs, int num_heads,
                           int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
