@@ -219,8 +219,7 @@ class VTensorImpl(AttentionImpl[VTensorMetadata]):
                 d_lens = meta.seq_lens_tensor[n_pre:]
                 d_out = output[num_prefill_tokens:]
             max_len = meta.max_decode_seq_len if n_pre > 0 and meta.max_decode_seq_len else meta.max_seq_len
-            if fuse and (self.head_size == 128 or (
-                    self.kv_cache_dtype == "auto" and self.num_queries_per_kv <= 16)):
+            if fuse and (self.head_size == 128 or self.kv_cache_dtype == "auto"):
                 # the cache write (xformers.py:310-312) and the decode attention (:357-371) in one launch.
                 # The row goes to position seq_len - 1 of each range, which is where slot_m points in the
                 # reference's flow (llama.py:340: the bytes used before this step).  Where the metadata also

@@ -1123,12 +1123,13 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16 + 24 + 2 + 18 + 28 + 6 + 18;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
+constexpr int kVariants = 16 + 24 + 2 + 18 + 28 + 6 + 18 + 10;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
                                                        // others, the fused append for fp16 at head size 128 (fp16 rows,
                                                        // fp8 rows), 18 that stream several kv heads per segment at other
                                                        // shapes, 28 for kv heads of more than 16 query heads (SPLIT), 6
                                                        // whose wave tiles hold several kv heads (GW), 18 with the fused
-                                                       // append for 16-bit rows of the other head sizes
+                                                       // append for 16-bit rows of the other head sizes, 10 more of
+                                                       // those for kv heads of more than 16 query heads
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
 int head_size_index(int head_size) {
@@ -1246,8 +1247,7 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
                "partition_tokens must be 0 or a multiple of %d that is at least %d", kTile, kWaves * kTile);
   if (append) {
     VTKV_REQUIRE(new_value != nullptr, "null argument");
-    VTKV_REQUIRE(head_size == 128 || (kv_dtype == q_dtype && kv_split == 1),
-                 "the fused append at head sizes other than 128 needs 16-bit rows and at most 16 query heads per kv head");
+    VTKV_REQUIRE(head_size == 128 || kv_dtype == q_dtype, "the fused append at head sizes other than 128 needs 16-bit rows");
     const int64_t row = (int64_t)kv_heads_real * head_size;
     VTKV_REQUIRE(key_stride >= row && value_stride >= row && key_stride % 8 == 0 && value_stride % 8 == 0 &&
                      (uintptr_t)new_key % 16 == 0 && (uintptr_t)new_value % 16 == 0,
@@ -1309,7 +1309,9 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   }
   // kv heads of more than 16 query heads: one variant per (head size, type, cache type), the fused append at 128
   if (kv_split > 1)
-    variant = append ? 84 + (f16 ? 2 : 0) + (fp8 ? 1 : 0) : 60 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
+    variant = append_other ? 112 + (d_index < 4 ? d_index : 4) * 2 + (f16 ? 1 : 0)
+              : append     ? 84 + (f16 ? 2 : 0) + (fp8 ? 1 : 0)
+                           : 60 + (d_index * 2 + (f16 ? 1 : 0)) * 2 + (fp8 ? 1 : 0);
 #define VTKV_ROW(F8, H)                                                                                      \
   decode_attn_stream_kernel<false, F8, false, H>, decode_attn_stream_kernel<true, F8, false, H>,             \
       decode_attn_stream_kernel<false, F8, true, H>, decode_attn_stream_kernel<true, F8, true, H>
@@ -1341,6 +1343,11 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
       VTKV_APPEND16(64, 1, 1), VTKV_APPEND16(80, 1, 1), VTKV_APPEND16(96, 1, 1), VTKV_APPEND16(112, 1, 1), VTKV_APPEND16(256, 1, 1),
       VTKV_APPEND16(64, 1, 2), VTKV_APPEND16(80, 1, 4), VTKV_APPEND16(96, 1, 2), VTKV_APPEND16(112, 4, 1),
 #undef VTKV_APPEND16
+#define VTKV_SPLIT_APPEND16(DD)                                                                                 \
+  decode_attn_stream_kernel<true, false, true, 1, DD, false, true>, decode_attn_stream_kernel<true, false, true, 1, DD, true, true>
+      VTKV_SPLIT_APPEND16(64), VTKV_SPLIT_APPEND16(80), VTKV_SPLIT_APPEND16(96), VTKV_SPLIT_APPEND16(112),
+      VTKV_SPLIT_APPEND16(256),
+#undef VTKV_SPLIT_APPEND16
   };
 #undef VTKV_ROW
 #undef VTKV_SIZE

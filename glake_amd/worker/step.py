@@ -174,10 +174,8 @@ class DecodeStepPlan:
         self._ws = torch.zeros(max(int(need), 1 << 20), dtype=torch.uint8, device=self.device)
         self._ws_p, self._ws_n = C.c_void_p(self._ws.data_ptr()), self._ws.numel()
         self.seq_lens = None  # numpy view of the last step's lengths (valid until the ring wraps)
-        # one launch per step: any cache type at head size 128; 16-bit caches at the other head sizes when a kv head
-        # has at most 16 query heads
-        self.fused = bool(fused) and self._src_dt != _C.F32 and (self.head_size == 128 or (
-            self._kv_dt == self._src_dt and self.num_heads // self.num_kv_heads <= 16))
+        # one launch per step: any cache type at head size 128; 16-bit caches at the other head sizes
+        self.fused = bool(fused) and self._src_dt != _C.F32 and (self.head_size == 128 or self._kv_dt == self._src_dt)
         self._inline = self.fused and n <= 512
         self._host_lens_p = [C.c_void_p(self._stage[i].data_ptr() + 8 * n) for i in range(ring)]
 

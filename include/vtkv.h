@@ -402,9 +402,8 @@ int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, cons
  * pass NULL for the other.  q_dtype VTKV_BF16 or VTKV_F16 (the paired-head variants for very many short
  * sequences exist for bf16 at head size 128 only).  kv_dtype is q_dtype, or at head size 128 VTKV_FP8_E4M3 with
  * k_scale / v_scale: the new rows are then stored as e4m3fn(x / scale), bit for bit as vtkv_reshape_and_cache
- * stores them, and attended to in that form.  Head sizes 64, 80, 96, 112 and 256 take 16-bit caches and at most
- * 16 query heads per kv head (VTKV_EINVAL otherwise: make the two calls).  Other arguments as for
- * vtkv_decode_attention. */
+ * stores them, and attended to in that form.  Head sizes 64, 80, 96, 112 and 256 take 16-bit caches
+ * (VTKV_EINVAL for an fp8 cache: make the two calls).  Other arguments as for vtkv_decode_attention. */
 int vtkv_decode_append_attention(void *out, const void *q, const void *key, const void *value, int64_t key_stride,
                                  int64_t value_stride, const int64_t *k_ptrs, const int64_t *v_ptrs,
                                  const int64_t *slot_ids, const int32_t *seq_lens, const int32_t *host_seq_lens,

@@ -311,14 +311,15 @@ def test_fused_append_for_fp16_models(gpu_pool, fp8, lens_from):
     run_append_case(gpu_pool, 90 + fp8, lens, 32, 8, 128, "f16", fp8=fp8, lens_from=lens_from)
 
 
-@pytest.mark.parametrize("heads", [(32, 8), (40, 40), (15, 5), (64, 8)])
+@pytest.mark.parametrize("heads", [(32, 8), (40, 40), (15, 5), (64, 8), (71, 1), (40, 2)])
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 @pytest.mark.parametrize("d", [64, 80, 96, 112, 256])
 def test_fused_append_on_other_head_sizes(gpu_pool, d, dtype, heads):
     """The one-launch decode step for 16-bit caches of every other head size.  The head counts take each way the
     rows are streamed: several kv heads per wave tile (64, 80, 96 with 32 over 8 and 40 over 40; 64 and 96 with 64
     over 8), four kv heads per segment (112 with 32 over 8 and 40 over 40), one kv head per segment (256; 5 kv heads;
-    80 and 112 with 64 over 8)."""
+    80 and 112 with 64 over 8), kv heads of more than 16 query heads served in parts (71 over 1: parts of 15 heads,
+    the shape of a multi-query model with head size 64; 40 over 2: parts of 10)."""
     hq, hkv = heads
     per = (2 << 20) // (hkv * d * 2)
     lens = [1, 2, 16, 17, 18, 33, 257, per, per + 1, 2 * per + 1, 1500]

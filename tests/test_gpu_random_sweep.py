@@ -145,8 +145,8 @@ def sweep_head_sizes(gpu_pool, seed, heads, cases, always_f16_at_128):
                   f"alibi {alibi} merge {merge}", flush=True)
             H.run_case(gpu_pool, sub, lens, hq, hkv, d, dtype, fp8=fp8, alibi=alibi, version=version, partition_tokens=pt)
             # the one-launch decode step on the same shape, where it exists: any cache at head size 128, 16-bit caches
-            # of kv heads with at most 16 query heads elsewhere
-            if (d == 128 or (not fp8 and hq // hkv <= 16)) and rng_append.integers(2) == 0:
+            # elsewhere
+            if (d == 128 or not fp8) and rng_append.integers(2) == 0:
                 src = "host" if rng_append.integers(2) else "device"
                 print(f"append case {case}: lengths from the {src}", flush=True)
                 H.run_append_case(gpu_pool, sub, lens, hq, hkv, d, dtype, fp8=fp8, lens_from=src, alibi=alibi,
