@@ -37,3 +37,14 @@ def test_bench_line_carries_every_configuration():
                for e in c5["swap_events"])
     assert c5["bit_exact"] is True and c5["swapped_bytes_checked"] > 1e9 and c5["appended_rows_checked"] == 256 * 64 * 2
     assert c5["chunks_mapped_while_growing"] > 0
+
+
+def test_bench_line_of_the_float32_configuration():
+    # BASELINE.json configs[0] (fp32, 8 sequences of 128..1024 rows) through the float32 kernels
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "1", "--config", "c1", "--steps", "3",
+                        "--warmup", "1"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    assert line["dtype"] == "f32" and line["unit"] == "GB/s" and line["n_gpus"] == 1 and line["value"] > 10
+    assert line["config"]["workload"].startswith("fp32 B=8") and line["roofline"]["bound"] == "hbm"
+    assert 2e7 < line["algorithmic_bytes_per_step"] < 5e7
