@@ -297,8 +297,8 @@ def main() -> int:
                     help="tile order of the decode kernel: (kv head, sequence, rows) or (sequence, kv head, rows)")
     ap.add_argument("--head-size", type=int, default=0,
                     help="run the chosen decode workload with another head size of the reference's list (64, 80, 96, 112, "
-                         "256): the step then is reshape_and_cache + attention as two launches (the fused append is "
-                         "built for 128)")
+                         "256); an fp8 cache then takes reshape_and_cache + attention as two launches (its fused append "
+                         "exists at 128)")
     ap.add_argument("--heads", default="", metavar="HQ,HKV", help="likewise with other head counts")
     ap.add_argument("--chunk-mib", type=int, default=2,
                     help="size of a physical chunk (the reference's granularity is 2 MiB; vtkv_pool_set_chunk_bytes)")
