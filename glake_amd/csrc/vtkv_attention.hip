@@ -202,6 +202,7 @@ __device__ __forceinline__ int span_of(const AttnParams &p, int total_tiles) {
 template <bool ALIBI, bool FP8, bool APPEND, int HPS, int D = 128, bool F16 = false, bool SPLIT = false, int GW = 1>
 __global__ void __launch_bounds__(kThreads)
     __attribute__((amdgpu_waves_per_eu(D > 128   ? 1
+                                       : GW > 1 && D == 112 ? 1  // (four head rows of 224 bytes: 28 registers of 16 bytes per tile)
                                        : GW > 1  ? (FP8 && D <= 64 ? 3 : 2)  // (a tile of several kv heads is held in registers)
                                        : D < 128 ? (FP8 ? VTKV_ATTN_SMALL_FP8_WAVES : VTKV_ATTN_SMALL_WAVES)
                                                  : (FP8 ? VTKV_ATTN_FP8_WAVES : VTKV_ATTN_BF16_WAVES))))
@@ -1123,13 +1124,14 @@ struct KernelTimer {
 KernelTimer g_timer;
 
 // Workgroups of the streaming kernel that the current device holds at once (per kernel variant).
-constexpr int kVariants = 16 + 24 + 2 + 18 + 28 + 6 + 18 + 10;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
+constexpr int kVariants = 16 + 24 + 2 + 18 + 28 + 6 + 18 + 10 + 4;  // instantiations of the streaming kernel: 16 of the tuned shape, 24
                                                        // others, the fused append for fp16 at head size 128 (fp16 rows,
                                                        // fp8 rows), 18 that stream several kv heads per segment at other
                                                        // shapes, 28 for kv heads of more than 16 query heads (SPLIT), 6
                                                        // whose wave tiles hold several kv heads (GW), 18 with the fused
                                                        // append for 16-bit rows of the other head sizes, 10 more of
-                                                       // those for kv heads of more than 16 query heads
+                                                       // those for kv heads of more than 16 query heads, 4 for wave
+                                                       // tiles of four kv heads at head size 112
 
 // 64, 80, 96, 112, 128, 256 (vllm/attention/ops/paged_attn.py:33-34) -> 0..5, anything else -> -1
 int head_size_index(int head_size) {
@@ -1294,15 +1296,16 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
   // token), 80 (4: 640 bytes) and 96 (2: 384 bytes), where the heads that make whole lines have room in the 16
   // columns together.  To everything below, the GW heads are one kv head of group * GW query heads.  64 sequences
   // of 512..4096 rows, 8 kv heads of 4 query heads, stream kernel, share of the HBM peak, against one wave per head
-  // with plain loads: 80: 0.675 against 0.62, 96: 0.766 against 0.67, 64: 0.73 either way.  Measured and left out:
-  // 112 with 4 heads per tile (28 registers of 16 bytes to hold a tile: spills, 0.57 against 0.66), fp8 rows of 64
+  // with plain loads: 80: 0.675 against 0.62, 96: 0.766 against 0.67, 64: 0.73 either way; 112 (4 heads: 896 bytes
+  // per token, 28 registers of 16 bytes to hold a K or V tile) spills at two waves per SIMD (0.57 against 0.66) and
+  // runs one wave per SIMD instead, like head size 256: 0.715 against 0.675.  Measured and left out: fp8 rows of 64
   // and 96 with 4 (0.48 and 0.49 against 0.56 and 0.61).
-  if (!tuned && !fp8 && kv_split == 1 && d_index < 3) {
-    static const int kGw16[3] = {2, 4, 2};
+  if (!tuned && !fp8 && kv_split == 1 && d_index < 4) {
+    static const int kGw16[4] = {2, 4, 2, 4};
     const int gw = kGw16[d_index];
     if (num_kv_heads % gw == 0 && group * gw <= 16) {
       seg_heads = 1;
-      variant = (append ? 104 : 88) + d_index * 2 + (f16 ? 1 : 0);
+      variant = d_index < 3 ? (append ? 104 : 88) + d_index * 2 + (f16 ? 1 : 0) : (append ? 124 : 122) + (f16 ? 1 : 0);
       num_kv_heads /= gw;
       group *= gw;
     }
@@ -1348,6 +1351,8 @@ int attention_batch(void *out, const void *q, const int64_t *k_ptrs, const int64
       VTKV_SPLIT_APPEND16(64), VTKV_SPLIT_APPEND16(80), VTKV_SPLIT_APPEND16(96), VTKV_SPLIT_APPEND16(112),
       VTKV_SPLIT_APPEND16(256),
 #undef VTKV_SPLIT_APPEND16
+      decode_attn_stream_kernel<true, false, false, 1, 112, false, false, 4>, decode_attn_stream_kernel<true, false, false, 1, 112, true, false, 4>,
+      decode_attn_stream_kernel<true, false, true, 1, 112, false, false, 4>, decode_attn_stream_kernel<true, false, true, 1, 112, true, false, 4>,
   };
 #undef VTKV_ROW
 #undef VTKV_SIZE
