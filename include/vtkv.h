@@ -383,7 +383,8 @@ int vtkv_prefill_unit_tokens(int num_heads, int num_kv_heads, int kv_dtype);
  * or 256 (the kernel is tuned for 128; units hold vtkv_prefill_unit_tokens_for(...) tokens), q_dtype
  * VTKV_BF16 or VTKV_F16, kv_dtype = q_dtype or VTKV_FP8_E4M3 with k_scale / v_scale, out_dtype = q_dtype or
  * VTKV_F32; the longest-units-first order inside each sequence, sequence by sequence, lets every row be fetched
- * from HBM once. */
+ * from HBM once.  q_dtype VTKV_F32 with kv_dtype = out_dtype = VTKV_F32 (float32 models): every token attends
+ * through the float32 decode kernel by itself, without reuse of rows between tokens. */
 int vtkv_prefill_attention(void *out, const void *q, const int64_t *k_ptrs, const int64_t *v_ptrs,
                            const int64_t *slot_ids, const int32_t *units, int num_units, int num_heads,
                            int num_kv_heads, int head_size, int64_t q_stride, float scale, int max_seq_len,
